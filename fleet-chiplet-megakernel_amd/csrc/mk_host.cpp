@@ -1,0 +1,1078 @@
+// Host side of the persistent decode megakernel: records the PersistentKernel task
+// list, lowers it to the stage program the kernel walks, owns intermediate tensors
+// and runtime state, and launches the kernel cooperatively.
+//
+// Replaces, for the decode path: src/kernel/graph.cc (register_task, attach_*,
+// shuffle_tensors), src/kernel/task_register.cc (per-task validation),
+// src/kernel/runtime.cc (register_mugraph / print_task_graph) and the host half of
+// include/mirage/persistent_kernel/persistent_kernel.cuh:1960-2429.
+#include <hip/hip_runtime.h>
+#include <math.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <array>
+#include <map>
+#include <numeric>
+#include <string>
+#include <vector>
+
+#include "../../include/fleet_mk.h"
+#include "mk_types.h"
+
+
+namespace {
+
+thread_local std::string g_err;
+
+int fail(int code, const char *fmt, ...) {
+  char buf[1024];
+  va_list ap;
+  va_start(ap, fmt);
+  vsnprintf(buf, sizeof(buf), fmt, ap);
+  va_end(ap);
+  g_err = buf;
+  return code;
+}
+
+#define HIP_TRY(expr)                                                                         \
+  do {                                                                                        \
+    hipError_t e_ = (expr);                                                                   \
+    if (e_ != hipSuccess) return fail(MK_EHIP, "%s failed: %s", #expr, hipGetErrorString(e_)); \
+  } while (0)
+
+enum TensorKind { T_ATTACHED, T_OWNED, T_SHUFFLED };
+
+struct Tensor {
+  std::string name;
+  int ndims = 0;
+  int64_t dims[4] = {1, 1, 1, 1};
+  int64_t strides[4] = {1, 1, 1, 1};
+  int dtype = MK_DT_BF16;
+  TensorKind kind = T_ATTACHED;
+  void *ptr = nullptr;
+  std::vector<int> sources;  // T_SHUFFLED
+  int num_groups = 1;
+  bool interleave = true;
+  int io_category = 0;
+  size_t elems() const {
+    size_t n = 1;
+    for (int i = 0; i < ndims; i++) n *= (size_t)dims[i];
+    return n;
+  }
+};
+
+struct Task {
+  std::string name;
+  int grid[3], block[3];
+  std::vector<int> ops;
+  std::vector<std::array<int, 3>> maps;
+  std::vector<int> forloop;
+  std::vector<int> params;
+};
+
+size_t dtype_size(int dt) {
+  switch (dt) {
+    case MK_DT_BF16:
+    case MK_DT_F16: return 2;
+    case MK_DT_F32:
+    case MK_DT_I32: return 4;
+    case MK_DT_I64:
+    case MK_DT_U64: return 8;
+    default: return 0;
+  }
+}
+
+}  // namespace
+
+struct mk_graph {
+  mk_config cfg;
+  int num_cus = 0;
+  int G = 0;
+  std::vector<Tensor> tensors;
+  std::vector<Task> tasks;
+  bool compiled = false;
+  std::vector<void *> allocs;
+  std::vector<MkStage> stages;
+  std::vector<std::string> stage_desc;
+  MkRuntime h_rt;
+  MkRuntime *d_rt = nullptr;
+  MkStage *d_stages = nullptr;
+  MkSync *d_sync = nullptr;
+  MkSched *d_sched = nullptr;
+  long long *d_timing = nullptr;
+  int timing_cap = 0;
+  std::string json, program_text;
+  hipEvent_t ev0 = nullptr, ev1 = nullptr;
+  bool launch_pending = false;
+  double last_ms = 0.0;
+  int last_nxcd = 0, last_aborted = 0;
+  int64_t weight_bytes = 0;
+  size_t attn_cnt_n = 0;
+  int num_ref_tasks = 0, num_ref_events = 0;
+};
+
+namespace {
+
+int dev_alloc(mk_graph *g, void **out, size_t bytes, bool zero = true) {
+  if (bytes == 0) bytes = 16;
+  HIP_TRY(hipMalloc(out, bytes));
+  g->allocs.push_back(*out);
+  if (zero) HIP_TRY(hipMemset(*out, 0, bytes));
+  return MK_OK;
+}
+
+bool is_norm(const std::string &n) { return n == "rmsnorm" || n == "gang_rmsnorm_mi300"; }
+
+// Classify linear-type task names: returns false if `n` is not a linear.
+bool linear_kind(const std::string &n, bool *res, bool *silu, int *n_extra_inputs) {
+  *res = false;
+  *silu = false;
+  *n_extra_inputs = 0;
+  static const char *plain[] = {"linear", "gang_linear_mi300", "gang_linear_n_tiling_mi300", "gang_linear_msplit_mi300",
+                                "splitk_linear_mi300"};
+  static const char *with_res[] = {"linear_with_residual", "gang_linear_res_mi300", "gang_linear_res_n_tiling_mi300",
+                                   "gang_linear_res_msplit_mi300"};
+  static const char *fused_silu[] = {"linear_silu_mi300", "gang_linear_silu_mi300"};
+  for (auto p : plain)
+    if (n == p) return true;
+  for (auto p : with_res)
+    if (n == p) {
+      *res = true;
+      return true;
+    }
+  for (auto p : fused_silu)
+    if (n == p) {
+      *silu = true;
+      return true;
+    }
+  if (n == "splitk_linear_res_atomic_mi300") {  // [input, weight, residual, workspace, done_counter, output]
+    *res = true;
+    *n_extra_inputs = 2;
+    return true;
+  }
+  if (n == "gang_splitk_linear_res_mi300") {  // [input, weight, residual, workspace, output]
+    *res = true;
+    *n_extra_inputs = 1;
+    return true;
+  }
+  return false;
+}
+
+int resolve_weight(mk_graph *g, int id, int64_t k, MkWeight *w, int64_t *rows_out, int *group_half) {
+  const Tensor &t = g->tensors[id];
+  memset(w, 0, sizeof(*w));
+  if (t.ndims != 2) return fail(MK_EINVAL, "weight '%s' must be 2-D", t.name.c_str());
+  if (t.dtype != MK_DT_BF16) return fail(MK_EINVAL, "weight '%s' must be bf16", t.name.c_str());
+  if (t.dims[1] != k) return fail(MK_EINVAL, "weight '%s' has k=%lld, expected %lld", t.name.c_str(), (long long)t.dims[1], (long long)k);
+  *rows_out = t.dims[0];
+  *group_half = 0;
+  if (t.kind != T_SHUFFLED) {
+    if (!t.ptr) return fail(MK_EINVAL, "weight '%s' has no storage", t.name.c_str());
+    w->nseg = 1;
+    w->seg[0] = t.ptr;
+    w->seg_rows[0] = (int)t.dims[0];
+    w->group_rows = (int)t.dims[0];
+    return MK_OK;
+  }
+  const int n = (int)t.sources.size();
+  if (n > MK_MAX_SEGS) return fail(MK_EUNSUPPORTED, "shuffled weight '%s' has %d sources (max %d)", t.name.c_str(), n, MK_MAX_SEGS);
+  int groups = t.interleave ? t.num_groups : 1;
+  int total = 0;
+  for (int i = 0; i < n; i++) {
+    const Tensor &s = g->tensors[t.sources[i]];
+    if (s.kind == T_SHUFFLED || !s.ptr) return fail(MK_EINVAL, "source '%s' of '%s' has no storage", s.name.c_str(), t.name.c_str());
+    if (s.dims[0] % groups) return fail(MK_EINVAL, "source '%s' rows %lld not divisible by %d groups", s.name.c_str(), (long long)s.dims[0], groups);
+    w->seg[i] = s.ptr;
+    w->seg_rows[i] = (int)(s.dims[0] / groups);
+    total += w->seg_rows[i];
+  }
+  w->nseg = n;
+  w->group_rows = total;
+  if (n == 2 && w->seg_rows[0] == w->seg_rows[1]) *group_half = w->seg_rows[0];
+  return MK_OK;
+}
+
+std::string fmt(const char *f, ...) {
+  char buf[512];
+  va_list ap;
+  va_start(ap, f);
+  vsnprintf(buf, sizeof(buf), f, ap);
+  va_end(ap);
+  return buf;
+}
+
+// Lower one linear-type task (optionally preceded by a norm task whose output it consumes, optionally
+// followed by a silu_mul consuming its output) into stages.
+int lower_linear(mk_graph *g, size_t &i) {
+  const Task *norm = nullptr;
+  if (is_norm(g->tasks[i].name)) {
+    norm = &g->tasks[i];
+    i++;
+  }
+  const Task &lt = g->tasks[i];
+  bool res, silu;
+  int extra;
+  if (!linear_kind(lt.name, &res, &silu, &extra)) return fail(MK_EINVAL, "internal: '%s' is not a linear", lt.name.c_str());
+  const size_t need_ops = 3 + (res ? 1 : 0) + extra;
+  if (lt.ops.size() != need_ops) return fail(MK_EINVAL, "task '%s' expects %zu operands, got %zu", lt.name.c_str(), need_ops, lt.ops.size());
+  const int in_id = lt.ops[0], w_id = lt.ops[1], res_id = res ? lt.ops[2] : -1, out_id = lt.ops.back();
+  const Tensor &tin = g->tensors[in_id];
+  Tensor &tout = g->tensors[out_id];
+  if (tin.ndims != 2 || tout.ndims != 2) return fail(MK_EINVAL, "task '%s': input/output must be 2-D", lt.name.c_str());
+  if (tin.dtype != MK_DT_BF16 || tout.dtype != MK_DT_BF16) return fail(MK_EINVAL, "task '%s': activations must be bf16", lt.name.c_str());
+  MkStage st;
+  memset(&st, 0, sizeof(st));
+  st.op = MK_OP_LINEAR;
+  st.k = (int)tin.dims[1];
+  if (st.k % 8) return fail(MK_EINVAL, "task '%s': reduction length %d must be a multiple of 8", lt.name.c_str(), st.k);
+  int64_t rows;
+  int half;
+  int rc = resolve_weight(g, w_id, st.k, &st.w, &rows, &half);
+  if (rc) return rc;
+  st.n = (int)rows;
+  st.eps = g->cfg.rms_eps;
+  // a following silu_mul over this linear's (library-owned) output is folded into the epilogue
+  const Task *act = nullptr;
+  if (!silu && !res && i + 1 < g->tasks.size() && g->tasks[i + 1].name == "silu_mul" && g->tasks[i + 1].ops.size() == 2 &&
+      g->tasks[i + 1].ops[0] == out_id && tout.kind == T_OWNED) {
+    act = &g->tasks[i + 1];
+  }
+  int final_out = out_id;
+  if (silu || act) {
+    st.flags |= MK_F_SILU;
+    if (act) {
+      final_out = act->ops[1];
+      const int groups = act->grid[0] * act->grid[1] * act->grid[2];
+      if (groups <= 0 || (rows / 2) % groups) return fail(MK_EINVAL, "silu_mul grid %d does not divide %lld outputs", groups, (long long)(rows / 2));
+      st.silu_half = (int)(rows / 2 / groups);
+    } else {
+      st.silu_half = half ? half : 128;  // physically interleaved weight: reference layout [gate128 ; up128]
+    }
+    if (half && half != st.silu_half) return fail(MK_EINVAL, "task '%s': shuffled group half %d != activation half %d", lt.name.c_str(), half, st.silu_half);
+    if (rows % (2 * st.silu_half)) return fail(MK_EINVAL, "task '%s': %lld rows not a multiple of %d", lt.name.c_str(), (long long)rows, 2 * st.silu_half);
+  }
+  const Tensor &tfo = g->tensors[final_out];
+  const int n_out = (st.flags & MK_F_SILU) ? st.n / 2 : st.n;
+  if (tfo.ndims != 2 || tfo.dims[1] < n_out) return fail(MK_EINVAL, "task '%s': output '%s' has %lld columns, need %d", lt.name.c_str(), tfo.name.c_str(), (long long)tfo.dims[1], n_out);
+  if (tin.dims[0] < g->cfg.max_num_batched_tokens || tfo.dims[0] < g->cfg.max_num_batched_tokens)
+    return fail(MK_EINVAL, "task '%s': activations need at least max_num_batched_tokens=%d rows", lt.name.c_str(), g->cfg.max_num_batched_tokens);
+  st.in = tin.ptr;
+  st.ld_in = (int)tin.strides[0];
+  st.out = tfo.ptr;
+  st.ld_out = (int)tfo.strides[0];
+  if (res) {
+    const Tensor &tr = g->tensors[res_id];
+    if (tr.ndims != 2 || tr.dims[1] < n_out || tr.dtype != MK_DT_BF16) return fail(MK_EINVAL, "task '%s': bad residual '%s'", lt.name.c_str(), tr.name.c_str());
+    st.flags |= MK_F_RES;
+    st.res = tr.ptr;
+    st.ld_res = (int)tr.strides[0];
+  }
+  if (norm) {
+    const Tensor &nx = g->tensors[norm->ops[0]];
+    const Tensor &nw = g->tensors[norm->ops[1]];
+    const Tensor &no = g->tensors[norm->ops[2]];
+    if (nx.ndims != 2 || nx.dims[1] != st.k || nw.elems() != (size_t)st.k || nw.dtype != MK_DT_BF16)
+      return fail(MK_EINVAL, "task '%s': norm shapes do not match k=%d", norm->name.c_str(), st.k);
+    MkStage ns;
+    memset(&ns, 0, sizeof(ns));
+    ns.op = MK_OP_NORM;
+    ns.flags = MK_F_ONLY_MULTI;
+    ns.k = st.k;
+    ns.eps = g->cfg.rms_eps;
+    ns.in = nx.ptr;
+    ns.ld_in = (int)nx.strides[0];
+    ns.norm_w = nw.ptr;
+    ns.out = no.ptr;
+    ns.ld_out = (int)no.strides[0];
+    g->stages.push_back(ns);
+    g->stage_desc.push_back(fmt("NORM[multi-token only] %s -> %s k=%d", nx.name.c_str(), no.name.c_str(), st.k));
+    st.flags |= MK_F_NORM;
+    st.in = nx.ptr;
+    st.ld_in = (int)nx.strides[0];
+    st.norm_w = nw.ptr;
+    st.norm_out = no.ptr;
+  }
+  g->stages.push_back(st);
+  g->stage_desc.push_back(fmt("LINEAR%s%s%s %s x %s -> %s n=%d k=%d segs=%d", (st.flags & MK_F_NORM) ? "+norm" : "", (st.flags & MK_F_RES) ? "+res" : "",
+                              (st.flags & MK_F_SILU) ? "+silu" : "", tin.name.c_str(), g->tensors[w_id].name.c_str(), tfo.name.c_str(), st.n, st.k,
+                              st.w.nseg));
+  g->weight_bytes += (int64_t)st.n * st.k * 2;
+  i += act ? 2 : 1;
+  return MK_OK;
+}
+
+int lower_attention(mk_graph *g, size_t &i) {
+  const Task &t0 = g->tasks[i];
+  int in_id, kc_id, vc_id, qn_id, kn_id, cos_id, sin_id, out_id, qws_id = -1, nq = 0;
+  size_t consumed = 1;
+  if (t0.name == "gang_attn_split_kv_mi300") {
+    if (t0.ops.size() != 10 || t0.params.size() < 10) return fail(MK_EINVAL, "gang_attn_split_kv_mi300 expects 10 operands / 10 params");
+    in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
+    out_id = t0.ops[8]; qws_id = t0.ops[9];
+    nq = t0.params[0];
+    if (t0.params[6] != 1) return fail(MK_EUNSUPPORTED, "num_kv_chunks=%d: the kernel splits KV internally; pass 1 and drop the merge layer", t0.params[6]);
+  } else if (t0.name == "kv_cache_update_mi300") {
+    if (t0.ops.size() != 8 || t0.params.size() < 7) return fail(MK_EINVAL, "kv_cache_update_mi300 expects 8 operands / 7 params");
+    if (i + 1 >= g->tasks.size() || g->tasks[i + 1].name != "paged_attention_ck_fmha_split_kv_mi300")
+      return fail(MK_EUNSUPPORTED, "kv_cache_update_mi300 must be followed by paged_attention_ck_fmha_split_kv_mi300");
+    const Task &t1 = g->tasks[i + 1];
+    if (t1.ops.size() != 5 || t1.params.size() < 9) return fail(MK_EINVAL, "paged_attention_ck_fmha_split_kv_mi300 expects 5 operands / 9 params");
+    in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
+    qws_id = t0.ops[7];
+    if (t1.ops[0] != qws_id || t1.ops[1] != kc_id || t1.ops[2] != vc_id) return fail(MK_EINVAL, "attention does not consume the q workspace / caches of the preceding kv_cache_update");
+    out_id = t1.ops[3];
+    nq = t0.params[0];
+    if (t1.params[5] != 1) return fail(MK_EUNSUPPORTED, "num_kv_chunks=%d: the kernel splits KV internally; pass 1 and drop the merge layer", t1.params[5]);
+    consumed = 2;
+  } else {
+    return fail(MK_EUNSUPPORTED, "attention task '%s' is not supported", t0.name.c_str());
+  }
+  const Tensor &tin = g->tensors[in_id], &kc = g->tensors[kc_id], &vc = g->tensors[vc_id], &to = g->tensors[out_id];
+  if (kc.ndims != 4 || vc.ndims != 4) return fail(MK_EINVAL, "k/v cache must be 4-D [pages, page_size, kv_heads, head_dim]");
+  const int nkv = (int)kc.dims[2], D = (int)kc.dims[3];
+  if (D != 128) return fail(MK_EUNSUPPORTED, "head_dim %d: only 128 is supported", D);
+  if (kc.dims[1] != g->cfg.page_size) return fail(MK_EINVAL, "k cache page size %lld != configured %d", (long long)kc.dims[1], g->cfg.page_size);
+  if (nkv <= 0 || nq % nkv) return fail(MK_EINVAL, "q heads %d not a multiple of kv heads %d", nq, nkv);
+  const int qpk = nq / nkv;
+  if (qpk != 4 && qpk != 8) return fail(MK_EUNSUPPORTED, "q heads per kv head = %d: supported 4 and 8", qpk);
+  if (tin.ndims != 2 || tin.dims[1] != (int64_t)(nq + 2 * nkv) * D) return fail(MK_EINVAL, "attention input must be [tokens, (q+2kv)*head_dim]");
+  if (to.ndims != 2 || to.dims[1] < (int64_t)nq * D) return fail(MK_EINVAL, "attention output must be [tokens, q_heads*head_dim]");
+  MkStage st;
+  memset(&st, 0, sizeof(st));
+  st.op = MK_OP_ATTN;
+  st.eps = g->cfg.rms_eps;
+  st.in = tin.ptr;
+  st.ld_in = (int)tin.strides[0];
+  st.out = to.ptr;
+  st.ld_out = (int)to.strides[0];
+  st.k_cache = kc.ptr;
+  st.v_cache = vc.ptr;
+  st.num_q_heads = nq;
+  st.num_kv_heads = nkv;
+  st.head_dim = D;
+  st.sm_scale_log2 = (float)(1.4426950408889634 / sqrt((double)D));
+  if (qn_id >= 0 && kn_id >= 0) {
+    st.flags |= MK_F_QK_NORM;
+    st.q_norm_w = g->tensors[qn_id].ptr;
+    st.k_norm_w = g->tensors[kn_id].ptr;
+    if (g->tensors[qn_id].elems() != (size_t)D || g->tensors[kn_id].elems() != (size_t)D) return fail(MK_EINVAL, "q/k norm weights must have head_dim elements");
+  }
+  if (cos_id >= 0 && sin_id >= 0) {
+    const Tensor &c = g->tensors[cos_id];
+    if (c.ndims != 2 || c.dims[1] < D / 2 || c.dims[0] < g->cfg.max_seq_length) return fail(MK_EINVAL, "cos/sin tables must be [>=max_seq_length, >=head_dim/2]");
+    st.flags |= MK_F_ROPE;
+    st.cos_tab = c.ptr;
+    st.sin_tab = g->tensors[sin_id].ptr;
+    st.ld_cos = (int)c.strides[0];
+  }
+  if (qws_id >= 0) {
+    st.q_ws = g->tensors[qws_id].ptr;
+    st.ld_qws = (int)g->tensors[qws_id].strides[0];
+  }
+  g->stages.push_back(st);
+  g->stage_desc.push_back(fmt("ATTN %s -> %s q=%d kv=%d d=%d norm=%d rope=%d", tin.name.c_str(), to.name.c_str(), nq, nkv, D, !!(st.flags & MK_F_QK_NORM),
+                              !!(st.flags & MK_F_ROPE)));
+  i += consumed;
+  return MK_OK;
+}
+
+int lower(mk_graph *g) {
+  g->stages.clear();
+  g->stage_desc.clear();
+  g->weight_bytes = 0;
+  size_t i = 0;
+  const int B = g->cfg.max_num_batched_tokens;
+  while (i < g->tasks.size()) {
+    const Task &t = g->tasks[i];
+    bool res, silu;
+    int extra;
+    if (t.name == "embedding") {
+      if (t.ops.size() != 3) return fail(MK_EINVAL, "embedding expects 3 operands");
+      const Tensor &ids = g->tensors[t.ops[0]], &w = g->tensors[t.ops[1]], &o = g->tensors[t.ops[2]];
+      if (ids.dtype != MK_DT_I64) return fail(MK_EINVAL, "embedding ids must be int64");
+      if (w.ndims != 2 || o.ndims != 2 || w.dims[1] != o.dims[1] || w.dims[1] % 8 || w.dtype != MK_DT_BF16) return fail(MK_EINVAL, "embedding shapes mismatch");
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_EMBED;
+      st.k = (int)w.dims[1];
+      st.in = ids.ptr;
+      st.out = o.ptr;
+      st.ld_out = (int)o.strides[0];
+      st.w.nseg = 1;
+      st.w.seg[0] = w.ptr;
+      if (!t.params.empty() && t.params[0] == 0) st.flags |= MK_F_EMBED_FROM_TOKENS;
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("EMBED %s[%s] -> %s k=%d", w.name.c_str(), ids.name.c_str(), o.name.c_str(), st.k));
+      i++;
+    } else if (is_norm(t.name)) {
+      if (t.ops.size() != 3) return fail(MK_EINVAL, "%s expects 3 operands", t.name.c_str());
+      if (i + 1 < g->tasks.size() && linear_kind(g->tasks[i + 1].name, &res, &silu, &extra) && g->tasks[i + 1].ops[0] == t.ops[2]) {
+        int rc = lower_linear(g, i);
+        if (rc) return rc;
+      } else {
+        const Tensor &x = g->tensors[t.ops[0]], &w = g->tensors[t.ops[1]], &o = g->tensors[t.ops[2]];
+        if (x.ndims != 2 || o.ndims != 2 || x.dims[1] != o.dims[1] || w.elems() != (size_t)x.dims[1] || x.dims[1] % 8)
+          return fail(MK_EINVAL, "%s shapes mismatch", t.name.c_str());
+        MkStage st;
+        memset(&st, 0, sizeof(st));
+        st.op = MK_OP_NORM;
+        st.k = (int)x.dims[1];
+        st.eps = g->cfg.rms_eps;
+        st.in = x.ptr;
+        st.ld_in = (int)x.strides[0];
+        st.norm_w = w.ptr;
+        st.out = o.ptr;
+        st.ld_out = (int)o.strides[0];
+        g->stages.push_back(st);
+        g->stage_desc.push_back(fmt("NORM %s -> %s k=%d", x.name.c_str(), o.name.c_str(), st.k));
+        i++;
+      }
+    } else if (linear_kind(t.name, &res, &silu, &extra)) {
+      int rc = lower_linear(g, i);
+      if (rc) return rc;
+    } else if (t.name == "silu_mul") {
+      if (t.ops.size() != 2) return fail(MK_EINVAL, "silu_mul expects 2 operands");
+      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[t.ops[1]];
+      const int groups = t.grid[0] * t.grid[1] * t.grid[2];
+      if (x.ndims != 2 || o.ndims != 2 || x.dims[1] != 2 * o.dims[1] || groups <= 0 || o.dims[1] % groups) return fail(MK_EINVAL, "silu_mul shapes mismatch");
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_SILU_MUL;
+      st.n = (int)o.dims[1];
+      st.silu_half = (int)(o.dims[1] / groups);
+      st.groups = groups;
+      st.in = x.ptr;
+      st.ld_in = (int)x.strides[0];
+      st.out = o.ptr;
+      st.ld_out = (int)o.strides[0];
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("SILU_MUL %s -> %s n=%d half=%d", x.name.c_str(), o.name.c_str(), st.n, st.silu_half));
+      i++;
+    } else if (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300") {
+      int rc = lower_attention(g, i);
+      if (rc) return rc;
+    } else if (t.name == "argmax_partial") {
+      if (t.ops.size() != 3) return fail(MK_EINVAL, "argmax_partial expects 3 operands");
+      if (i + 1 >= g->tasks.size() || g->tasks[i + 1].name != "argmax_reduce" || g->tasks[i + 1].ops.size() != 3)
+        return fail(MK_EUNSUPPORTED, "argmax_partial must be followed by argmax_reduce");
+      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[g->tasks[i + 1].ops[2]];
+      if (x.ndims != 2 || x.dtype != MK_DT_BF16 || o.dtype != MK_DT_I64) return fail(MK_EINVAL, "argmax: logits must be 2-D bf16 and the output int64");
+      void *pv = nullptr, *pi = nullptr;
+      int rc = dev_alloc(g, &pv, sizeof(float) * (size_t)B * g->G);
+      if (rc) return rc;
+      rc = dev_alloc(g, &pi, sizeof(int) * (size_t)B * g->G);
+      if (rc) return rc;
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_ARGMAX_PARTIAL;
+      st.n = (int)x.dims[1];
+      st.in = x.ptr;
+      st.ld_in = (int)x.strides[0];
+      st.aux0 = pv;
+      st.aux1 = pi;
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("ARGMAX_PARTIAL %s n=%d", x.name.c_str(), st.n));
+      MkStage sr;
+      memset(&sr, 0, sizeof(sr));
+      sr.op = MK_OP_ARGMAX_REDUCE;
+      sr.aux0 = pv;
+      sr.aux1 = pi;
+      sr.out = o.ptr;
+      g->stages.push_back(sr);
+      g->stage_desc.push_back(fmt("ARGMAX_REDUCE -> %s", o.name.c_str()));
+      i += 2;
+    } else {
+      return fail(MK_EUNSUPPORTED, "task '%s' has no MI355X lowering", t.name.c_str());
+    }
+  }
+  g->program_text.clear();
+  for (size_t s = 0; s < g->stage_desc.size(); s++) g->program_text += fmt("%3zu ", s) + g->stage_desc[s] + "\n";
+  return MK_OK;
+}
+
+// ---- reference-shaped task graph (JSON) ------------------------------------------------------
+// One task per grid block of every recorded operator, events between consecutive operators with
+// the gcd partition-matching rule of the reference (src/kernel/runtime.cc:519-557), task 0 =
+// TERMINATE, task 1 = BEGIN_TASK_GRAPH, event 0 = TERMINATION, event 1 = LAUNCH_DEPENDENT_TASKS over
+// [2, N), last event = END_OF_TASK_GRAPH (runtime.cc:176-182,590-595,1662-1665).
+struct RefTask {
+  int op_index;
+  int bid[3];
+  long long trigger_event, dependent_event;
+};
+struct RefEvent {
+  int type, num_triggers, first_task, last_task;
+};
+
+int task_type_id(const std::string &n) {
+  // runtime_header.h:91-188 task ids for the tasks this library lowers
+  static const std::map<std::string, int> ids = {
+      {"embedding", 101},       {"rmsnorm", 119},          {"gang_rmsnorm_mi300", 143}, {"linear", 120},
+      {"linear_with_residual", 108}, {"silu_mul", 118},    {"argmax_partial", 110},     {"argmax_reduce", 111},
+      {"splitk_linear_res_atomic_mi300", 133}, {"gang_linear_mi300", 136}, {"gang_linear_res_mi300", 137},
+      {"gang_attn_split_kv_mi300", 138}, {"kv_cache_update_mi300", 140}, {"paged_attention_ck_fmha_split_kv_mi300", 141},
+      {"gang_linear_silu_mi300", 142}, {"linear_silu_mi300", 182}, {"splitk_linear_mi300", 129}, {"gang_splitk_linear_res_mi300", 144},
+      {"gang_linear_n_tiling_mi300", 147}, {"gang_linear_res_n_tiling_mi300", 148}, {"gang_linear_msplit_mi300", 183},
+      {"gang_linear_res_msplit_mi300", 184}};
+  auto it = ids.find(n);
+  return it == ids.end() ? 0 : it->second;
+}
+
+// partition of the tensor shared by producer and consumer along each of its dims
+void partition_of(const Task &t, int operand, int ndims, int part[4]) {
+  for (int d = 0; d < 4; d++) part[d] = 1;
+  for (int a = 0; a < 3; a++) {
+    const int d = t.maps[operand][a];
+    if (d >= 0 && d < ndims) part[d] = t.grid[a];
+  }
+}
+
+int build_task_graph_json(mk_graph *g) {
+  std::vector<RefTask> tasks;
+  std::vector<RefEvent> events;
+  tasks.push_back({-1, {0, 0, 0}, 0, 0});  // TERMINATE
+  tasks.push_back({-1, {0, 0, 0}, 0, 0});  // BEGIN_TASK_GRAPH
+  events.push_back({911 /*EVENT_TERMINATION*/, 0, 0, 0});
+  events.push_back({903 /*EVENT_LAUNCH_DEPENDENT_TASKS*/, 1, 2, 0});
+  std::vector<std::pair<int, int>> op_range;  // [first, last) task per operator
+  for (size_t oi = 0; oi < g->tasks.size(); oi++) {
+    const Task &t = g->tasks[oi];
+    const int first = (int)tasks.size();
+    for (int x = 0; x < t.grid[0]; x++)
+      for (int y = 0; y < t.grid[1]; y++)
+        for (int z = 0; z < t.grid[2]; z++) tasks.push_back({(int)oi, {x, y, z}, 0, 0});
+    op_range.push_back({first, (int)tasks.size()});
+  }
+  tasks[1].trigger_event = 1;
+  // events between consecutive operators
+  for (size_t oi = 0; oi + 1 < g->tasks.size(); oi++) {
+    const Task &p = g->tasks[oi], &c = g->tasks[oi + 1];
+    // the shared tensor: an operand of the consumer that the producer also lists
+    int po = -1, co = -1;
+    for (size_t a = 0; a < c.ops.size() && po < 0; a++)
+      for (size_t b = p.ops.size(); b-- > 0;)
+        if (p.ops[b] == c.ops[a]) {
+          po = (int)b;
+          co = (int)a;
+          break;
+        }
+    int ev_parts = 1;
+    int pp[4] = {1, 1, 1, 1}, cp[4] = {1, 1, 1, 1};
+    if (po >= 0) {
+      const int nd = g->tensors[p.ops[po]].ndims;
+      partition_of(p, po, nd, pp);
+      partition_of(c, co, nd, cp);
+      for (int d = 0; d < nd; d++) ev_parts *= std::gcd(pp[d], cp[d]);
+    }
+    const int np = op_range[oi].second - op_range[oi].first, nc = op_range[oi + 1].second - op_range[oi + 1].first;
+    if (np % ev_parts || nc % ev_parts) ev_parts = 1;
+    for (int e = 0; e < ev_parts; e++) {
+      const int ev = (int)events.size();
+      const int pf = op_range[oi].first + e * (np / ev_parts), cf = op_range[oi + 1].first + e * (nc / ev_parts);
+      events.push_back({900 /*EVENT_EMPTY: consumers carry dependent_event*/, np / ev_parts, cf, cf + nc / ev_parts});
+      for (int k = 0; k < np / ev_parts; k++) tasks[pf + k].trigger_event = ev;
+      for (int k = 0; k < nc / ev_parts; k++) tasks[cf + k].dependent_event = ev;
+    }
+  }
+  // last operator triggers END_OF_TASK_GRAPH
+  const int end_ev = (int)events.size();
+  if (!g->tasks.empty()) {
+    const int lf = op_range.back().first, ll = op_range.back().second;
+    events.push_back({910 /*EVENT_END_OF_TASK_GRAPH*/, ll - lf, 0, 0});
+    for (int k = lf; k < ll; k++) tasks[k].trigger_event = end_ev;
+  }
+  events[1].last_task = (int)tasks.size();
+  g->num_ref_tasks = (int)tasks.size();
+  g->num_ref_events = (int)events.size();
+  // sanity check (reference: runtime.cc:614-674): simulate once; every task runs once, every event fires once
+  {
+    std::vector<int> counter(events.size(), 0), fired(events.size(), 0), ran(tasks.size(), 0);
+    std::vector<int> ready;
+    ran[1] = 1;
+    fired[1] = 1;
+    for (int k = 2; k < (int)tasks.size(); k++)
+      if (tasks[k].dependent_event == 0) ready.push_back(k);
+    size_t head = 0;
+    while (head < ready.size()) {
+      const int k = ready[head++];
+      if (ran[k]++) return fail(MK_EINVAL, "task graph sanity check: task %d scheduled twice", k);
+      const long long ev = tasks[k].trigger_event;
+      if (++counter[ev] == events[ev].num_triggers) {
+        if (fired[ev]++) return fail(MK_EINVAL, "task graph sanity check: event %lld fired twice", ev);
+        for (int c2 = events[ev].first_task; c2 < events[ev].last_task && events[ev].type == 900; c2++) ready.push_back(c2);
+      }
+    }
+    for (int k = 2; k < (int)tasks.size(); k++)
+      if (ran[k] != 1) return fail(MK_EINVAL, "task graph sanity check: task %d ran %d times", k, ran[k]);
+    if (!g->tasks.empty() && fired[end_ev] != 1) return fail(MK_EINVAL, "task graph sanity check: END_OF_TASK_GRAPH fired %d times", fired[end_ev]);
+  }
+  // JSON
+  std::string &j = g->json;
+  j.clear();
+  j += "{\n \"all_tasks\": [\n";
+  for (size_t k = 0; k < tasks.size(); k++) {
+    const RefTask &rt = tasks[k];
+    int type = k == 0 ? 0 /*TASK_TERMINATE*/ : (k == 1 ? 10 /*TASK_BEGIN_TASK_GRAPH*/ : task_type_id(g->tasks[rt.op_index].name));
+    j += fmt("  {\"task_type\": %d, \"variant_id\": 0, \"inputs\": [", type);
+    std::string outs;
+    if (rt.op_index >= 0) {
+      const Task &t = g->tasks[rt.op_index];
+      // operands: inputs first, outputs last; count outputs by task type
+      int n_out = 1;
+      if (t.name == "argmax_partial") n_out = 2;
+      if (t.name == "gang_attn_split_kv_mi300") n_out = 3;
+      if (t.name == "paged_attention_ck_fmha_split_kv_mi300") n_out = 2;
+      const int n_in = (int)t.ops.size() - n_out;
+      bool first_in = true, first_out = true;
+      for (size_t a = 0; a < t.ops.size(); a++) {
+        const Tensor &tn = g->tensors[t.ops[a]];
+        long long off = 0;
+        long long dims[4];
+        for (int d = 0; d < tn.ndims; d++) dims[d] = tn.dims[d];
+        for (int ax = 0; ax < 3; ax++) {
+          const int d = t.maps[a][ax];
+          if (d >= 0 && d < tn.ndims && t.grid[ax] > 0) {
+            const long long per = tn.dims[d] / std::gcd((long long)tn.dims[d], (long long)t.grid[ax]);
+            dims[d] = per;
+            off += per * rt.bid[ax] * tn.strides[d] * (long long)dtype_size(tn.dtype);
+          }
+        }
+        std::string e = fmt("{\"base_ptr\": \"%s\", \"offset\": %lld, \"data_type\": %d, \"dims\": [", tn.name.c_str(), off, tn.dtype);
+        for (int d = 0; d < tn.ndims; d++) e += fmt(d ? ", %lld" : "%lld", dims[d]);
+        e += "], \"strides\": [";
+        for (int d = 0; d < tn.ndims; d++) e += fmt(d ? ", %lld" : "%lld", (long long)tn.strides[d]);
+        e += "]}";
+        if ((int)a < n_in) {
+          j += (first_in ? "" : ", ") + e;
+          first_in = false;
+        } else {
+          outs += (first_out ? "" : ", ") + e;
+          first_out = false;
+        }
+      }
+    }
+    j += "], \"outputs\": [" + outs + "], ";
+    j += fmt("\"trigger_event\": %lld, \"dependent_event\": %lld, \"request_id\": %d, \"expert_offset\": 0, \"kv_idx\": %d, "
+             "\"merge_task_offset\": 0, \"n_tile_start\": 0, \"n_tile_count\": 0}%s\n",
+             rt.trigger_event, rt.dependent_event, rt.bid[0], rt.bid[1], k + 1 < tasks.size() ? "," : "");
+  }
+  j += " ],\n \"all_events\": [\n";
+  for (size_t e = 0; e < events.size(); e++)
+    j += fmt("  {\"event_type\": %d, \"num_triggers\": %d, \"first_task_id\": %d, \"last_task_id\": %d}%s\n", events[e].type, events[e].num_triggers,
+             events[e].first_task, events[e].last_task, e + 1 < events.size() ? "," : "");
+  j += " ],\n \"first_tasks\": [1]\n}\n";
+  return MK_OK;
+}
+
+int upload_runtime(mk_graph *g) {
+  HIP_TRY(hipMemcpy(g->d_rt, &g->h_rt, sizeof(MkRuntime), hipMemcpyHostToDevice));
+  return MK_OK;
+}
+
+int do_launch(mk_graph *g, hipStream_t stream, int max_iters, int run_scheduler) {
+  if (!g->compiled) return fail(MK_ESTATE, "mk_compile has not been called");
+  if (g->launch_pending) return fail(MK_ESTATE, "a launch is still pending: call mk_wait first");
+  HIP_TRY(hipSetDevice(g->cfg.device));
+  HIP_TRY(hipMemsetAsync(g->d_sync, 0, sizeof(MkSync), stream));
+  const MkRuntime *rtp = g->d_rt;
+  void *args[] = {(void *)&rtp, (void *)&max_iters, (void *)&run_scheduler};
+  HIP_TRY(hipEventRecord(g->ev0, stream));
+  HIP_TRY(hipLaunchCooperativeKernel((const void *)mk_persistent_kernel, dim3(g->G), dim3(MK_THREADS), args, MK_LDS_BYTES, stream));
+  HIP_TRY(hipEventRecord(g->ev1, stream));
+  g->launch_pending = true;
+  return MK_OK;
+}
+
+int do_wait(mk_graph *g, hipStream_t stream, int *finished_out) {
+  if (!g->launch_pending) return fail(MK_ESTATE, "no launch pending");
+  HIP_TRY(hipStreamSynchronize(stream));
+  g->launch_pending = false;
+  float ms = 0.f;
+  HIP_TRY(hipEventElapsedTime(&ms, g->ev0, g->ev1));
+  g->last_ms = ms;
+  MkSync hs;
+  HIP_TRY(hipMemcpy(&hs, g->d_sync, sizeof(MkSync), hipMemcpyDeviceToHost));
+  int nx = 0;
+  for (int i = 0; i < MK_MAX_XCD; i++) nx += hs.xcd_count[i] > 0;
+  g->last_nxcd = nx;
+  g->last_aborted = hs.abort_flag != 0;
+  MkSched sc;
+  HIP_TRY(hipMemcpy(&sc, g->d_sched, sizeof(MkSched), hipMemcpyDeviceToHost));
+  if (finished_out) *finished_out = sc.finished;
+  if (hs.abort_flag) return fail(MK_EABORT, "kernel watchdog fired (barrier epoch %u): a workgroup waited longer than the spin limit", hs.abort_where);
+  return MK_OK;
+}
+
+}  // namespace
+
+// ============================================================================ C ABI
+extern "C" {
+
+const char *mk_last_error(void) { return g_err.c_str(); }
+const char *mk_version(void) { return "fleet_mk 0.1 (gfx950)"; }
+
+int mk_graph_create(const mk_config *cfg, mk_graph **out) {
+  if (!cfg || !out) return fail(MK_EINVAL, "null argument");
+  if (cfg->max_num_batched_tokens < 1 || cfg->max_num_batched_tokens > MK_MAX_TOKENS)
+    return fail(MK_EINVAL, "max_num_batched_tokens=%d outside [1, %d]", cfg->max_num_batched_tokens, MK_MAX_TOKENS);
+  if (cfg->max_num_batched_requests < 1 || cfg->max_num_batched_requests > MK_MAX_TOKENS)
+    return fail(MK_EINVAL, "max_num_batched_requests=%d outside [1, %d]", cfg->max_num_batched_requests, MK_MAX_TOKENS);
+  if (cfg->page_size < 1 || cfg->max_num_pages < 1 || cfg->max_seq_length < 2) return fail(MK_EINVAL, "bad page_size / max_num_pages / max_seq_length");
+  if ((int64_t)cfg->max_num_pages * cfg->page_size < cfg->max_seq_length)
+    return fail(MK_EINVAL, "max_num_pages*page_size=%lld cannot hold one sequence of max_seq_length=%d", (long long)cfg->max_num_pages * cfg->page_size,
+                cfg->max_seq_length);
+  if (cfg->max_num_pages > (MK_LDS_BYTES / 4)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 4);
+  int ndev = 0;
+  HIP_TRY(hipGetDeviceCount(&ndev));
+  if (ndev < 1) return fail(MK_EHIP, "no HIP device visible: the megakernel has no CPU fallback");
+  if (cfg->device < 0 || cfg->device >= ndev) return fail(MK_EINVAL, "device %d out of range", cfg->device);
+  HIP_TRY(hipSetDevice(cfg->device));
+  hipDeviceProp_t prop;
+  HIP_TRY(hipGetDeviceProperties(&prop, cfg->device));
+  if (strncmp(prop.gcnArchName, "gfx950", 6) != 0) return fail(MK_EUNSUPPORTED, "device is %s; this library is built for gfx950 only", prop.gcnArchName);
+  if (!prop.cooperativeLaunch) return fail(MK_EUNSUPPORTED, "device does not support cooperative launch");
+  mk_graph *g = new mk_graph();
+  g->cfg = *cfg;
+  if (g->cfg.rms_eps == 0.f) g->cfg.rms_eps = 1e-6f;
+  g->num_cus = prop.multiProcessorCount;
+  g->G = cfg->num_workers > 0 ? cfg->num_workers : g->num_cus;
+  if (g->G > g->num_cus) {
+    delete g;
+    return fail(MK_EINVAL, "num_workers=%d exceeds the %d CUs that can be co-resident", cfg->num_workers, prop.multiProcessorCount);
+  }
+  memset(&g->h_rt, 0, sizeof(g->h_rt));
+  *out = g;
+  return MK_OK;
+}
+
+int mk_graph_destroy(mk_graph *g) {
+  if (!g) return MK_OK;
+  if (g->launch_pending) (void)hipDeviceSynchronize();
+  for (void *p : g->allocs) (void)hipFree(p);
+  if (g->ev0) (void)hipEventDestroy(g->ev0);
+  if (g->ev1) (void)hipEventDestroy(g->ev1);
+  delete g;
+  return MK_OK;
+}
+
+static int add_tensor(mk_graph *g, Tensor &&t) {
+  g->tensors.push_back(std::move(t));
+  return (int)g->tensors.size() - 1;
+}
+
+int mk_tensor_attach(mk_graph *g, void *device_ptr, int ndims, const int64_t *dims, const int64_t *strides, int dtype, const char *name) {
+  if (!g || !dims || !name) return fail(MK_EINVAL, "null argument");
+  if (g->compiled) return fail(MK_ESTATE, "graph already compiled");
+  if (ndims < 1 || ndims > 4) return fail(MK_EINVAL, "tensor '%s': %d dims (1..4 supported)", name, ndims);
+  if (!dtype_size(dtype)) return fail(MK_EINVAL, "tensor '%s': unsupported dtype %d", name, dtype);
+  if (!device_ptr) return fail(MK_EINVAL, "tensor '%s': null device pointer", name);
+  Tensor t;
+  t.name = name;
+  t.ndims = ndims;
+  t.dtype = dtype;
+  t.kind = T_ATTACHED;
+  t.ptr = device_ptr;
+  int64_t expect = 1;
+  for (int i = ndims - 1; i >= 0; i--) {
+    t.dims[i] = dims[i];
+    t.strides[i] = strides ? strides[i] : expect;
+    if (t.strides[i] != expect) return fail(MK_EINVAL, "tensor '%s' is not row-major contiguous (stride[%d]=%lld, expected %lld)", name, i, (long long)t.strides[i], (long long)expect);
+    expect *= dims[i];
+  }
+  return add_tensor(g, std::move(t));
+}
+
+int mk_tensor_new(mk_graph *g, int ndims, const int64_t *dims, const int64_t *strides, int dtype, const char *name, int io_category) {
+  if (!g || !dims || !name) return fail(MK_EINVAL, "null argument");
+  if (g->compiled) return fail(MK_ESTATE, "graph already compiled");
+  if (ndims < 1 || ndims > 4) return fail(MK_EINVAL, "tensor '%s': %d dims (1..4 supported)", name, ndims);
+  if (!dtype_size(dtype)) return fail(MK_EINVAL, "tensor '%s': unsupported dtype %d", name, dtype);
+  if (io_category != MK_IO_DEVICE && io_category != MK_IO_SYMMETRIC) return fail(MK_EINVAL, "Invalid io_category: %d", io_category);
+  Tensor t;
+  t.name = name;
+  t.ndims = ndims;
+  t.dtype = dtype;
+  t.kind = T_OWNED;
+  t.io_category = io_category;
+  int64_t expect = 1;
+  size_t span = 1;
+  for (int i = ndims - 1; i >= 0; i--) {
+    t.dims[i] = dims[i];
+    t.strides[i] = strides ? strides[i] : expect;
+    expect *= dims[i];
+    span += (size_t)(dims[i] - 1) * (size_t)t.strides[i];
+  }
+  // allocate right away so later tasks can capture the address; freed in mk_graph_destroy
+  void *p = nullptr;
+  int rc = dev_alloc(g, &p, span * dtype_size(dtype));
+  if (rc) return rc;
+  t.ptr = p;
+  return add_tensor(g, std::move(t));
+}
+
+int mk_tensor_shuffle(mk_graph *g, const int *ids, int n, int dim, int num_groups, int interleave, const char *name) {
+  if (!g || !ids || !name) return fail(MK_EINVAL, "null argument");
+  if (dim != 0) return fail(MK_EUNSUPPORTED, "only dimension 0 can be shuffled/fused");
+  if (n < 1 || n > MK_MAX_SEGS) return fail(MK_EUNSUPPORTED, "shuffle of %d tensors (1..%d supported)", n, MK_MAX_SEGS);
+  if (num_groups < 1) return fail(MK_EINVAL, "num_groups must be positive");
+  Tensor t;
+  t.name = name;
+  t.kind = T_SHUFFLED;
+  t.num_groups = num_groups;
+  t.interleave = interleave != 0;
+  int64_t rows = 0;
+  for (int i = 0; i < n; i++) {
+    if (ids[i] < 0 || ids[i] >= (int)g->tensors.size()) return fail(MK_EINVAL, "bad tensor id %d", ids[i]);
+    const Tensor &s = g->tensors[ids[i]];
+    if (s.ndims != 2) return fail(MK_EINVAL, "shuffle source '%s' must be 2-D", s.name.c_str());
+    if (i && (s.dims[1] != g->tensors[ids[0]].dims[1] || s.dtype != g->tensors[ids[0]].dtype)) return fail(MK_EINVAL, "shuffle sources disagree on columns/dtype");
+    if (s.dims[0] % num_groups) return fail(MK_EINVAL, "source '%s' rows %lld not divisible by num_groups %d", s.name.c_str(), (long long)s.dims[0], num_groups);
+    rows += s.dims[0];
+    t.sources.push_back(ids[i]);
+  }
+  t.ndims = 2;
+  t.dtype = g->tensors[ids[0]].dtype;
+  t.dims[0] = rows;
+  t.dims[1] = g->tensors[ids[0]].dims[1];
+  t.strides[0] = t.dims[1];
+  t.strides[1] = 1;
+  return add_tensor(g, std::move(t));
+}
+
+int mk_tensor_num_dims(mk_graph *g, int id) {
+  if (!g || id < 0 || id >= (int)g->tensors.size()) return fail(MK_EINVAL, "bad tensor id %d", id);
+  return g->tensors[id].ndims;
+}
+int64_t mk_tensor_dim(mk_graph *g, int id, int i) {
+  if (!g || id < 0 || id >= (int)g->tensors.size()) return fail(MK_EINVAL, "bad tensor id %d", id);
+  if (i < 0 || i >= g->tensors[id].ndims) return fail(MK_EINVAL, "bad dim %d", i);
+  return g->tensors[id].dims[i];
+}
+void *mk_tensor_ptr(mk_graph *g, int id) {
+  if (!g || id < 0 || id >= (int)g->tensors.size()) return nullptr;
+  return g->tensors[id].ptr;
+}
+
+int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const int block_dim[3], int n_operands, const int *tensor_ids,
+                const int *input_maps, const int *forloop_dims, int n_params, const int *params) {
+  if (!g || !task_name || !grid_dim || !block_dim || (n_operands > 0 && !tensor_ids)) return fail(MK_EINVAL, "null argument");
+  if (g->compiled) return fail(MK_ESTATE, "graph already compiled");
+  Task t;
+  t.name = task_name;
+  for (int i = 0; i < 3; i++) {
+    t.grid[i] = grid_dim[i];
+    t.block[i] = block_dim[i];
+    if (grid_dim[i] < 1) return fail(MK_EINVAL, "task '%s': grid_dim[%d]=%d", task_name, i, grid_dim[i]);
+  }
+  for (int i = 0; i < n_operands; i++) {
+    // id -1 = optional operand that is absent (e.g. no q/k norm)
+    if (tensor_ids[i] < -1 || tensor_ids[i] >= (int)g->tensors.size()) return fail(MK_EINVAL, "task '%s': bad tensor id %d", task_name, tensor_ids[i]);
+    t.ops.push_back(tensor_ids[i]);
+    std::array<int, 3> m = {-1, -1, -1};
+    if (input_maps) m = {input_maps[3 * i], input_maps[3 * i + 1], input_maps[3 * i + 2]};
+    t.maps.push_back(m);
+    t.forloop.push_back(forloop_dims ? forloop_dims[i] : -1);
+  }
+  for (int i = 0; i < n_params; i++) t.params.push_back(params[i]);
+  // reject unknown names here, like Graph::register_task (src/kernel/graph.cc:844-847)
+  bool a, b;
+  int c;
+  static const char *known[] = {"embedding", "rmsnorm", "gang_rmsnorm_mi300", "silu_mul", "gang_attn_split_kv_mi300", "kv_cache_update_mi300",
+                                "paged_attention_ck_fmha_split_kv_mi300", "argmax_partial", "argmax_reduce"};
+  bool ok = linear_kind(t.name, &a, &b, &c);
+  for (auto k : known) ok = ok || t.name == k;
+  if (!ok) return fail(MK_EUNSUPPORTED, "Unsupported task name: %s", task_name);
+  g->tasks.push_back(std::move(t));
+  return MK_OK;
+}
+
+int mk_generate_task_graph(mk_graph *g, int num_gpus, int my_gpu_id, const char **json_out) {
+  if (!g || !json_out) return fail(MK_EINVAL, "null argument");
+  if (num_gpus != 1 || my_gpu_id != 0) return fail(MK_EUNSUPPORTED, "this build runs on one GPU (num_gpus=%d, my_gpu_id=%d)", num_gpus, my_gpu_id);
+  int rc = build_task_graph_json(g);
+  if (rc) return rc;
+  *json_out = g->json.c_str();
+  return MK_OK;
+}
+
+int mk_compile(mk_graph *g) {
+  if (!g) return fail(MK_EINVAL, "null argument");
+  if (g->compiled) return fail(MK_ESTATE, "graph already compiled");
+  HIP_TRY(hipSetDevice(g->cfg.device));
+  const mk_config &c = g->cfg;
+  if (!c.step || !c.tokens || !c.input_tokens || !c.output_tokens || !c.prompt_lengths || !c.qo_indptr || !c.paged_kv_indptr || !c.paged_kv_indices ||
+      !c.paged_kv_last_page_len)
+    return fail(MK_EINVAL, "all meta tensors except num_new_tokens must be non-null device pointers");
+  int rc = lower(g);
+  if (rc) return rc;
+  rc = build_task_graph_json(g);
+  if (rc) return rc;
+  // co-residency: every workgroup must be resident for the in-kernel barriers to make progress
+  HIP_TRY(hipFuncSetAttribute((const void *)mk_persistent_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MK_LDS_BYTES));
+  int per_cu = 0;
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)mk_persistent_kernel, MK_THREADS, MK_LDS_BYTES));
+  if (per_cu < 1 || g->G > per_cu * g->num_cus) return fail(MK_EINVAL, "grid of %d workgroups cannot be co-resident (%d per CU x %d CUs)", g->G, per_cu, g->num_cus);
+  MkRuntime &rt = g->h_rt;
+  rt.num_stages = (int)g->stages.size();
+  rt.max_tokens = c.max_num_batched_tokens;
+  rt.max_requests = c.max_num_batched_requests;
+  rt.max_seq = c.max_seq_length;
+  rt.page_size = c.page_size;
+  rt.max_pages = c.max_num_pages;
+  rt.total_requests = c.total_num_requests;
+  rt.max_new_per_req = MK_MAX_NEW_PER_REQ;
+  rt.eos_token_id = c.eos_token_id;
+  rt.step = c.step;
+  rt.tokens = (long long *)c.tokens;
+  rt.input_tokens = (long long *)c.input_tokens;
+  rt.output_tokens = (long long *)c.output_tokens;
+  rt.num_new_tokens = c.num_new_tokens;
+  rt.prompt_lengths = c.prompt_lengths;
+  rt.qo_indptr = c.qo_indptr;
+  rt.kv_indptr = c.paged_kv_indptr;
+  rt.kv_indices = c.paged_kv_indices;
+  rt.kv_last_page_len = c.paged_kv_last_page_len;
+  void *p;
+  if ((rc = dev_alloc(g, &p, sizeof(int) * rt.max_requests))) return rc;
+  rt.request_ids = (int *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(int) * rt.max_pages))) return rc;
+  rt.page_queue = (int *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(int) * rt.max_tokens))) return rc;
+  rt.tok_slot = (int *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(int) * rt.max_tokens))) return rc;
+  rt.tok_pos = (int *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(int) * rt.max_tokens))) return rc;
+  rt.tok_first = (int *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(MkSched)))) return rc;
+  rt.sched = g->d_sched = (MkSched *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(MkSync)))) return rc;
+  rt.sync = g->d_sync = (MkSync *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(MkStage) * (g->stages.size() + 1)))) return rc;
+  g->d_stages = (MkStage *)p;
+  rt.stages = g->d_stages;
+  if (!g->stages.empty()) HIP_TRY(hipMemcpy(g->d_stages, g->stages.data(), sizeof(MkStage) * g->stages.size(), hipMemcpyHostToDevice));
+  // attention split-KV workspace: one partial (max, sum, 128 values) per q head of every work unit
+  int max_kv = 1;
+  for (auto &s : g->stages)
+    if (s.op == MK_OP_ATTN && s.num_kv_heads > max_kv) max_kv = s.num_kv_heads;
+  const size_t units = (size_t)std::max(g->G, rt.max_tokens * max_kv) + MK_ATTN_MAX_CHUNKS;
+  if ((rc = dev_alloc(g, &p, units * 8 * (128 + 2) * sizeof(float)))) return rc;
+  rt.attn_part = (float *)p;
+  g->attn_cnt_n = (size_t)rt.max_tokens * max_kv;
+  if ((rc = dev_alloc(g, &p, sizeof(unsigned) * g->attn_cnt_n))) return rc;
+  rt.attn_cnt = (unsigned *)p;
+  g->timing_cap = 8192;
+  if ((rc = dev_alloc(g, &p, sizeof(long long) * (g->timing_cap + 2)))) return rc;
+  rt.timing = g->d_timing = (long long *)p;
+  rt.timing_cap = g->timing_cap;
+  if ((rc = dev_alloc(g, &p, sizeof(MkRuntime)))) return rc;
+  g->d_rt = (MkRuntime *)p;
+  if ((rc = upload_runtime(g))) return rc;
+  HIP_TRY(hipEventCreate(&g->ev0));
+  HIP_TRY(hipEventCreate(&g->ev1));
+  g->compiled = true;
+  return mk_init_requests(g);
+}
+
+int mk_init_requests(mk_graph *g) {
+  if (!g || !g->compiled) return fail(MK_ESTATE, "mk_compile has not been called");
+  if (g->launch_pending) return fail(MK_ESTATE, "a launch is still pending");
+  HIP_TRY(hipSetDevice(g->cfg.device));
+  const MkRuntime &rt = g->h_rt;
+  HIP_TRY(hipDeviceSynchronize());
+  HIP_TRY(hipMemset(rt.step, 0, sizeof(int) * rt.total_requests));
+  HIP_TRY(hipMemset(rt.request_ids, 0xFF, sizeof(int) * rt.max_requests));
+  HIP_TRY(hipMemset(rt.qo_indptr, 0, sizeof(int) * (rt.max_requests + 1)));
+  HIP_TRY(hipMemset(rt.kv_indptr, 0, sizeof(int) * (rt.max_requests + 1)));
+  std::vector<int> pq(rt.max_pages);
+  for (int i = 0; i < rt.max_pages; i++) pq[i] = i;
+  HIP_TRY(hipMemcpy(rt.page_queue, pq.data(), sizeof(int) * rt.max_pages, hipMemcpyHostToDevice));
+  MkSched sc;
+  memset(&sc, 0, sizeof(sc));
+  sc.page_queue_head = 0;
+  sc.page_queue_tail = rt.max_pages;
+  HIP_TRY(hipMemcpy(g->d_sched, &sc, sizeof(sc), hipMemcpyHostToDevice));
+  HIP_TRY(hipMemset(rt.attn_cnt, 0, sizeof(unsigned) * g->attn_cnt_n));
+  return MK_OK;
+}
+
+int mk_enqueue_steps(mk_graph *g, void *stream, int max_iterations) {
+  if (!g) return fail(MK_EINVAL, "null argument");
+  if (max_iterations < 1) return fail(MK_EINVAL, "max_iterations must be positive");
+  return do_launch(g, (hipStream_t)stream, max_iterations, 1);
+}
+
+int mk_wait(mk_graph *g, void *stream, int *finished_out) {
+  if (!g) return fail(MK_EINVAL, "null argument");
+  return do_wait(g, (hipStream_t)stream, finished_out);
+}
+
+int mk_launch_steps(mk_graph *g, void *stream, int max_iterations, int *finished_out) {
+  int rc = mk_enqueue_steps(g, stream, max_iterations);
+  if (rc) return rc;
+  return mk_wait(g, stream, finished_out);
+}
+
+int mk_launch(mk_graph *g, void *stream) {
+  int finished = 0;
+  int rc = mk_launch_steps(g, stream, 0x7fffffff, &finished);
+  if (rc) return rc;
+  if (!finished) return fail(MK_EABORT, "kernel returned before all requests finished");
+  return MK_OK;
+}
+
+int mk_run_once(mk_graph *g, void *stream, int num_tokens, const int32_t *tok_slot, const int32_t *tok_pos, const int32_t *tok_first) {
+  if (!g || !g->compiled) return fail(MK_ESTATE, "mk_compile has not been called");
+  const MkRuntime &rt = g->h_rt;
+  if (num_tokens < 1 || num_tokens > rt.max_tokens) return fail(MK_EINVAL, "num_tokens=%d outside [1, %d]", num_tokens, rt.max_tokens);
+  if (!tok_slot || !tok_pos || !tok_first) return fail(MK_EINVAL, "null argument");
+  for (int t = 0; t < num_tokens; t++) {
+    if (tok_slot[t] < 0 || tok_slot[t] >= rt.max_requests) return fail(MK_EINVAL, "tok_slot[%d]=%d out of range", t, tok_slot[t]);
+    if (tok_pos[t] < 0 || tok_pos[t] >= rt.max_seq) return fail(MK_EINVAL, "tok_pos[%d]=%d outside [0, max_seq_length)", t, tok_pos[t]);
+    if (tok_first[t] < 0 || tok_first[t] > t || tok_slot[tok_first[t]] != tok_slot[t] || tok_pos[t] - tok_pos[tok_first[t]] != t - tok_first[t] ||
+        t - tok_first[t] >= MK_MAX_NEW_PER_REQ)
+      return fail(MK_EINVAL, "tok_first[%d]=%d is not the first row of a contiguous run of <= %d tokens of the same request", t, tok_first[t], MK_MAX_NEW_PER_REQ);
+  }
+  HIP_TRY(hipSetDevice(g->cfg.device));
+  hipStream_t s = (hipStream_t)stream;
+  HIP_TRY(hipStreamSynchronize(s));
+  HIP_TRY(hipMemcpy(rt.tok_slot, tok_slot, sizeof(int) * num_tokens, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(rt.tok_pos, tok_pos, sizeof(int) * num_tokens, hipMemcpyHostToDevice));
+  HIP_TRY(hipMemcpy(rt.tok_first, tok_first, sizeof(int) * num_tokens, hipMemcpyHostToDevice));
+  MkSched sc;
+  HIP_TRY(hipMemcpy(&sc, g->d_sched, sizeof(sc), hipMemcpyDeviceToHost));
+  sc.num_tokens = num_tokens;
+  HIP_TRY(hipMemcpy(g->d_sched, &sc, sizeof(sc), hipMemcpyHostToDevice));
+  int rc = do_launch(g, s, 1, 0);
+  if (rc) return rc;
+  return do_wait(g, s, nullptr);
+}
+
+int mk_get_stats(mk_graph *g, mk_stats *out) {
+  if (!g || !out) return fail(MK_EINVAL, "null argument");
+  memset(out, 0, sizeof(*out));
+  out->num_workgroups = g->G;
+  out->num_stages = (int)g->stages.size();
+  out->num_tasks = g->num_ref_tasks;
+  out->num_events = g->num_ref_events;
+  out->num_xcds = g->last_nxcd;
+  out->aborted = g->last_aborted;
+  out->weight_bytes = g->weight_bytes;
+  out->last_launch_ms = g->last_ms;
+  if (g->compiled && !g->launch_pending) {
+    MkSched sc;
+    HIP_TRY(hipMemcpy(&sc, g->d_sched, sizeof(sc), hipMemcpyDeviceToHost));
+    out->iterations = sc.iterations;
+  }
+  return MK_OK;
+}
+
+int mk_describe_program(mk_graph *g, const char **text_out) {
+  if (!g || !text_out) return fail(MK_EINVAL, "null argument");
+  *text_out = g->program_text.c_str();
+  return MK_OK;
+}
+
+}  // extern "C"

@@ -1,0 +1,762 @@
+// Persistent decode megakernel for gfx950 (MI355X): one cooperative launch runs
+// every decode iteration of every request.  Each iteration walks a static stage
+// program; every stage is tiled over all workgroups, with workgroups ordered
+// by the XCD they run on so that one die streams one contiguous chunk of a
+// weight matrix and shares activations through its own L2.
+//
+// Replaces, for the decode path, the reference's device runtime
+// (include/mirage/persistent_kernel/persistent_kernel.cuh:693-1907: execute_worker,
+// execute_scheduler, prepare_next_batch) and its MI300 task kernels
+// (include/mirage/persistent_kernel/tasks/mi300/*.cuh).
+#include <hip/hip_runtime.h>
+#include <stdint.h>
+#include "mk_types.h"
+
+typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+
+#define MK_SPIN_LIMIT (1u << 24)
+
+struct Ctx {
+  int vid;   // virtual workgroup id: xcd-major, so vids [x*quota, (x+1)*quota) share an L2
+  int G;     // workgroups in the grid
+  int xcd;   // XCC_ID of the CU this workgroup landed on
+  int quota; // workgroups on this XCD
+  int nxcd;  // XCDs that received at least one workgroup
+  unsigned epoch;
+  MkSync *sync;
+};
+
+// ----------------------------------------------------------------------------- small helpers
+__device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
+__device__ __forceinline__ float bf_hi(uint32_t u) { return __uint_as_float(u & 0xffff0000u); }
+__device__ __forceinline__ float bf2f(uint16_t h) { return __uint_as_float(((uint32_t)h) << 16); }
+// round-to-nearest-even float -> bf16 (hardware v_cvt_pk_bf16_f32 on gfx950)
+__device__ __forceinline__ uint32_t f2bf(float f) { return (uint32_t)__builtin_bit_cast(uint16_t, (__bf16)f); }
+__device__ __forceinline__ uint32_t pack2(float a, float b) { return f2bf(a) | (f2bf(b) << 16); }
+__device__ __forceinline__ float bfround(float f) { return __uint_as_float(f2bf(f) << 16); }
+
+__device__ __forceinline__ float dot2(uint32_t a, uint32_t b, float c) {
+  return __builtin_amdgcn_fdot2_f32_bf16(__builtin_bit_cast(bf16x2_t, a), __builtin_bit_cast(bf16x2_t, b), c, false);
+}
+__device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float c) {
+  c = dot2(a.x, b.x, c);
+  c = dot2(a.y, b.y, c);
+  c = dot2(a.z, b.z, c);
+  c = dot2(a.w, b.w, c);
+  return c;
+}
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ float group16_sum(float v) {
+#pragma unroll
+  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  return v;
+}
+__device__ __forceinline__ unsigned xcc_id() {
+  // HW_REG_XCC_ID (id 20), bits [3:0]
+  return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u;
+}
+__device__ __forceinline__ u32x4 ldg_stream(const u32x4 *p) { return __builtin_nontemporal_load(p); }
+
+// ----------------------------------------------------------------------------- grid barrier
+// Two-level barrier: workgroups of one XCD count arrivals in a counter that lives in that XCD's
+// L2; the last arriver of each XCD publishes one cross-XCD signal and waits for the other dies,
+// then releases its own die through an L2-local flag.  Replaces the reference's per-event
+// two-level counters (persistent_kernel.cuh:1214-1284).
+__device__ __forceinline__ bool spin_ok(MkSync *s, unsigned &spins, unsigned where) {
+  ++spins;
+  if ((spins & 1023u) == 0) {
+    if (__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT)) return false;
+    if (spins >= MK_SPIN_LIMIT) {
+      __hip_atomic_store(&s->abort_where, where, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      __hip_atomic_store(&s->abort_flag, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      return false;
+    }
+  }
+  return true;
+}
+
+__device__ __forceinline__ bool grid_barrier(Ctx &c, int *sh_dead) {
+  MkSync *s = c.sync;
+  asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  __syncthreads();
+  c.epoch++;
+  if (threadIdx.x == 0) {
+    const unsigned epoch = c.epoch;
+    unsigned spins = 0;
+    unsigned old = __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (old + 1 == (unsigned)c.quota * epoch) {
+      __hip_atomic_fetch_add(&s->global_ctr, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+      while (__hip_atomic_load(&s->global_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)c.nxcd * epoch &&
+             spin_ok(s, spins, epoch))
+        __builtin_amdgcn_s_sleep(1);
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      __hip_atomic_fetch_max(&s->local_flag[c.xcd][0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    } else {
+      // poll with a compare-and-swap that never succeeds: it executes in the L2 (never served by
+      // the CU's vector L1) and cannot be folded into a plain load by the compiler
+      while (true) {
+        unsigned expect = 0xFFFFFFFFu;
+        __hip_atomic_compare_exchange_strong(&s->local_flag[c.xcd][0], &expect, 0xFFFFFFFFu, __ATOMIC_RELAXED,
+                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        if (expect >= epoch || !spin_ok(s, spins, epoch)) break;
+        __builtin_amdgcn_s_sleep(1);
+      }
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    }
+    *sh_dead = (spins >= 1024u) ? (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+  }
+  __syncthreads();
+  return *sh_dead != 0;
+}
+
+// ----------------------------------------------------------------------------- scheduler
+// On-GPU continuous batching for offline serving: commit the tokens produced by the previous
+// iteration, retire finished requests and recycle their pages, then build the next batch
+// (running requests first, then new prefills).  Same observable behaviour on the ten meta
+// tensors as the reference's MODE_OFFLINE prepare_next_batch (persistent_kernel.cuh:380-536).
+// Runs on one thread.  Returns the number of tokens scheduled.
+__device__ int mk_prepare_next_batch(const MkRuntime &rt, int *scratch_pages) {
+  MkSched *sc = rt.sched;
+  const int R = rt.max_requests, B = rt.max_tokens, PS = rt.page_size, NP = rt.max_pages;
+  int head = sc->page_queue_head, tail = sc->page_queue_tail;
+  // 1. commit outputs of the previous iteration, retire finished requests
+  for (int i = 0; i < R; i++) {
+    const int req = rt.request_ids[i];
+    if (req < 0) continue;
+    const int st = rt.step[req];
+    const int q0 = rt.qo_indptr[i];
+    const int n = rt.qo_indptr[i + 1] - q0;
+    const int plen = rt.prompt_lengths[req];
+    for (int j = 0; j < n; j++) {
+      const int pos = st + j + 1;
+      if (pos >= plen && pos < rt.max_seq) rt.tokens[(long long)req * rt.max_seq + pos] = rt.output_tokens[q0 + j];
+    }
+    const int ns = st + n;
+    rt.step[req] = ns;
+    const bool full = ns + 1 >= rt.max_seq;
+    const bool eos = ns >= plen && rt.tokens[(long long)req * rt.max_seq + ns] == rt.eos_token_id;
+    if (full || eos) {
+      rt.request_ids[i] = -1;
+      const int k0 = rt.kv_indptr[i], k1 = rt.kv_indptr[i + 1];
+      for (int j = k0; j < k1; j++) {
+        rt.page_queue[tail % NP] = rt.kv_indices[j];
+        tail++;
+      }
+    }
+  }
+  // 2. snapshot the page table (it is compacted in place below)
+  const int old_pages = rt.kv_indptr[R];
+  for (int i = 0; i < old_pages; i++) scratch_pages[i] = rt.kv_indices[i];
+  // 3. running requests keep their slot order; compact over retired slots
+  int nreq = 0, ntok = 0, npage = 0;
+  for (int i = 0; i < R; i++) {
+    const int req = rt.request_ids[i];
+    if (req < 0) continue;
+    const int k0 = rt.kv_indptr[i];
+    const int had = rt.kv_indptr[i + 1] - k0;
+    rt.request_ids[nreq] = req;
+    rt.qo_indptr[nreq] = ntok;
+    rt.kv_indptr[nreq] = npage;
+    const int st = rt.step[req];
+    int n = rt.prompt_lengths[req] - st;
+    if (n > 0) n = min(n, min(rt.max_new_per_req, B - ntok));  // prefill chunk
+    else n = min(1, B - ntok);                                 // decode
+    for (int j = 0; j < n; j++) {
+      rt.input_tokens[ntok + j] = rt.tokens[(long long)req * rt.max_seq + st + j];
+      rt.tok_slot[ntok + j] = nreq;
+      rt.tok_pos[ntok + j] = st + j;
+      rt.tok_first[ntok + j] = ntok;
+    }
+    const int need = (st + n + PS - 1) / PS;
+    const int last = (st + n) % PS;
+    rt.kv_last_page_len[nreq] = last == 0 ? PS : last;
+    for (int j = 0; j < had; j++) rt.kv_indices[npage + j] = scratch_pages[k0 + j];
+    for (int j = had; j < need; j++) {
+      rt.kv_indices[npage + j] = rt.page_queue[head % NP];
+      head++;
+    }
+    npage += need;
+    ntok += n;
+    nreq++;
+  }
+  // 4. admit new requests while there is room
+  while (nreq < R && ntok < B) {
+    const int req = sc->next_request_id;
+    if (req >= rt.total_requests) break;
+    rt.request_ids[nreq] = req;
+    rt.qo_indptr[nreq] = ntok;
+    rt.kv_indptr[nreq] = npage;
+    const int n = min(rt.prompt_lengths[req], min(rt.max_new_per_req, B - ntok));
+    for (int j = 0; j < n; j++) {
+      rt.input_tokens[ntok + j] = rt.tokens[(long long)req * rt.max_seq + j];
+      rt.tok_slot[ntok + j] = nreq;
+      rt.tok_pos[ntok + j] = j;
+      rt.tok_first[ntok + j] = ntok;
+    }
+    const int need = (n + PS - 1) / PS;
+    const int last = n % PS;
+    rt.kv_last_page_len[nreq] = last == 0 ? PS : last;
+    for (int j = 0; j < need; j++) {
+      rt.kv_indices[npage + j] = rt.page_queue[head % NP];
+      head++;
+    }
+    ntok += n;
+    npage += need;
+    nreq++;
+    sc->next_request_id = req + 1;
+  }
+  // 5. clear unused slots
+  for (int i = nreq; i < R; i++) rt.request_ids[i] = -1;
+  for (int i = nreq; i <= R; i++) {
+    rt.qo_indptr[i] = ntok;
+    rt.kv_indptr[i] = npage;
+  }
+  sc->page_queue_head = head;
+  sc->page_queue_tail = tail;
+  sc->num_tokens = ntok;
+  sc->num_reqs = nreq;
+  return ntok;
+}
+
+// ----------------------------------------------------------------------------- weights
+__device__ __forceinline__ const u32x4 *weight_row(const MkWeight &w, int r, int k8) {
+  if (w.nseg == 1) return (const u32x4 *)w.seg[0] + (size_t)r * k8;
+  const int g = r / w.group_rows;
+  int o = r - g * w.group_rows;
+  int s = 0;
+  if (o >= w.seg_rows[0]) {
+    o -= w.seg_rows[0];
+    s = 1;
+    if (w.nseg > 2 && o >= w.seg_rows[1]) {
+      o -= w.seg_rows[1];
+      s = 2;
+    }
+  }
+  return (const u32x4 *)w.seg[s] + (size_t)(g * w.seg_rows[s] + o) * k8;
+}
+
+// ----------------------------------------------------------------------------- stages
+// Gather embedding rows.  Reference task: tasks/ampere/embedding.cuh:42-72.
+__device__ void stage_embed(const MkStage &st, const Ctx &c, const MkRuntime &rt, int M) {
+  const int k8 = st.k / 8;
+  for (int t = c.vid; t < M; t += c.G) {
+    long long id;
+    if (st.flags & MK_F_EMBED_FROM_TOKENS) {
+      const int req = rt.request_ids[rt.tok_slot[t]];
+      id = rt.tokens[(long long)req * rt.max_seq + rt.tok_pos[t]];
+    } else {
+      id = ((const long long *)st.in)[t];
+    }
+    const u32x4 *src = (const u32x4 *)st.w.seg[0] + (size_t)(id < 0 ? 0 : id) * k8;
+    u32x4 *dst = (u32x4 *)st.out + (size_t)t * (st.ld_out / 8);
+    const u32x4 zero = {0u, 0u, 0u, 0u};
+    for (int i = threadIdx.x; i < k8; i += MK_THREADS) dst[i] = id < 0 ? zero : src[i];
+  }
+}
+
+// Block-wide sum of one float per thread.
+__device__ __forceinline__ float block_sum(float v, float *red) {
+  v = wave_sum(v);
+  __syncthreads();
+  if ((threadIdx.x & 63) == 0) red[threadIdx.x >> 6] = v;
+  __syncthreads();
+  return red[0] + red[1] + red[2] + red[3];
+}
+
+// RMSNorm of full rows, one workgroup per token row (used when an iteration has several tokens;
+// single-token iterations fuse the norm into the consuming linear).  y = bf16((x * r) * w) with
+// r = rsqrt(mean(x^2) + eps) in fp32.  Reference task: tasks/mi300/rmsnorm_mi300.cuh:37-188.
+__device__ void stage_norm(const MkStage &st, const Ctx &c, int M, char *smem) {
+  float *red = (float *)smem;
+  const int k2 = st.k / 2;
+  for (int t = c.vid; t < M; t += c.G) {
+    const uint32_t *x = (const uint32_t *)st.in + (size_t)t * (st.ld_in / 2);
+    const uint32_t *w = (const uint32_t *)st.norm_w;
+    uint32_t *y = (uint32_t *)st.out + (size_t)t * (st.ld_out / 2);
+    float ss = 0.f;
+    for (int i = threadIdx.x; i < k2; i += MK_THREADS) {
+      const uint32_t u = x[i];
+      ss += bf_lo(u) * bf_lo(u) + bf_hi(u) * bf_hi(u);
+    }
+    ss = block_sum(ss, red);
+    const float r = rsqrtf(ss / (float)st.k + st.eps);
+    for (int i = threadIdx.x; i < k2; i += MK_THREADS) {
+      const uint32_t u = x[i], g = w[i];
+      y[i] = pack2((bf_lo(u) * r) * bf_lo(g), (bf_hi(u) * r) * bf_hi(g));
+    }
+  }
+}
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + __expf(-g)) * u; }
+
+// Single-token linear: out[n] = bf16(sum_k W[n,k] * x[k] (+ res[n])), optionally with the RMSNorm of x
+// fused in front and with the SwiGLU epilogue fused behind.  The weight matrix is streamed from HBM
+// exactly once with 128-bit loads, one 1 KB row segment per wavefront instruction; x lives in LDS as
+// packed bf16 and the products run on v_dot2_f32_bf16 with fp32 accumulation.
+// Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
+// (tasks/mi300/gang_linear_mi300.cuh:359-576).
+__device__ void stage_linear_m1(const MkStage &st, const Ctx &c, char *smem) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = st.k, k2 = K / 2, k8 = K / 8;
+  uint32_t *xs = (uint32_t *)smem;
+  float *red = (float *)(smem + 64 * 1024);
+  const uint32_t *xin = (const uint32_t *)st.in;
+  if (st.flags & MK_F_NORM) {
+    float ss = 0.f;
+    for (int i = tid; i < k2; i += MK_THREADS) {
+      const uint32_t u = xin[i];
+      xs[i] = u;
+      ss += bf_lo(u) * bf_lo(u) + bf_hi(u) * bf_hi(u);
+    }
+    ss = block_sum(ss, red);
+    const float r = rsqrtf(ss / (float)K + st.eps);
+    const uint32_t *nw = (const uint32_t *)st.norm_w;
+    uint32_t *no = (c.vid == 0) ? (uint32_t *)st.norm_out : nullptr;
+    for (int i = tid; i < k2; i += MK_THREADS) {
+      const uint32_t u = xs[i], g = nw[i];
+      const uint32_t y = pack2((bf_lo(u) * r) * bf_lo(g), (bf_hi(u) * r) * bf_hi(g));
+      xs[i] = y;
+      if (no) no[i] = y;
+    }
+  } else {
+    for (int i = tid; i < k2; i += MK_THREADS) xs[i] = xin[i];
+  }
+  __syncthreads();
+
+  const bool silu = st.flags & MK_F_SILU;
+  const int n_out = silu ? st.n / 2 : st.n;
+  const int nwaves = c.G * MK_WAVES;
+  const int rpw = (n_out + nwaves - 1) / nwaves;
+  const int r0 = (c.vid * MK_WAVES + wave) * rpw;
+  const int r1 = min(n_out, r0 + rpw);
+  const u32x4 *xs4 = (const u32x4 *)xs;
+  uint16_t *out = (uint16_t *)st.out;
+  const uint16_t *res = (const uint16_t *)st.res;
+  if (silu) {
+    const int half = st.silu_half;
+    for (int r = r0; r < r1; r++) {
+      const int vr = (r / half) * 2 * half + (r % half);
+      const u32x4 *wg = weight_row(st.w, vr, k8);
+      const u32x4 *wu = weight_row(st.w, vr + half, k8);
+      float ag = 0.f, au = 0.f;
+#pragma unroll 4
+      for (int kc = lane; kc < k8; kc += 64) {
+        const u32x4 a = ldg_stream(wg + kc);
+        const u32x4 b = ldg_stream(wu + kc);
+        const u32x4 x = xs4[kc];
+        ag = dot8(a, x, ag);
+        au = dot8(b, x, au);
+      }
+      ag = wave_sum(ag);
+      au = wave_sum(au);
+      if (lane == 0) out[r] = (uint16_t)f2bf(silu_mul(ag, au));
+    }
+  } else {
+    int r = r0;
+    for (; r + 1 < r1; r += 2) {
+      const u32x4 *w0 = weight_row(st.w, r, k8);
+      const u32x4 *w1 = weight_row(st.w, r + 1, k8);
+      float a0 = 0.f, a1 = 0.f;
+#pragma unroll 4
+      for (int kc = lane; kc < k8; kc += 64) {
+        const u32x4 a = ldg_stream(w0 + kc);
+        const u32x4 b = ldg_stream(w1 + kc);
+        const u32x4 x = xs4[kc];
+        a0 = dot8(a, x, a0);
+        a1 = dot8(b, x, a1);
+      }
+      a0 = wave_sum(a0);
+      a1 = wave_sum(a1);
+      if (lane == 0) {
+        if (st.flags & MK_F_RES) {
+          a0 += bf2f(res[r]);
+          a1 += bf2f(res[r + 1]);
+        }
+        out[r] = (uint16_t)f2bf(a0);
+        out[r + 1] = (uint16_t)f2bf(a1);
+      }
+    }
+    for (; r < r1; r++) {
+      const u32x4 *w0 = weight_row(st.w, r, k8);
+      float a0 = 0.f;
+#pragma unroll 4
+      for (int kc = lane; kc < k8; kc += 64) a0 = dot8(ldg_stream(w0 + kc), xs4[kc], a0);
+      a0 = wave_sum(a0);
+      if (lane == 0) {
+        if (st.flags & MK_F_RES) a0 += bf2f(res[r]);
+        out[r] = (uint16_t)f2bf(a0);
+      }
+    }
+  }
+}
+
+// Standalone SwiGLU over interleaved [gate ; up] groups (used when the graph keeps the
+// gate/up linear and the activation apart).  Reference task: tasks/mi300/silu_mul_mi300.cuh:42-184.
+__device__ void stage_silu_mul(const MkStage &st, const Ctx &c, int M) {
+  const int n = st.n, half = st.silu_half;
+  const uint16_t *in = (const uint16_t *)st.in;
+  uint16_t *out = (uint16_t *)st.out;
+  const int total = M * n;
+  for (int i = c.vid * MK_THREADS + threadIdx.x; i < total; i += c.G * MK_THREADS) {
+    const int t = i / n, j = i - t * n;
+    const int g = j / half, jj = j - g * half;
+    const uint16_t *row = in + (size_t)t * st.ld_in + (size_t)g * 2 * half;
+    out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(silu_mul(bf2f(row[jj]), bf2f(row[half + jj])));
+  }
+}
+
+// Per-head RMSNorm + rotate-half RoPE of one 128-wide head row by one wavefront (lane l owns elements
+// l and l+64, the two halves of a rotation pair).  The normalised value is rounded to bf16 before the
+// rotation, as in the reference (tasks/mi300/kv_cache_update_mi300.cuh:129-182).
+__device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst, const uint16_t *nw, const uint16_t *cos_row,
+                                              const uint16_t *sin_row, int flags, float eps, int lane) {
+  float x0 = bf2f(src[lane]), x1 = bf2f(src[lane + 64]);
+  if (flags & MK_F_QK_NORM) {
+    const float ss = wave_sum(x0 * x0 + x1 * x1);
+    const float r = rsqrtf(ss * (1.f / 128.f) + eps);
+    x0 = bfround((x0 * r) * bf2f(nw[lane]));
+    x1 = bfround((x1 * r) * bf2f(nw[lane + 64]));
+  }
+  if (flags & MK_F_ROPE) {
+    const float cs = bf2f(cos_row[lane]), sn = bf2f(sin_row[lane]);
+    const float y0 = x0 * cs - x1 * sn;
+    const float y1 = x0 * sn + x1 * cs;
+    x0 = y0;
+    x1 = y1;
+  }
+  dst[lane] = (uint16_t)f2bf(x0);
+  dst[lane + 64] = (uint16_t)f2bf(x1);
+}
+
+// GQA decode attention with the q/k-norm, RoPE and KV append fused in front.  Work unit =
+// (token, kv head, KV chunk); chunks of one (token, kv head) are adjacent virtual workgroups so a
+// kv head stays on one XCD.  Inside a workgroup, sixteen 16-lane groups each walk every 16th
+// position of the chunk with their own online-softmax state (fp32 running max / sum, exp2 with
+// log2e folded into the scale); each lane owns 8 of the 128 head dims.  Groups are merged through
+// LDS, chunks through an HBM workspace by the last workgroup to arrive.
+// Reference tasks: kv_cache_update_impl (tasks/mi300/kv_cache_update_mi300.cuh:41-327),
+// paged_attention_minimal_decode (tasks/mi300/paged_attention_decode_minimal_mi300.cuh:100-371),
+// gang_attention_split_kv_kernel (tasks/mi300/gang_attention_mi300.cuh:49-153).
+template <int QPK>
+__device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt, int M, char *smem) {
+  constexpr int D = 128;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int j16 = lane & 15, gg = wave * 4 + (lane >> 4);
+  const int nkv = st.num_kv_heads;
+  uint16_t *qs = (uint16_t *)smem;                          // [QPK][128]
+  uint16_t *knew = (uint16_t *)(smem + 2048);               // [8][128]
+  uint16_t *vnew = (uint16_t *)(smem + 2048 + 2048);        // [8][128]
+  int *sflag = (int *)(smem + 6144);
+  float *part = (float *)(smem + 8192);                     // [16][QPK][132]
+  const int n_items = M * nkv;
+  int cmax = c.G / n_items;
+  cmax = cmax < 1 ? 1 : (cmax > MK_ATTN_MAX_CHUNKS ? MK_ATTN_MAX_CHUNKS : cmax);
+  const int n_units = n_items * cmax;
+  const int ps = rt.page_size;
+  const u32x4 *kc = (const u32x4 *)st.k_cache;
+  const u32x4 *vc = (const u32x4 *)st.v_cache;
+
+  for (int u = c.vid; u < n_units; u += c.G) {
+    const int item = u / cmax, cidx = u - item * cmax;
+    const int t = item / nkv, h = item - t * nkv;
+    const int p = rt.tok_pos[t], L = p + 1;
+    int C = (L + 31) / 32;
+    C = C > cmax ? cmax : C;
+    if (cidx >= C) continue;
+    const int start = (int)(((long long)L * cidx) / C), end = (int)(((long long)L * (cidx + 1)) / C);
+    const int slot = rt.tok_slot[t], t0 = rt.tok_first[t], p0 = rt.tok_pos[t0];
+    const int *pages = rt.kv_indices + rt.kv_indptr[slot];
+    const int new_lo = max(start, p0);                 // new positions handled here: [new_lo, end)
+    const int n_new = end > new_lo ? end - new_lo : 0;
+    __syncthreads();  // LDS reuse across units
+    // ---- phase A: prepare q heads and the new K/V rows of this chunk
+    for (int row = wave; row < QPK + n_new; row += MK_WAVES) {
+      if (row < QPK) {
+        const uint16_t *src = (const uint16_t *)st.in + (size_t)t * st.ld_in + (size_t)h * (QPK + 2) * D + row * D;
+        prep_head_row(src, qs + row * D, (const uint16_t *)st.q_norm_w, (const uint16_t *)st.cos_tab + (size_t)p * st.ld_cos,
+                      (const uint16_t *)st.sin_tab + (size_t)p * st.ld_cos, st.flags, st.eps, lane);
+      } else {
+        const int j = row - QPK, pos = new_lo + j, tt = t0 + (pos - p0);
+        const uint16_t *src = (const uint16_t *)st.in + (size_t)tt * st.ld_in + (size_t)h * (QPK + 2) * D + QPK * D;
+        prep_head_row(src, knew + j * D, (const uint16_t *)st.k_norm_w, (const uint16_t *)st.cos_tab + (size_t)pos * st.ld_cos,
+                      (const uint16_t *)st.sin_tab + (size_t)pos * st.ld_cos, st.flags, st.eps, lane);
+        vnew[j * D + lane] = src[D + lane];
+        vnew[j * D + lane + 64] = src[D + lane + 64];
+      }
+    }
+    __syncthreads();
+    // the chunk that owns the newest position appends this token's K/V and publishes q
+    if (cidx == C - 1) {
+      const int j = p - new_lo;
+      const size_t rowi = (size_t)pages[p / ps] * ps + (p % ps);
+      uint32_t *kd = (uint32_t *)st.k_cache + (rowi * nkv + h) * (D / 2);
+      uint32_t *vd = (uint32_t *)st.v_cache + (rowi * nkv + h) * (D / 2);
+      if (tid < 64) kd[tid] = ((const uint32_t *)(knew + j * D))[tid];
+      else if (tid < 128) vd[tid - 64] = ((const uint32_t *)(vnew + j * D))[tid - 64];
+      if (st.q_ws) {
+        uint32_t *qd = (uint32_t *)st.q_ws + ((size_t)t * st.ld_qws + (size_t)h * QPK * D) / 2;
+        for (int i = tid; i < QPK * D / 2; i += MK_THREADS) qd[i] = ((const uint32_t *)qs)[i];
+      }
+    }
+    // ---- phase B: online softmax over the chunk
+    u32x4 qv[QPK];
+#pragma unroll
+    for (int hh = 0; hh < QPK; hh++) qv[hh] = ((const u32x4 *)qs)[hh * 16 + j16];
+    float m[QPK], l[QPK], acc[QPK][8];
+#pragma unroll
+    for (int hh = 0; hh < QPK; hh++) {
+      m[hh] = -INFINITY;
+      l[hh] = 0.f;
+#pragma unroll
+      for (int d = 0; d < 8; d++) acc[hh][d] = 0.f;
+    }
+    auto process = [&](const u32x4 kv, const u32x4 vv) {
+      float v[8] = {bf_lo(vv.x), bf_hi(vv.x), bf_lo(vv.y), bf_hi(vv.y), bf_lo(vv.z), bf_hi(vv.z), bf_lo(vv.w), bf_hi(vv.w)};
+#pragma unroll
+      for (int hh = 0; hh < QPK; hh++) {
+        float s = group16_sum(dot8(kv, qv[hh], 0.f)) * st.sm_scale_log2;
+        const float mn = fmaxf(m[hh], s);
+        const float alpha = __builtin_amdgcn_exp2f(m[hh] - mn);
+        const float pr = __builtin_amdgcn_exp2f(s - mn);
+        l[hh] = l[hh] * alpha + pr;
+#pragma unroll
+        for (int d = 0; d < 8; d++) acc[hh][d] = acc[hh][d] * alpha + pr * v[d];
+        m[hh] = mn;
+      }
+    };
+    const int cend = min(end, p0);
+    for (int pos = start + gg; pos < cend; pos += 16) {
+      const size_t rowi = (size_t)pages[pos / ps] * ps + (pos % ps);
+      const size_t off = (rowi * nkv + h) * (D / 8) + j16;
+      process(kc[off], vc[off]);
+    }
+    for (int j = gg; j < n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
+    // ---- phase C: merge the 16 groups through LDS
+#pragma unroll
+    for (int hh = 0; hh < QPK; hh++) {
+      float *pp = part + (gg * QPK + hh) * 132;
+#pragma unroll
+      for (int d = 0; d < 8; d++) pp[j16 * 8 + d] = acc[hh][d];
+      if (j16 == 0) {
+        pp[128] = m[hh];
+        pp[129] = l[hh];
+      }
+    }
+    __syncthreads();
+    float *gpart = rt.attn_part + (size_t)u * QPK * (D + 2);
+    uint16_t *orow = (uint16_t *)st.out + (size_t)t * st.ld_out + (size_t)h * QPK * D;
+    for (int o = tid; o < QPK * D; o += MK_THREADS) {
+      const int hh = o >> 7, d = o & 127;
+      float mx = -INFINITY;
+#pragma unroll
+      for (int g = 0; g < 16; g++) mx = fmaxf(mx, part[(g * QPK + hh) * 132 + 128]);
+      float ls = 0.f, os = 0.f;
+#pragma unroll
+      for (int g = 0; g < 16; g++) {
+        const float *pp = part + (g * QPK + hh) * 132;
+        const float wgt = __builtin_amdgcn_exp2f(pp[128] - mx);
+        ls += pp[129] * wgt;
+        os += pp[d] * wgt;
+      }
+      if (C == 1) {
+        orow[o] = (uint16_t)f2bf(os / ls);
+      } else {
+        gpart[hh * (D + 2) + d] = os;
+        if (d == 0) {
+          gpart[hh * (D + 2) + D] = mx;
+          gpart[hh * (D + 2) + D + 1] = ls;
+        }
+      }
+    }
+    if (C > 1) {
+      // ---- phase D: the last chunk to finish merges all chunks of this (token, kv head)
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0) {
+        const unsigned old = __hip_atomic_fetch_add(&rt.attn_cnt[item], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const int last = (old == (unsigned)(C - 1));
+        if (last) __hip_atomic_store(&rt.attn_cnt[item], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *sflag = last;
+      }
+      __syncthreads();
+      if (*sflag) {
+        const float *ip = rt.attn_part + (size_t)item * cmax * QPK * (D + 2);
+        for (int o = tid; o < QPK * D; o += MK_THREADS) {
+          const int hh = o >> 7, d = o & 127;
+          float mx = -INFINITY;
+          for (int cc = 0; cc < C; cc++) mx = fmaxf(mx, ip[((size_t)cc * QPK + hh) * (D + 2) + D]);
+          float ls = 0.f, os = 0.f;
+          for (int cc = 0; cc < C; cc++) {
+            const float *pp = ip + ((size_t)cc * QPK + hh) * (D + 2);
+            const float wgt = __builtin_amdgcn_exp2f(pp[D] - mx);
+            ls += pp[D + 1] * wgt;
+            os += pp[d] * wgt;
+          }
+          orow[o] = (uint16_t)f2bf(os / ls);
+        }
+      }
+    }
+  }
+}
+
+// Greedy sampling, stage 1: every workgroup scans a contiguous slice of each token's logits and keeps
+// (max, lowest index attaining it).  Reference task: tasks/mi300/argmax_mi300.cuh:78-127.
+__device__ void stage_argmax_partial(const MkStage &st, const Ctx &c, int M, char *smem) {
+  float *sv = (float *)smem;
+  int *si = (int *)(smem + 1024);
+  const int n = st.n;
+  const int per = (n + c.G - 1) / c.G;
+  const int c0 = c.vid * per, c1 = min(n, c0 + per);
+  float *pv = (float *)st.aux0;
+  int *pi = (int *)st.aux1;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int t = 0; t < M; t++) {
+    const uint16_t *row = (const uint16_t *)st.in + (size_t)t * st.ld_in;
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = c0 + threadIdx.x; i < c1; i += MK_THREADS) {
+      const float v = bf2f(row[i]);
+      if (v > best) {
+        best = v;
+        bi = i;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) {
+        best = ov;
+        bi = oi;
+      }
+    }
+    __syncthreads();
+    if (lane == 0) {
+      sv[wave] = best;
+      si[wave] = bi;
+    }
+    __syncthreads();
+    if (threadIdx.x == 0) {
+      for (int w = 1; w < MK_WAVES; w++)
+        if (sv[w] > best || (sv[w] == best && si[w] < bi)) {
+          best = sv[w];
+          bi = si[w];
+        }
+      pv[t * c.G + c.vid] = best;
+      pi[t * c.G + c.vid] = bi;
+    }
+  }
+}
+
+// Greedy sampling, stage 2: one wavefront per token reduces the per-workgroup partials.
+// Reference task: tasks/mi300/argmax_mi300.cuh:129-158.
+__device__ void stage_argmax_reduce(const MkStage &st, const Ctx &c, int M) {
+  const float *pv = (const float *)st.aux0;
+  const int *pi = (const int *)st.aux1;
+  long long *out = (long long *)st.out;
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  for (int t = c.vid * MK_WAVES + wave; t < M; t += c.G * MK_WAVES) {
+    float best = -INFINITY;
+    int bi = 0x7fffffff;
+    for (int i = lane; i < c.G; i += 64) {
+      const float v = pv[t * c.G + i];
+      const int ix = pi[t * c.G + i];
+      if (v > best || (v == best && ix < bi)) {
+        best = v;
+        bi = ix;
+      }
+    }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(best, o, 64);
+      const int oi = __shfl_xor(bi, o, 64);
+      if (ov > best || (ov == best && oi < bi)) {
+        best = ov;
+        bi = oi;
+      }
+    }
+    if (lane == 0) out[t] = (long long)bi;
+  }
+}
+
+// ----------------------------------------------------------------------------- the kernel
+extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel(const MkRuntime *rtp, int max_iters,
+                                                                                int run_scheduler) {
+  extern __shared__ __attribute__((aligned(16))) char smem[];
+  __shared__ int sh_bcast[4];
+  const MkRuntime rt = *rtp;
+  Ctx c;
+  c.G = gridDim.x;
+  c.sync = rt.sync;
+  c.xcd = xcc_id();
+  c.epoch = 0;
+  // ---- XCD discovery: rank of this workgroup inside its die, dies in use, workgroups per die
+  if (threadIdx.x == 0) {
+    MkSync *s = rt.sync;
+    const unsigned rank = __hip_atomic_fetch_add(&s->xcd_count[c.xcd], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    __hip_atomic_fetch_add(&s->init_ctr, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+    unsigned spins = 0;
+    while (__hip_atomic_load(&s->init_ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)c.G && spin_ok(s, spins, 0xFFFF0000u))
+      __builtin_amdgcn_s_sleep(1);
+    int nx = 0, before = 0;
+    for (int i = 0; i < MK_MAX_XCD; i++) {
+      const unsigned n = __hip_atomic_load(&s->xcd_count[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      nx += n > 0;
+      if (i < c.xcd) before += (int)n;
+    }
+    sh_bcast[0] = before + (int)rank;
+    sh_bcast[1] = nx;
+    sh_bcast[2] = (int)__hip_atomic_load(&s->xcd_count[c.xcd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  __syncthreads();
+  c.vid = sh_bcast[0];
+  c.nxcd = sh_bcast[1];
+  c.quota = sh_bcast[2];
+  __syncthreads();
+
+  for (int it = 0; it < max_iters; it++) {
+    // ---- scheduler step on one thread of virtual workgroup 0, published through the barrier
+    if (run_scheduler && c.vid == 0 && threadIdx.x == 0) {
+      const int ntok = mk_prepare_next_batch(rt, (int *)smem);
+      if (ntok == 0) rt.sched->finished = 1;
+      else rt.sched->iterations++;
+      if (rt.timing && rt.sched->iterations <= rt.timing_cap) rt.timing[rt.sched->iterations] = (long long)wall_clock64();
+    }
+    bool dead = false;
+    if (run_scheduler) dead = grid_barrier(c, &sh_bcast[3]);
+    if (threadIdx.x == 0) sh_bcast[0] = rt.sched->num_tokens;
+    __syncthreads();
+    const int M = sh_bcast[0];
+    __syncthreads();
+    if (M == 0 || dead) break;
+
+    for (int s = 0; s < rt.num_stages && !dead; s++) {
+      const MkStage &st = rt.stages[s];
+      const int op = st.op, flags = st.flags;
+      if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
+      switch (op) {
+        case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
+        case MK_OP_NORM: stage_norm(st, c, M, smem); break;
+        case MK_OP_LINEAR:
+          if (M == 1) stage_linear_m1(st, c, smem);
+          break;
+        case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
+        case MK_OP_ATTN:
+          if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4>(st, c, rt, M, smem);
+          else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8>(st, c, rt, M, smem);
+          break;
+        case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, M, smem); break;
+        case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, M); break;
+        default: break;
+      }
+      dead = grid_barrier(c, &sh_bcast[3]);
+    }
+    if (dead) break;
+  }
+  if (c.vid == 0 && threadIdx.x == 0 && rt.timing) rt.timing[0] = (long long)wall_clock64();
+}

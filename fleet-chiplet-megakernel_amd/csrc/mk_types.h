@@ -1,0 +1,134 @@
+// Descriptors shared between the host lowering (mk_host.cpp) and the persistent
+// decode megakernel (mk_kernel.hip).  Everything here is plain-old-data that is
+// copied to HBM once at compile() time; the kernel is data-driven and never
+// recompiled per model.
+//
+// Role in the reference: these structs take the place of TaskDesc / EventDesc /
+// RuntimeConfig (include/mirage/persistent_kernel/runtime_header.h:200-375), but
+// describe a *stage program* (one entry per fused operator, statically tiled
+// over the workgroups of the 8 XCDs) instead of per-tile tasks in queues.
+#pragma once
+#include <stdint.h>
+
+#define MK_THREADS 256        // threads per workgroup (4 wavefronts of 64)
+#define MK_WAVES 4
+#define MK_MAX_XCD 16
+#define MK_MAX_SEGS 3         // a shuffled weight has at most 3 sources (q,k,v)
+#define MK_MAX_TOKENS 64      // max tokens per iteration supported by the kernels
+#define MK_ATTN_MAX_CHUNKS 32 // split-KV fan-out limit per (token, kv head)
+#define MK_MAX_NEW_PER_REQ 8  // prefill tokens per request per iteration (reference: MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
+#define MK_LDS_BYTES (96 * 1024)  // dynamic LDS per workgroup; > 80 KB pins one workgroup per CU
+
+enum MkOp {
+  MK_OP_NONE = 0,
+  MK_OP_EMBED = 1,
+  MK_OP_NORM = 2,
+  MK_OP_LINEAR = 3,
+  MK_OP_SILU_MUL = 4,
+  MK_OP_ATTN = 5,
+  MK_OP_ARGMAX_PARTIAL = 6,
+  MK_OP_ARGMAX_REDUCE = 7,
+};
+
+enum MkStageFlags {
+  MK_F_NORM = 1,         // LINEAR: RMSNorm(in, norm_w) is applied to the input rows
+  MK_F_RES = 2,          // LINEAR: out = acc + res
+  MK_F_SILU = 4,         // LINEAR: weight rows interleave [gate ; up]; out = silu(gate)*up
+  MK_F_QK_NORM = 8,      // ATTN: per-head RMSNorm on q and k
+  MK_F_ROPE = 16,        // ATTN: rotate-half RoPE on q and k
+  MK_F_ONLY_MULTI = 32,  // stage runs only when the iteration has more than one token
+  MK_F_EMBED_FROM_TOKENS = 64,  // EMBED: ids come from tokens[req, step+j] instead of input_tokens
+};
+
+// A (possibly shuffled) weight matrix [rows, k] bf16.  Virtual row r of a shuffled
+// tensor lives in source `seg` at a row computed from the group structure, so no
+// interleaved copy is ever made (the reference materialises one,
+// src/kernel/runtime.cc:904-943).
+struct MkWeight {
+  const void *seg[MK_MAX_SEGS];
+  int seg_rows[MK_MAX_SEGS];  // rows each source contributes to one group
+  int nseg;
+  int group_rows;  // sum of seg_rows (== total rows when nseg == 1)
+  int pad0, pad1;
+};
+
+struct MkStage {
+  int op;
+  int flags;
+  int n;  // LINEAR: virtual weight rows; ARGMAX: vocabulary; SILU_MUL: output columns
+  int k;  // LINEAR: reduction length; NORM / EMBED: row length
+  int ld_in, ld_out, ld_res, silu_half;  // leading dimensions in elements; silu_half = rows of gate per group
+  float eps;
+  int groups;  // SILU_MUL: number of [gate;up] groups
+  const void *in;
+  void *out;
+  const void *res;
+  const void *norm_w;
+  void *norm_out;
+  MkWeight w;
+  // attention
+  void *k_cache, *v_cache;
+  const void *q_norm_w, *k_norm_w, *cos_tab, *sin_tab;
+  void *q_ws;
+  int num_q_heads, num_kv_heads, head_dim, ld_qws;
+  int ld_cos, pad2;
+  float sm_scale_log2;  // log2(e) / sqrt(head_dim)
+  int pad3;
+  // argmax
+  void *aux0, *aux1;
+};
+
+// Hierarchical barrier state.  One 128-byte line per counter so that XCD-local
+// counters stay in that XCD's L2.
+struct MkSync {
+  unsigned global_ctr;
+  unsigned pad0[31];
+  unsigned local_ctr[MK_MAX_XCD][32];
+  unsigned local_flag[MK_MAX_XCD][32];
+  unsigned xcd_count[MK_MAX_XCD];
+  unsigned pad1[32 - MK_MAX_XCD];
+  unsigned init_ctr;
+  unsigned pad2[31];
+  unsigned abort_flag;
+  unsigned abort_where;
+  unsigned pad3[30];
+};
+
+// Scheduler state that persists across launches (continuous batching, page ring).
+struct MkSched {
+  int page_queue_head, page_queue_tail, next_request_id, num_tokens;
+  int num_reqs, finished, pad0, pad1;
+  long long iterations;   // decode iterations executed so far (all launches)
+  long long pad2;
+};
+
+struct MkRuntime {
+  int num_stages, max_tokens, max_requests, max_seq;
+  int page_size, max_pages, total_requests, max_new_per_req;
+  long long eos_token_id;
+  // meta tensors (persistent_kernel.py:2590-2600 order)
+  int *step;
+  long long *tokens;
+  long long *input_tokens;
+  long long *output_tokens;
+  int *num_new_tokens;
+  int *prompt_lengths;
+  int *qo_indptr;
+  int *kv_indptr;
+  int *kv_indices;
+  int *kv_last_page_len;
+  // library-owned scheduler memory
+  int *request_ids;   // [max_requests] request id per batch slot, -1 = free
+  int *page_queue;    // [max_pages] ring of free page ids
+  int *tok_slot;      // [max_tokens] batch slot of each token of this iteration
+  int *tok_pos;       // [max_tokens] absolute position of each token
+  int *tok_first;     // [max_tokens] index of the first token of the same request in this iteration
+  MkSched *sched;
+  const MkStage *stages;
+  MkSync *sync;
+  // attention split-KV workspace
+  float *attn_part;     // [units][qpk][head_dim + 2]
+  unsigned *attn_cnt;   // [max_tokens * num_kv_heads]
+  long long *timing;    // optional [2 + 2*max] wall-clock ticks per iteration
+  int timing_cap, pad0;
+};

@@ -1,0 +1,553 @@
+"""PersistentKernel: the layer/task-builder API of the decode megakernel.
+
+Same surface as the reference class (python/mirage/mpk/persistent_kernel.py:368-2786) for the
+methods demo/qwen3/demo.py uses: each `*_layer` call validates shapes, then records one task
+(name, grid, operands with their partition maps, params) through the C ABI.  `compile()` lowers the
+recorded list to the MI355X stage program; `__call__` launches the persistent kernel once for the
+whole generation.  Nothing here computes: without libfleet_mk.so and a gfx950 device it raises.
+"""
+import ctypes
+import math
+
+import torch
+
+from .. import _capi
+from ..kernel import DTensor, KNGraph, bfloat16, convert_torch_type_to_dtype
+
+valid_persistent_kernel_modes = ["offline", "online", "online_notoken", "onepass", "multi_turn"]
+
+_META_ORDER = ["step", "tokens", "input_tokens", "output_tokens", "num_new_tokens", "prompt_lengths",
+               "qo_indptr_buffer", "paged_kv_indptr_buffer", "paged_kv_indices_buffer", "paged_kv_last_page_len_buffer"]
+
+_REPL = (-1, -1, -1)
+
+
+class PersistentKernel:
+    def __init__(
+        self,
+        mode: str,
+        world_size: int,
+        mpi_rank: int,
+        num_workers: int,
+        num_local_schedulers: int,
+        num_remote_schedulers: int,
+        max_seq_length: int,
+        max_num_batched_requests: int,
+        max_num_batched_tokens: int,
+        max_num_pages: int,
+        page_size: int,
+        meta_tensors: dict,
+        profiler_tensor: torch.Tensor = None,
+        trace_name: str = None,
+        spec_decode_config=None,
+        use_cutlass_kernel: bool = False,
+        eos_token_id: int = -1,
+    ):
+        self.__finalized__ = False
+        self._is_compiled = False
+        self._handle = None
+        if mode not in valid_persistent_kernel_modes:
+            raise ValueError(f"Invalid persistent kernel mode: {mode}")
+        if world_size != 1 or mpi_rank != 0:
+            raise NotImplementedError("the MI355X megakernel runs on one GPU (world_size=1, mpi_rank=0)")
+        if spec_decode_config is not None:
+            raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
+        self.mode = mode
+        self.world_size = world_size
+        self.mpi_rank = mpi_rank
+        self.num_workers = num_workers
+        self.num_local_schedulers = num_local_schedulers
+        self.num_remote_schedulers = num_remote_schedulers
+        self.max_seq_length = max_seq_length
+        self.max_num_batched_requests = max_num_batched_requests
+        self.max_num_batched_tokens = max_num_batched_tokens
+        self.max_num_pages = max_num_pages
+        self.page_size = page_size
+        self.eos_token_id = eos_token_id
+        self.meta_tensors = meta_tensors
+        self.profiler_tensor = profiler_tensor
+        self.trace_name = trace_name
+        self.use_nvshmem = False
+        self.spec_decode_config = None
+        self.use_cutlass_kernel = False
+        self.is_rocm = True
+        self.target_cc = 94  # the reference's tag for its MI300/MI350 task set (persistent_kernel.py:425-427)
+        for key in _META_ORDER:
+            if key not in meta_tensors:
+                raise KeyError(f"meta_tensors is missing '{key}'")
+        self.total_num_requests = meta_tensors["tokens"].shape[0]
+        assert self.max_seq_length == meta_tensors["tokens"].shape[1]
+        mt = meta_tensors
+        assert mt["qo_indptr_buffer"].shape[0] <= max_num_batched_requests + 1, f"qo_indptr_buffer.shape: {mt['qo_indptr_buffer'].shape}"
+        assert mt["paged_kv_indptr_buffer"].shape[0] <= max_num_batched_requests + 1, f"paged_kv_indptr_buffer.shape: {mt['paged_kv_indptr_buffer'].shape}"
+        assert mt["paged_kv_indices_buffer"].shape[0] <= max_num_pages, f"paged_kv_indices_buffer.shape: {mt['paged_kv_indices_buffer'].shape}"
+        assert mt["paged_kv_last_page_len_buffer"].shape[0] <= max_num_batched_requests, f"paged_kv_last_page_len_buffer.shape: {mt['paged_kv_last_page_len_buffer'].shape}"
+        for key in ("tokens", "input_tokens", "output_tokens"):
+            assert mt[key].dtype == torch.int64, f"{key}.dtype: {mt[key].dtype}"
+        for key in ("step", "num_new_tokens", "prompt_lengths", "qo_indptr_buffer", "paged_kv_indptr_buffer",
+                    "paged_kv_indices_buffer", "paged_kv_last_page_len_buffer"):
+            assert mt[key].dtype == torch.int32, f"{key}.dtype: {mt[key].dtype}"
+        # the library sizes the kernel-side buffers from the configuration, so the tensors must cover it
+        assert mt["qo_indptr_buffer"].shape[0] == max_num_batched_requests + 1
+        assert mt["paged_kv_indptr_buffer"].shape[0] == max_num_batched_requests + 1
+        assert mt["paged_kv_indices_buffer"].shape[0] == max_num_pages
+        assert mt["paged_kv_last_page_len_buffer"].shape[0] == max_num_batched_requests
+        assert mt["input_tokens"].numel() >= max_num_batched_tokens and mt["output_tokens"].numel() >= max_num_batched_tokens
+        device = mt["tokens"].device
+        if device.type != "cuda":
+            raise RuntimeError("meta tensors must live on the GPU: the megakernel has no CPU path")
+        self.device = device
+        lib = _capi.load()
+        cfg = _capi.MkConfig()
+        cfg.num_workers = int(num_workers) if num_workers else 0
+        cfg.max_seq_length = max_seq_length
+        cfg.max_num_batched_requests = max_num_batched_requests
+        cfg.max_num_batched_tokens = max_num_batched_tokens
+        cfg.max_num_pages = max_num_pages
+        cfg.page_size = page_size
+        cfg.total_num_requests = self.total_num_requests
+        cfg.device = device.index if device.index is not None else torch.cuda.current_device()
+        cfg.eos_token_id = int(eos_token_id)
+        cfg.rms_eps = 1e-6
+        cfg.step = mt["step"].data_ptr()
+        cfg.tokens = mt["tokens"].data_ptr()
+        cfg.input_tokens = mt["input_tokens"].data_ptr()
+        cfg.output_tokens = mt["output_tokens"].data_ptr()
+        cfg.num_new_tokens = mt["num_new_tokens"].data_ptr()
+        cfg.prompt_lengths = mt["prompt_lengths"].data_ptr()
+        cfg.qo_indptr = mt["qo_indptr_buffer"].data_ptr()
+        cfg.paged_kv_indptr = mt["paged_kv_indptr_buffer"].data_ptr()
+        cfg.paged_kv_indices = mt["paged_kv_indices_buffer"].data_ptr()
+        cfg.paged_kv_last_page_len = mt["paged_kv_last_page_len_buffer"].data_ptr()
+        handle = ctypes.c_void_p()
+        _capi.check(lib.mk_graph_create(ctypes.byref(cfg), ctypes.byref(handle)))
+        self._handle = handle
+        self._lib = lib
+        self.kn_graph = KNGraph(self)
+        self._tensors = []
+
+    # ------------------------------------------------------------------ tensors
+    def attach_input(self, torch_tensor: torch.Tensor, name: str = None) -> DTensor:
+        dims = tuple(int(d) for d in torch_tensor.shape)
+        strides = tuple(int(s) for s in torch_tensor.stride())
+        for d in range(len(dims) - 1):
+            assert strides[d] == strides[d + 1] * dims[d + 1], f"{name}: only row-major tensors can be attached"
+        assert name is not None
+        dt = convert_torch_type_to_dtype(torch_tensor.dtype)
+        if torch_tensor.device.type != "cuda":
+            raise RuntimeError(f"{name}: attached tensors must live on the GPU")
+        tid = _capi.check(self._lib.mk_tensor_attach(
+            self._handle, ctypes.c_void_p(torch_tensor.data_ptr()), len(dims), _capi.int_array(dims, ctypes.c_int64),
+            _capi.int_array(strides, ctypes.c_int64), dt.code, name.encode()))
+        t = DTensor(self, tid, dims, dt, name, torch_tensor)
+        self._tensors.append(t)
+        return t
+
+    def new_tensor(self, dims: tuple, strides: tuple = None, dtype=bfloat16, name: str = None,
+                   io_category: str = "cuda_tensor") -> DTensor:
+        assert name is not None
+        if io_category == "cuda_tensor":
+            cat = 0
+        elif io_category == "nvshmem_tensor":
+            cat = 1
+        else:
+            raise RuntimeError(f"Invalid io_category: {io_category}")
+        dims = tuple(int(d) for d in dims)
+        sp = _capi.int_array(strides, ctypes.c_int64) if strides is not None else None
+        tid = _capi.check(self._lib.mk_tensor_new(self._handle, len(dims), _capi.int_array(dims, ctypes.c_int64), sp,
+                                                  dtype.code, name.encode(), cat))
+        t = DTensor(self, tid, dims, dtype, name)
+        t._strides = tuple(strides) if strides is not None else None
+        self._tensors.append(t)
+        return t
+
+    def _shuffle(self, inputs, dim, num_groups, name, interleave):
+        ids = [t.id for t in inputs]
+        tid = _capi.check(self._lib.mk_tensor_shuffle(self._handle, _capi.int_array(ids), len(ids), dim, num_groups,
+                                                      1 if interleave else 0, (name or "shuffled").encode()))
+        rows = sum(t.dim(0) for t in inputs)
+        t = DTensor(self, tid, (rows,) + tuple(inputs[0].shape[1:]), inputs[0].dtype, name)
+        t.sources = list(inputs)
+        self._tensors.append(t)
+        return t
+
+    def fuse_tensors(self, inputs: list, fused_dim: int, num_groups: int, name: str = None) -> DTensor:
+        assert fused_dim == 0
+        return self._shuffle(inputs, fused_dim, num_groups, name, True)
+
+    def shuffle_tensors(self, inputs: list, shuffled_dim: int, num_groups: int, name: str = None) -> DTensor:
+        assert shuffled_dim == 0
+        return self._shuffle(inputs, shuffled_dim, num_groups, name, True)
+
+    def _torch_view(self, t: DTensor):
+        ptr = self._lib.mk_tensor_ptr(self._handle, t.id)
+        if not ptr:
+            raise RuntimeError(f"tensor {t.name} has no device storage (shuffled views are resolved at run time)")
+        n = 1
+        strides = getattr(t, "_strides", None)
+        if strides is None:
+            for d in t.shape:
+                n *= d
+        else:
+            n = 1 + sum((d - 1) * s for d, s in zip(t.shape, strides))
+        holder = _DevicePtr(ptr, n * t.dtype.size, t.shape, t.dtype, self.device, strides)
+        view = torch.as_tensor(holder, device=self.device)
+        return view.view(torch.bfloat16) if t.dtype.name == "bfloat16" else view
+
+    # ------------------------------------------------------------------ task recording
+    def _task(self, name, grid_dim, block_dim, operands, params=()):
+        """operands: list of (DTensor | None, input_map, forloop_dim), inputs first, outputs last."""
+        assert not self._is_compiled, "graph already compiled"
+        grid_dim = tuple(int(x) for x in grid_dim)
+        block_dim = tuple(int(x) for x in block_dim)
+        assert len(grid_dim) == 3 and len(block_dim) == 3
+        ids, maps, fl = [], [], []
+        for t, m, f in operands:
+            ids.append(-1 if t is None else t.id)
+            maps.extend(int(x) for x in m)
+            fl.append(int(f))
+        params = [int(p) for p in params]
+        _capi.check(self._lib.mk_add_task(self._handle, name.encode(), _capi.int_array(grid_dim), _capi.int_array(block_dim),
+                                          len(ids), _capi.int_array(ids), _capi.int_array(maps), _capi.int_array(fl),
+                                          len(params), _capi.int_array(params)))
+
+    # ------------------------------------------------------------------ layers (reference line numbers in each docstring)
+    def embed_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple, input_source: int = 0):
+        """persistent_kernel.py:521. input_source 0: ids are tokens[req, step+j]; 1: ids are the input tensor."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("embedding", grid_dim, block_dim,
+                   [(input, (-1, 1, -1), -1), (weight, (1, -1, -1), -1), (output, (1, 0, -1), -1)], [input_source])
+
+    def rmsnorm_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:544."""
+        assert input.num_dims == 2 and weight.num_dims == 1 and output.num_dims == 2
+        self._task("rmsnorm", grid_dim, block_dim,
+                   [(input, (0, -1, -1), 1), (weight, _REPL, 0), (output, (0, -1, -1), 1)])
+
+    def gang_rmsnorm_layer(self, input: DTensor, weight: DTensor, output: DTensor, block_dim: tuple = (128, 1, 1)):
+        """persistent_kernel.py:1553."""
+        assert input.num_dims == 2 and weight.num_dims == 1 and output.num_dims == 2
+        self._task("gang_rmsnorm_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, -1), (weight, _REPL, -1), (output, _REPL, -1)], [input.dim(0)])
+
+    def linear_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2045."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("linear", grid_dim, block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (output, (1, -1, -1), -1)])
+
+    def linear_with_residual_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2077."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        self._task("linear_with_residual", grid_dim, block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), -1), (output, (1, -1, -1), -1)])
+
+    def splitk_linear_res_atomic_layer(self, input: DTensor, weight: DTensor, residual: DTensor, workspace: DTensor, done_counter: DTensor,
+                                       output: DTensor, k_splits: int, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1920.  The MI355X kernel needs no split-K workspace; the operands are accepted and unused."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        assert grid_dim[1] == k_splits
+        assert input.dim(1) % k_splits == 0
+        self._task("splitk_linear_res_atomic_mi300", grid_dim, block_dim,
+                   [(input, (-1, 1, -1), 1), (weight, (0, 1, -1), 1), (residual, (1, -1, -1), -1), (workspace, (1, -1, -1), -1),
+                    (done_counter, (0, -1, -1), -1), (output, (1, -1, -1), -1)], [k_splits])
+
+    def _gang_params(self, weight, tile_n, output_stride, m_tiles, wg, out_rows=None):
+        batch_size = self.max_num_batched_tokens
+        output_size = weight.dim(0) if out_rows is None else out_rows
+        assert output_size % 8 == 0, f"Output size {output_size} must be divisible by 8"
+        chunk_n = output_size // 8
+        assert chunk_n % tile_n == 0, f"Chunk {chunk_n} must be divisible by tile_n {tile_n}"
+        n_tiles_per_xcd = chunk_n // tile_n
+        assert batch_size % m_tiles == 0, f"batch {batch_size} must be divisible by m_tiles {m_tiles}"
+        m_per_tile = batch_size // m_tiles
+        return [output_stride, tile_n, m_tiles, m_per_tile, n_tiles_per_xcd * m_tiles, n_tiles_per_xcd, wg]
+
+    def gang_linear_layer(self, input: DTensor, weight: DTensor, output: DTensor, tile_n: int, output_stride: int, m_tiles: int = 1,
+                          wgm: int = 0, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1571."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("gang_linear_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (output, (1, -1, -1), -1)],
+                   self._gang_params(weight, tile_n, output_stride, m_tiles, wgm))
+
+    def gang_linear_n_tiling_layer(self, input: DTensor, weight: DTensor, output: DTensor, tile_n: int, output_stride: int, m_tiles: int = 1,
+                                   wgn: int = 0, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1618 (tile traversal variant; same mathematics)."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("gang_linear_n_tiling_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (output, (1, -1, -1), -1)],
+                   self._gang_params(weight, tile_n, output_stride, m_tiles, wgn))
+
+    def gang_linear_with_residual_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, tile_n: int,
+                                        output_stride: int, m_tiles: int = 1, wgm: int = 0, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1670."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        self._task("gang_linear_res_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), -1), (output, (1, -1, -1), -1)],
+                   self._gang_params(weight, tile_n, output_stride, m_tiles, wgm))
+
+    def gang_linear_with_residual_n_tiling_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, tile_n: int,
+                                                 output_stride: int, m_tiles: int = 1, wgn: int = 0, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1737."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        self._task("gang_linear_res_n_tiling_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), -1), (output, (1, -1, -1), -1)],
+                   self._gang_params(weight, tile_n, output_stride, m_tiles, wgn))
+
+    def _msplit_params(self, weight, tile_n, output_stride, m_tiles):
+        batch_size = self.max_num_batched_tokens
+        output_size = weight.dim(0)
+        assert output_size % 8 == 0 and (output_size // 8) % tile_n == 0
+        assert batch_size % m_tiles == 0
+        n_tiles_per_xcd = output_size // 8 // tile_n
+        return [output_stride, tile_n, m_tiles, n_tiles_per_xcd, batch_size // m_tiles]
+
+    def gang_linear_msplit_layer(self, input: DTensor, weight: DTensor, output: DTensor, tile_n: int, output_stride: int, m_tiles: int = 2,
+                                 block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1782."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("gang_linear_msplit_mi300", (8 * m_tiles, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, _REPL, 1), (output, _REPL, -1)], self._msplit_params(weight, tile_n, output_stride, m_tiles))
+
+    def gang_linear_with_residual_msplit_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, tile_n: int,
+                                               output_stride: int, m_tiles: int = 2, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1817."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        self._task("gang_linear_res_msplit_mi300", (8 * m_tiles, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, _REPL, 1), (residual, _REPL, -1), (output, _REPL, -1)],
+                   self._msplit_params(weight, tile_n, output_stride, m_tiles))
+
+    def gang_splitk_linear_with_residual_layer(self, input: DTensor, weight: DTensor, residual: DTensor, workspace: DTensor, output: DTensor,
+                                               tile_n: int, output_stride: int, k_splits: int = 4, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1515.  Computed without split-K atomics (deterministic); the workspace is unused."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        output_size = weight.dim(0)
+        assert output_size % 8 == 0 and (output_size // 8) % tile_n == 0
+        self._task("gang_splitk_linear_res_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), -1), (workspace, (1, -1, -1), -1), (output, (1, -1, -1), -1)],
+                   [output_stride, tile_n, output_size // 8 // tile_n, k_splits])
+
+    def gang_ksplit_linear_with_residual_layer(self, input, weight, residual, workspace, output, tile_n, output_stride, k_splits=8,
+                                               block_dim=(256, 1, 1)):
+        """persistent_kernel.py:1468.  Same mathematics as gang_linear_with_residual_layer; lowered identically."""
+        return self.gang_splitk_linear_with_residual_layer(input, weight, residual, workspace, output, tile_n, output_stride, k_splits, block_dim)
+
+    def gang_linear_silu_layer(self, input: DTensor, weight: DTensor, output: DTensor, tile_n: int, output_stride: int, m_tiles: int = 1,
+                               wgm: int = 0, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1852.  weight interleaves [gate ; up] groups; output has half as many columns."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        assert weight.dim(0) % 2 == 0 and output.dim(1) * 2 == weight.dim(0), "output must have weight.dim(0)/2 columns"
+        self._task("gang_linear_silu_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (output, (1, -1, -1), -1)],
+                   self._gang_params(weight, tile_n, output_stride, m_tiles, wgm, out_rows=weight.dim(0) // 2))
+
+    def linear_silu_layer(self, input, weight, output, output_stride, tile_n=64, m_tiles=1, wgm=0, block_dim=(256, 1, 1)):
+        """persistent_kernel.py:1716."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        assert weight.dim(0) % 2 == 0 and output.dim(1) * 2 == weight.dim(0), "output must have weight.dim(0)/2 columns"
+        batch_size = self.max_num_batched_tokens
+        n_output_tiles = weight.dim(0) // tile_n // 2
+        m_per_tile = batch_size // m_tiles if m_tiles > 0 else batch_size
+        total_tiles = n_output_tiles * m_tiles
+        self._task("linear_silu_mi300", (total_tiles, 1, 1), block_dim,
+                   [(input, _REPL, 1), (weight, _REPL, 1), (output, _REPL, -1)],
+                   [output_stride, tile_n, m_tiles, m_per_tile, total_tiles, n_output_tiles, wgm])
+
+    def silu_mul_layer(self, input: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2137.  Each of the grid_dim[0] blocks owns one [gate ; up] column group."""
+        assert input.num_dims == 2 and output.num_dims == 2
+        assert input.dim(1) == 2 * output.dim(1)
+        self._task("silu_mul", grid_dim, block_dim, [(input, (1, -1, -1), -1), (output, (1, -1, -1), -1)])
+
+    def kv_cache_update_layer(self, input: DTensor, k_cache: DTensor, v_cache: DTensor, q_norm: DTensor, k_norm: DTensor,
+                              cos_pos_embed: DTensor, sin_pos_embed: DTensor, q_workspace: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:937."""
+        assert input.num_dims == 2
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4
+        assert q_workspace.num_dims == 2
+        head_dim = k_cache.dim(3)
+        num_kv_heads = k_cache.dim(2)
+        num_q_heads = q_workspace.dim(1) // head_dim
+        rotary_embed = 1 if cos_pos_embed is not None else 0
+        qk_norm = 1 if q_norm is not None else 0
+        params = [num_q_heads, num_kv_heads, qk_norm, rotary_embed, self.max_seq_length, self.page_size, q_workspace.dim(1)]
+        self._task("kv_cache_update_mi300", grid_dim, block_dim,
+                   [(input, (-1, 1, -1), -1), (k_cache, (-1, 2, -1), 1), (v_cache, (-1, 2, -1), 1), (q_norm, _REPL, -1), (k_norm, _REPL, -1),
+                    (cos_pos_embed, _REPL, -1), (sin_pos_embed, _REPL, -1), (q_workspace, (-1, 1, -1), -1)], params)
+
+    def paged_attention_ck_fmha_layer(self, q_workspace: DTensor, k_cache: DTensor, v_cache: DTensor, o_acc: DTensor, lse_acc: DTensor,
+                                      attention_params: tuple, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:981.  With num_kv_chunks == 1 `o_acc` is the final bf16 attention output."""
+        assert q_workspace.num_dims == 2
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4
+        assert o_acc.num_dims == 2 and lse_acc.num_dims == 2
+        head_dim = k_cache.dim(3)
+        num_kv_heads = k_cache.dim(2)
+        num_q_heads, num_kv_chunks, num_requests = attention_params[0], attention_params[1], attention_params[2]
+        kv_stride = num_kv_heads * head_dim
+        params = [num_q_heads, num_kv_heads, head_dim, self.page_size, self.max_seq_length, num_kv_chunks, q_workspace.dim(1), kv_stride, num_requests]
+        self._task("paged_attention_ck_fmha_split_kv_mi300", grid_dim, block_dim,
+                   [(q_workspace, _REPL, -1), (k_cache, (-1, 2, -1), 1), (v_cache, (-1, 2, -1), 1), (o_acc, _REPL, -1), (lse_acc, _REPL, -1)], params)
+
+    def gang_paged_attention_split_kv_layer(self, input: DTensor, k_cache: DTensor, v_cache: DTensor, q_norm: DTensor, k_norm: DTensor,
+                                            cos_pos_embed: DTensor, sin_pos_embed: DTensor, lse: DTensor, output: DTensor, q_workspace: DTensor,
+                                            attention_params: tuple, block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1064: KV append + q/k-norm + RoPE + attention in one task."""
+        assert input.num_dims == 2
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4
+        num_kv_heads = k_cache.dim(2)
+        num_q_heads, num_kv_chunks, q_workspace_stride = attention_params[0], attention_params[1], attention_params[2]
+        rotary_embed = 0
+        if cos_pos_embed is not None or sin_pos_embed is not None:
+            assert cos_pos_embed.num_dims == 2 and sin_pos_embed.num_dims == 2
+            rotary_embed = 1
+        qk_norm = 0
+        if q_norm is not None or k_norm is not None:
+            assert q_norm.num_dims == 1 and k_norm.num_dims == 1
+            qk_norm = 1
+        total = self.max_num_batched_requests * num_kv_heads * num_kv_chunks
+        params = [num_q_heads, num_kv_heads, qk_norm, rotary_embed, self.max_seq_length, self.page_size, num_kv_chunks,
+                  math.ceil(total / 8), total, q_workspace_stride]
+        self._task("gang_attn_split_kv_mi300", (8, 1, 1), block_dim,
+                   [(input, _REPL, 1), (k_cache, _REPL, 1), (v_cache, _REPL, 1), (q_norm, _REPL, -1), (k_norm, _REPL, -1), (cos_pos_embed, _REPL, -1),
+                    (sin_pos_embed, _REPL, -1), (lse, _REPL, -1), (output, _REPL, -1), (q_workspace, _REPL, -1)], params)
+
+    def argmax_partial_layer(self, input: DTensor, output: tuple, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2207."""
+        assert input.num_dims == 2
+        assert len(output) == 2
+        output_value, output_index = output
+        assert output_value.num_dims == 2 and output_index.num_dims == 2
+        num_tasks = grid_dim[0]
+        self.argmax_partial_output_size = input.dim(1) // num_tasks
+        self._task("argmax_partial", grid_dim, block_dim,
+                   [(input, (1, 0, -1), -1), (output_value, (1, 0, -1), -1), (output_index, (1, 0, -1), -1)], [num_tasks])
+
+    def argmax_reduce_layer(self, input: tuple, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2232."""
+        assert len(input) == 2
+        input_value, input_index = input
+        assert input_value.num_dims == 2 and input_index.num_dims == 2
+        assert output.num_dims == 2
+        self._task("argmax_reduce", grid_dim, block_dim,
+                   [(input_value, (1, 0, -1), -1), (input_index, (1, 0, -1), -1), (output, (0, 1, -1), -1)],
+                   [getattr(self, "argmax_partial_output_size", 0)])
+
+    # layers of the reference that are outside the one-GPU dense decode path
+    def allreduce_layer(self, *args, **kwargs):
+        raise NotImplementedError("allreduce_layer: the MI355X megakernel runs on one GPU")
+
+    def draft_forward_layer_dispatcher(self, *args, **kwargs):
+        raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
+
+    def verify_layer_dispatcher(self, *args, **kwargs):
+        raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
+
+    def paged_attention_ck_fmha_merge_layer(self, *args, **kwargs):
+        raise NotImplementedError("split-KV merge layers are not needed: the attention stage splits and merges KV chunks internally; "
+                                  "build the attention layer with num_kv_chunks=1")
+
+    gang_paged_attention_split_kv_merge_layer = paged_attention_ck_fmha_merge_layer
+
+    # ------------------------------------------------------------------ compile / run
+    def describe_program(self) -> str:
+        out = ctypes.c_char_p()
+        _capi.check(self._lib.mk_describe_program(self._handle, ctypes.byref(out)))
+        return out.value.decode()
+
+    def compile(self, **kwargs):
+        """persistent_kernel.py:2404.  Lowers the recorded tasks and uploads descriptors; nothing is compiled at run time."""
+        assert not self._is_compiled
+        output_dir = kwargs.get("output_dir", None)
+        _capi.check(self._lib.mk_compile(self._handle))
+        self._is_compiled = True
+        if output_dir is not None:
+            import os
+            os.makedirs(output_dir, exist_ok=True)
+            res = self.kn_graph.generate_task_graph(1, 0)
+            with open(os.path.join(output_dir, "task_graph.json"), "w") as f:
+                f.write(res["json_file"])
+            with open(os.path.join(output_dir, "stage_program.txt"), "w") as f:
+                f.write(self.describe_program())
+
+    @staticmethod
+    def _stream_ptr(stream):
+        if stream is None:
+            stream = torch.cuda.current_stream()
+        if hasattr(stream, "cuda_stream"):
+            return int(stream.cuda_stream)
+        if isinstance(stream, int):
+            return stream
+        raise ValueError("Invalid stream object")
+
+    def __call__(self, **kwargs):
+        """persistent_kernel.py:2622: run every request to completion in one persistent launch (blocking)."""
+        assert self._is_compiled, "call compile() first"
+        sp = self._stream_ptr(kwargs.get("default_stream", None))
+        _capi.check(self._lib.mk_launch(self._handle, ctypes.c_void_p(sp)))
+
+    def init_request_resources(self):
+        """Reset step[], batch slots and the page ring (reference: init_request_func, persistent_kernel.py:63-68)."""
+        _capi.check(self._lib.mk_init_requests(self._handle))
+
+    def run_steps(self, max_iterations: int, default_stream=None) -> bool:
+        """Run at most `max_iterations` decode iterations; returns True when all requests have finished."""
+        fin = ctypes.c_int(0)
+        sp = self._stream_ptr(default_stream)
+        _capi.check(self._lib.mk_launch_steps(self._handle, ctypes.c_void_p(sp), int(max_iterations), ctypes.byref(fin)))
+        return bool(fin.value)
+
+    def enqueue_steps(self, max_iterations: int, default_stream=None):
+        _capi.check(self._lib.mk_enqueue_steps(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), int(max_iterations)))
+
+    def wait(self, default_stream=None) -> bool:
+        fin = ctypes.c_int(0)
+        _capi.check(self._lib.mk_wait(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), ctypes.byref(fin)))
+        return bool(fin.value)
+
+    def run_once(self, tok_slot, tok_pos, tok_first=None, default_stream=None):
+        """Host-driven single pass over the stage program (onepass mode): row t belongs to batch slot tok_slot[t] at
+        absolute position tok_pos[t]; paged_kv_indptr/indices must already describe each slot's pages."""
+        n = len(tok_slot)
+        if tok_first is None:
+            tok_first, first = [], {}
+            for t in range(n):
+                if t > 0 and tok_slot[t] == tok_slot[t - 1]:
+                    tok_first.append(tok_first[-1])
+                else:
+                    tok_first.append(t)
+        i32 = ctypes.c_int32
+        _capi.check(self._lib.mk_run_once(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), n,
+                                          _capi.int_array(tok_slot, i32), _capi.int_array(tok_pos, i32), _capi.int_array(tok_first, i32)))
+
+    def stats(self) -> dict:
+        st = _capi.MkStats()
+        _capi.check(self._lib.mk_get_stats(self._handle, ctypes.byref(st)))
+        return {name: getattr(st, name) for name, _ in st._fields_}
+
+    def finalize(self):
+        assert not self.__finalized__
+        if self._handle is not None:
+            self._lib.mk_graph_destroy(self._handle)
+            self._handle = None
+        self.__finalized__ = True
+
+    def __del__(self):
+        try:
+            if not self.__finalized__:
+                self.finalize()
+        except Exception:
+            pass
+
+
+class _DevicePtr:
+    """Minimal __cuda_array_interface__ holder so torch can view library-owned device memory without copying."""
+
+    def __init__(self, ptr, nbytes, shape, dt, device, strides=None):
+        typestr = {"bfloat16": "<u2", "float16": "<f2", "float32": "<f4", "int32": "<i4", "int64": "<i8", "uint64": "<u8"}[dt.name]
+        self._dt = dt
+        iface = {"shape": tuple(shape), "typestr": typestr, "data": (int(ptr), False), "version": 2}
+        if strides is not None:
+            iface["strides"] = tuple(int(s) * dt.size for s in strides)
+        self.__cuda_array_interface__ = iface

@@ -1,0 +1,156 @@
+/* C ABI of the MI355X persistent decode megakernel library (libfleet_mk.so).
+ *
+ * This is the drop-in boundary for the decode path of mirage's PersistentKernel:
+ * the Python front end (fleet-chiplet-megakernel_amd/mirage) binds these entry
+ * points with ctypes where the reference binds its C++ graph through Cython
+ * (python/mirage/_cython/core.pyx, CCore.pxd:236-253) and its generated launcher
+ * through a CPython module (python/mirage/mpk/persistent_kernel.py:17-130).
+ *
+ * Conventions: plain pointers and sizes only; every function returns 0 on success
+ * or a negative MK_E* code, and mk_last_error() then returns a description (thread
+ * local).  Tensor ids are small non-negative ints scoped to one graph handle.
+ * Device pointers passed in stay owned by the caller and must outlive the handle;
+ * tensors created with mk_tensor_new are owned (and freed) by the library.
+ */
+#ifndef FLEET_MK_H
+#define FLEET_MK_H
+#include <stdint.h>
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef struct mk_graph mk_graph;
+
+enum mk_status {
+  MK_OK = 0,
+  MK_EINVAL = -1,   /* bad argument / shape / unsupported configuration */
+  MK_EHIP = -2,     /* a HIP runtime call failed */
+  MK_ESTATE = -3,   /* call out of order (e.g. launch before compile) */
+  MK_EABORT = -4,   /* the kernel hit its bounded-spin watchdog and exited early */
+  MK_EUNSUPPORTED = -5
+};
+
+/* dtype codes: the reference's type::DataType values used by the decode path
+ * (include/mirage/type.h:58-73): */
+enum mk_dtype {
+  MK_DT_F16 = 940,
+  MK_DT_BF16 = 941,
+  MK_DT_F32 = 950,
+  MK_DT_I32 = 955,
+  MK_DT_I64 = 965,
+  MK_DT_U64 = 966
+};
+
+enum mk_io_category { MK_IO_DEVICE = 0 /* "cuda_tensor" */, MK_IO_SYMMETRIC = 1 /* "nvshmem_tensor": single GPU => same */ };
+
+/* Constructor arguments of PersistentKernel (persistent_kernel.py:368-387) plus the
+ * ten meta tensors in the order the reference hands them to init_func
+ * (persistent_kernel.py:2590-2600).  All meta pointers are device pointers. */
+typedef struct mk_config {
+  int num_workers;              /* workgroups of the persistent grid; 0 = one per CU */
+  int max_seq_length;
+  int max_num_batched_requests;
+  int max_num_batched_tokens;
+  int max_num_pages;
+  int page_size;
+  int total_num_requests;       /* rows of `tokens` */
+  int device;                   /* HIP device ordinal */
+  int64_t eos_token_id;
+  float rms_eps;                /* 0 => 1e-6, the constant baked into the reference kernels */
+  int reserved0;
+  int32_t *step;                /* [total_num_requests] */
+  int64_t *tokens;              /* [total_num_requests, max_seq_length] */
+  int64_t *input_tokens;        /* [max_num_batched_tokens] */
+  int64_t *output_tokens;       /* [max_num_batched_tokens] */
+  int32_t *num_new_tokens;      /* [total_num_requests] */
+  int32_t *prompt_lengths;      /* [total_num_requests] */
+  int32_t *qo_indptr;           /* [max_num_batched_requests + 1] */
+  int32_t *paged_kv_indptr;     /* [max_num_batched_requests + 1] */
+  int32_t *paged_kv_indices;    /* [max_num_pages] */
+  int32_t *paged_kv_last_page_len; /* [max_num_batched_requests] */
+} mk_config;
+
+/* Replaces CyKNGraph(disable_fingerprint=True) + the PersistentKernel ctor
+ * (persistent_kernel.py:404; src/kernel/graph.cc Graph::Graph). */
+int mk_graph_create(const mk_config *cfg, mk_graph **out);
+/* Replaces finalize_persistent_kernel (persistent_kernel.cuh:2331) and frees library-owned tensors. */
+int mk_graph_destroy(mk_graph *g);
+
+/* Replaces KNGraph.new_input + attach_torch_tensor (python/mirage/_cython/core.pyx:718,944;
+ * src/kernel/graph.cc:338-344).  Row-major only, like the reference (persistent_kernel.py:473-474).
+ * Returns the tensor id (>= 0) or a negative status. */
+int mk_tensor_attach(mk_graph *g, void *device_ptr, int ndims, const int64_t *dims, const int64_t *strides, int dtype,
+                     const char *name);
+/* Replaces new_input + attach_cuda_tensor / attach_nvshmem_tensor (core.pyx:951-965): the library allocates
+ * (zero-filled) device memory at mk_compile. */
+int mk_tensor_new(mk_graph *g, int ndims, const int64_t *dims, const int64_t *strides, int dtype, const char *name,
+                  int io_category);
+/* Replaces Graph::shuffle_tensors / fuse_tensors (src/kernel/graph.cc:398-437).  The result is a *view*:
+ * row r of the shuffled tensor is resolved to its source at run time; no interleaved copy is made.
+ * interleave != 0: groups of [src0 rows ; src1 rows ; ...] (shuffle_tensors); 0: plain concatenation (fuse_tensors
+ * with one group). */
+int mk_tensor_shuffle(mk_graph *g, const int *ids, int n, int dim, int num_groups, int interleave, const char *name);
+/* DTensor.num_dims / DTensor.dim(i) (core.pyx:431-482). */
+int mk_tensor_num_dims(mk_graph *g, int id);
+int64_t mk_tensor_dim(mk_graph *g, int id, int i);
+/* Device address of a tensor after mk_compile (library-owned tensors included); NULL for shuffled views. */
+void *mk_tensor_ptr(mk_graph *g, int id);
+
+/* Replaces TBGraph.new_input per operand + KNGraph.customized + Graph::register_task(name, params)
+ * (core.pyx:1023-1059,817,1011; src/kernel/graph.cc:439-848).  Operands are given inputs first, outputs last,
+ * in the order the reference layer builders use; `input_maps` holds 3 ints per operand, `forloop_dims` one. */
+int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const int block_dim[3], int n_operands,
+                const int *tensor_ids, const int *input_maps, const int *forloop_dims, int n_params, const int *params);
+
+/* Replaces Graph::generate_task_graph (src/kernel/runtime.cc:1652-1685): returns the task/event graph as JSON in
+ * the reference's task_graph.json schema (runtime.cc:948-1437).  The string is owned by the handle and stays valid
+ * until the next call or mk_graph_destroy.  The persistent kernel is precompiled, so there is no generated source. */
+int mk_generate_task_graph(mk_graph *g, int num_gpus, int my_gpu_id, const char **json_out);
+
+/* Replaces PersistentKernel.compile's hipcc step + init_persistent_kernel (persistent_kernel.py:2404-2618;
+ * persistent_kernel.cuh:1966-2256): lowers the recorded tasks to the stage program, allocates library-owned
+ * tensors and runtime state, uploads descriptors, and resets the request scheduler. */
+int mk_compile(mk_graph *g);
+/* Replaces init_request_resources (persistent_kernel.cuh:1960): resets step[], the page ring and batch slots so the
+ * same handle can serve `tokens` again. */
+int mk_init_requests(mk_graph *g);
+/* Replaces launch_persistent_kernel (persistent_kernel.cuh:2260-2329): one cooperative launch that runs until all
+ * requests are finished.  Blocks until the kernel has drained, like the reference. `stream` is a hipStream_t (may be 0). */
+int mk_launch(mk_graph *g, void *stream);
+/* Same kernel, but returns after at most `max_iterations` decode iterations; scheduler state persists in HBM so the
+ * next call continues where this one stopped (the reference has no counterpart: its TPOT is an average over one whole
+ * launch, demo/qwen3/demo.py:1303-1328).  *finished_out (optional) is set to 1 when no request is left. */
+int mk_launch_steps(mk_graph *g, void *stream, int max_iterations, int *finished_out);
+/* Non-blocking variant of mk_launch_steps used for timing with events on the caller's stream: enqueues the
+ * launch and returns; mk_wait() synchronises and reports watchdog aborts. */
+int mk_enqueue_steps(mk_graph *g, void *stream, int max_iterations);
+int mk_wait(mk_graph *g, void *stream, int *finished_out);
+/* Host-driven single pass (the reference's MODE_ONEPASS / online modes, persistent_kernel.cuh:538-582): the caller
+ * supplies the batch -- for each of `num_tokens` rows its batch slot, absolute position and the index of the first
+ * row of the same request -- and has filled input_tokens / paged_kv_* itself.  Runs the stage program once. */
+int mk_run_once(mk_graph *g, void *stream, int num_tokens, const int32_t *tok_slot, const int32_t *tok_pos,
+                const int32_t *tok_first);
+
+/* Introspection. */
+typedef struct mk_stats {
+  int num_workgroups;      /* persistent grid size */
+  int num_stages;          /* stages of the lowered program */
+  int num_tasks;           /* reference-style tasks in the task graph */
+  int num_events;
+  int num_xcds;            /* dies that received workgroups in the last launch */
+  int aborted;             /* watchdog fired in the last launch */
+  int64_t iterations;      /* decode iterations executed since mk_init_requests */
+  int64_t weight_bytes;    /* bytes of weight matrices streamed by one iteration */
+  double last_launch_ms;   /* HIP-event time of the last launch's kernel, on the stream it ran on */
+} mk_stats;
+int mk_get_stats(mk_graph *g, mk_stats *out);
+/* Stage listing (one line per stage) for debugging and tests; owned by the handle. */
+int mk_describe_program(mk_graph *g, const char **text_out);
+
+const char *mk_last_error(void);
+const char *mk_version(void);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -1,0 +1,58 @@
+"""BASELINE config 1: RMSNorm(4096) -> linear 4096x4096, BS=1 bf16, as a two-task graph through the C ABI.
+
+Closest reference checks (CUDA-only, formula only): tests/runtime_python/test_norm_linear.py:13-19."""
+import pytest
+import torch
+
+from helpers import bf16_ulp_diff, make_meta, make_mpk
+
+pytestmark = pytest.mark.gpu
+
+
+def _inputs(H, N, seed=0):
+    g = torch.Generator().manual_seed(seed)
+    x = torch.randn(1, H, generator=g).to(torch.bfloat16)
+    nw = (1.0 + 0.02 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    W = (0.02 * torch.randn(N, H, generator=g)).to(torch.bfloat16)
+    return x, nw, W
+
+
+@pytest.mark.parametrize("gang", [False, True])
+@pytest.mark.parametrize("H,N", [(4096, 4096), (1024, 3000), (12288, 512)])
+def test_norm_linear_bs1(gang, H, N):
+    import mirage as mi
+    from oracle.qwen3_ref import linear_k, rmsnorm_k
+    if gang and (N % 8 or (N // 8) % 64):
+        pytest.skip("gang layers need N divisible by 8*tile_n")
+    x, nw, W = _inputs(H, N)
+    meta = make_meta(1, 64, 1, 1, 1)
+    mpk = make_mpk(meta, 64, 1, 1, 1, 64, mode="onepass")
+    xd, nwd, Wd = x.cuda(), nw.cuda(), W.cuda()
+    tx = mpk.attach_input(xd, "x")
+    tnw = mpk.attach_input(nwd, "norm_w")
+    tW = mpk.attach_input(Wd, "W")
+    tn = mpk.new_tensor((1, H), dtype=mi.bfloat16, name="norm_out")
+    ty = mpk.new_tensor((1, N), dtype=mi.bfloat16, name="y")
+    if gang:
+        mpk.gang_rmsnorm_layer(input=tx, weight=tnw, output=tn)
+        mpk.gang_linear_layer(input=tn, weight=tW, output=ty, tile_n=64, output_stride=N)
+    else:
+        mpk.rmsnorm_layer(input=tx, weight=tnw, output=tn, grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
+        mpk.linear_layer(input=tn, weight=tW, output=ty, grid_dim=(N // 8 if N % 8 == 0 else 1, 1, 1), block_dim=(128, 1, 1))
+    mpk.compile()
+    mpk.run_once([0], [0])
+    y = ty.to_torch().cpu()
+    n_gpu = tn.to_torch().cpu()
+    n_ref = rmsnorm_k(x, nw)
+    y_ref = linear_k(n_ref, W)
+    # the fused norm output must be bit-exact up to rsqrt rounding: allow 1 bf16 ulp
+    ulp_n, _ = bf16_ulp_diff(n_gpu, n_ref)
+    assert ulp_n <= 1.0, f"norm differs by {ulp_n} bf16 ulp"
+    # fp32 accumulation order differs from torch's matmul: allow 1 bf16 ulp of the row scale + small abs
+    torch.testing.assert_close(y.float(), y_ref.float(), atol=2e-2, rtol=1e-2)  # north-star tolerance
+    d = (y.float() - y_ref.float()).abs()
+    assert float(d.max()) <= 0.016, f"max abs diff {float(d.max())}"
+    assert float((d > 0).float().mean()) < 0.05, "more than 5% of outputs differ from the fp32-accumulate oracle"
+    st = mpk.stats()
+    assert st["num_xcds"] == 8 and st["aborted"] == 0
+    mpk.finalize()
