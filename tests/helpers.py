@@ -32,10 +32,11 @@ def make_mpk(meta, max_seq, max_tokens, max_requests, max_pages, page_size, mode
         trace_name=None, spec_decode_config=None, use_cutlass_kernel=False)
 
 
-def bf16_ulp_diff(a, b):
-    """Max difference in units of bf16 ulp of the larger magnitude, plus max abs diff."""
+def bf16_ulp_diff(a, b, floor=1e-30):
+    """Max difference in units of bf16 ulp of the larger magnitude (magnitudes below `floor` count as `floor`, so
+    cancellation near zero is measured against the scale of the operands), plus max abs diff."""
     af, bf = a.float().cpu(), b.float().cpu()
     d = (af - bf).abs()
-    scale = torch.maximum(af.abs(), bf.abs()).clamp_min(1e-30)
+    scale = torch.maximum(af.abs(), bf.abs()).clamp_min(floor)
     ulp = torch.exp2(torch.floor(torch.log2(scale)) - 7)
     return float((d / ulp).max()), float(d.max())
