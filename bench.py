@@ -1,0 +1,158 @@
+"""Headline benchmark: decode TPOT (ms/token) of the 36-layer Qwen3-8B-shaped random-init bf16 model on one MI355X.
+
+A "step" is one decode iteration of the persistent megakernel for the whole batch.  The prompt (80 seeded random ids
+per request) is ingested and W warm-up decode steps run untimed; then EXACTLY K decode steps run inside ONE persistent
+launch, bracketed by torch.cuda.synchronize() on both sides.  Weights, KV cache and meta tensors are resident in HBM
+before the timed region.  Prints one JSON line (see README of the driver contract).
+
+roofline: the dominant (only) kernel is mk_persistent_kernel; its algorithmic bytes per launch are
+K x (all bf16 weight matrices once + the K/V rows of every cached position of every request), divided by the launch
+duration measured with HIP events on the launch stream, against the 8 TB/s HBM peak.
+cpu_baseline: the CPU oracle's torch-order decode (the reference's PyTorch path restated) timed on the host cores on a
+bounded sample (a few layers + LM head for a few steps), extrapolated to 36 layers; a reported baseline, not a target.
+"""
+import argparse
+import json
+import math
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+sys.path.insert(0, os.path.join(ROOT, "fleet-chiplet-megakernel_amd"))
+sys.path.insert(0, ROOT)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def cpu_baseline(shape, n_layers_sample=2, steps=3, context=80):
+    """Time the oracle (reference's torch decode restated) on the host: `n_layers_sample` full-width layers + LM head."""
+    import torch
+    from oracle.qwen3_ref import KVCache, Qwen3Config, Qwen3Oracle, make_layer_weights
+    cores = os.cpu_count() or 1
+    cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
+    torch.set_num_threads(cores)
+    cfg = Qwen3Config(hidden_size=shape.hidden_size, num_q_heads=shape.num_q_heads, num_kv_heads=shape.num_kv_heads, head_dim=shape.head_dim,
+                      intermediate_size=shape.intermediate_size, num_layers=n_layers_sample, vocab_size=shape.vocab_size, rope_theta=shape.rope_theta)
+    g = torch.Generator().manual_seed(0)
+    w = {"layers": [make_layer_weights(cfg, g) for _ in range(n_layers_sample)]}
+    w["embed"] = torch.zeros(8, cfg.hidden_size, dtype=torch.bfloat16)
+    w["embed"][:] = torch.randn(8, cfg.hidden_size, generator=g).to(torch.bfloat16) * 0.02
+    w["final_norm"] = torch.ones(cfg.hidden_size, dtype=torch.bfloat16)
+    # LM head: reuse one 4096-row random block 37x + remainder to bound the generation time; timing only depends on shape
+    blk = (torch.randn(4096, cfg.hidden_size, generator=g) * 0.02).to(torch.bfloat16)
+    reps = math.ceil(cfg.vocab_size / 4096)
+    w["lm_head"] = blk.repeat(reps, 1)[:cfg.vocab_size].contiguous()
+    orc = Qwen3Oracle(cfg, w, "torch")
+    cache = KVCache(cfg, context + steps + 2)
+    cache.k.normal_(0, 1, generator=g)
+    cache.v.normal_(0, 1, generator=g)
+    ids = torch.tensor([1])
+
+    def layers_only(pos):
+        x = w["embed"][ids]
+        for li in range(cfg.num_layers):
+            x = orc.layer(li, x, cache, pos)
+        return x
+
+    def head_only(x):
+        from oracle.qwen3_ref import rmsnorm_t
+        import torch.nn.functional as F
+        return F.linear(rmsnorm_t(x, w["final_norm"]), w["lm_head"]).argmax(-1)
+
+    x = layers_only(context)  # warm-up
+    head_only(x)
+    t_layers, t_head = [], []
+    for s in range(steps):
+        t0 = time.perf_counter()
+        x = layers_only(context + s)
+        t1 = time.perf_counter()
+        head_only(x)
+        t2 = time.perf_counter()
+        t_layers.append((t1 - t0) / n_layers_sample)
+        t_head.append(t2 - t1)
+    per_layer = sorted(t_layers)[len(t_layers) // 2]
+    head = sorted(t_head)[len(t_head) // 2]
+    ms = (per_layer * shape.num_layers + head) * 1e3
+    return {"value": round(ms, 2), "unit": "ms/token", "cores": cores, "kind": "port",
+            "sample": f"BS=1, context {context}: {n_layers_sample} of {shape.num_layers} full-width layers + LM head, median of {steps} steps, "
+                      f"extrapolated to {shape.num_layers} layers; torch-order bf16 oracle"}
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1024)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=1, help="requests decoded concurrently (BS)")
+    ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--prompt-length", type=int, default=80)
+    ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the decode megakernel on ONE GPU; --gpus must be 1 "
+              "(multi-GPU tensor parallelism is described in DESIGN.md, not built)", file=sys.stderr)
+        sys.exit(2)
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: launched with WORLD_SIZE>1; this benchmark is single-GPU", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from demo_qwen3 import Qwen3Decoder, Qwen3Shape, random_weights
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the megakernel has no CPU path", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    shape = Qwen3Shape(num_layers=args.layers)
+    B, K, W, P = args.batch, args.steps, args.warmup, args.prompt_length
+    max_seq = max(1200, P + W + K + 2)
+    weights = random_weights(shape, seed=0)
+    dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
+    prompts = [torch.randint(0, shape.vocab_size, (P,), generator=torch.Generator().manual_seed(r)) for r in range(B)]
+    dec.load_prompts(prompts)
+    # prompt ingestion: run until every request has consumed its prompt (first decode token produced), then warm up
+    prefill_iters = 0
+    while True:
+        dec.mpk.run_steps(1)
+        prefill_iters += 1
+        if int(dec.meta["step"].min().item()) >= P:
+            break
+        assert prefill_iters < 10 * P * B, "prompt ingestion did not finish"
+    if W > 0:
+        dec.mpk.run_steps(W)
+    ctx0 = int(dec.meta["step"].min().item())  # cached positions per request at the first timed step
+    stream = torch.cuda.current_stream()
+    torch.cuda.synchronize()
+    t0 = time.perf_counter()
+    dec.mpk.enqueue_steps(K, default_stream=stream)
+    finished = dec.mpk.wait(default_stream=stream)
+    torch.cuda.synchronize()
+    t1 = time.perf_counter()
+    st = dec.mpk.stats()
+    assert not finished, "requests finished inside the timed region; lower --steps"
+    assert int(dec.meta["step"].min().item()) == ctx0 + K, "timed region did not run exactly K decode steps"
+    wall_ms = (t1 - t0) * 1e3
+    kernel_ms = st["last_launch_ms"]
+    ms_per_step = wall_ms / K
+    # algorithmic bytes: weights once per step + K/V rows of every cached position (positions ctx0+1 .. ctx0+K incl. the new one)
+    kv_positions = sum(ctx0 + 1 + i for i in range(K))
+    bytes_total = K * shape.weight_bytes_per_token() + B * kv_positions * shape.kv_bytes_per_position()
+    achieved = bytes_total / (kernel_ms * 1e-3) / 1e9
+    out = {
+        "metric": "decode TPOT ms/token Qwen3-8B-shape bf16", "value": round(ms_per_step, 4), "unit": "ms/token", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (random-init weights ~N(0,0.02), seeded random prompts)",
+        "config": {"workload": f"Qwen3-8B shape, {shape.num_layers} layers, vocab {shape.vocab_size}, BS={B}, prompt {P}, "
+                               f"context {ctx0}..{ctx0 + K}, max_seq_len {max_seq}, page_size 4096, graph mode {args.mode}",
+                   "batch": B, "tokens_per_s": round(B * 1e3 / ms_per_step, 1), "prefill_iterations": prefill_iters},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
+                     "traffic": None, "kernel": "mk_persistent_kernel", "kernel_ms_per_launch": round(kernel_ms, 3),
+                     "algorithmic_bytes_per_launch": bytes_total},
+    }
+    if not args.no_cpu_baseline:
+        out["cpu_baseline"] = cpu_baseline(shape)
+    print(json.dumps(out))
+
+
+if __name__ == "__main__":
+    main()
