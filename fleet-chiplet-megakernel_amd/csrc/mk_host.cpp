@@ -967,6 +967,8 @@ int mk_compile(mk_graph *g) {
   if ((rc = dev_alloc(g, &p, sizeof(long long) * (g->timing_cap + 2)))) return rc;
   rt.timing = g->d_timing = (long long *)p;
   rt.timing_cap = g->timing_cap;
+  if ((rc = dev_alloc(g, &p, sizeof(long long) * 4 * (g->stages.size() + 1) * g->G))) return rc;
+  rt.stage_prof = (long long *)p;
   if ((rc = dev_alloc(g, &p, sizeof(MkRuntime)))) return rc;
   g->d_rt = (MkRuntime *)p;
   if ((rc = upload_runtime(g))) return rc;
@@ -1067,6 +1069,16 @@ int mk_get_stats(mk_graph *g, mk_stats *out) {
     out->iterations = sc.iterations;
   }
   return MK_OK;
+}
+
+int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages) {
+  if (!g || !ticks_out) return fail(MK_EINVAL, "null argument");
+  if (!g->compiled || g->launch_pending) return fail(MK_ESTATE, "no finished launch to report");
+  if (workgroup < 0 || workgroup >= g->G) return fail(MK_EINVAL, "workgroup %d outside [0, %d)", workgroup, g->G);
+  const int n = std::min<int>(max_stages, (int)g->stages.size());
+  if (n > 0)
+    HIP_TRY(hipMemcpy(ticks_out, g->h_rt.stage_prof + (size_t)4 * workgroup * g->stages.size(), sizeof(int64_t) * 4 * n, hipMemcpyDeviceToHost));
+  return n;
 }
 
 int mk_describe_program(mk_graph *g, const char **text_out) {

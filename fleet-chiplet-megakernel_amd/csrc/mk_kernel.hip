@@ -24,6 +24,11 @@ struct Ctx {
   int quota; // workgroups on this XCD
   int nxcd;  // XCDs that received at least one workgroup
   unsigned epoch;
+  bool pending;  // an arrive has been posted that no wait has consumed yet
+  bool leader;   // (thread 0 only) this workgroup was the last of its XCD to arrive
+  bool dead;     // the watchdog fired somewhere: unwind
+  long long t_wait;  // (profiling) tick at which the last barrier_wait completed
+  int *sh_dead;
   MkSync *sync;
 };
 
@@ -62,6 +67,29 @@ __device__ __forceinline__ unsigned xcc_id() {
 }
 __device__ __forceinline__ u32x4 ldg_stream(const u32x4 *p) { return __builtin_nontemporal_load(p); }
 
+// Loads of data another workgroup produced earlier in this launch.  The per-XCD L2s are write-back and
+// not coherent with each other, and the CU's vector L1 is not coherent with anything: producers write back
+// their L2 at the barrier (release by the XCD's last arriver), consumers read with device-scope loads
+// (sc1: miss the L1, coherent in L2), so no cache invalidate is ever issued.
+__device__ __forceinline__ uint32_t ldc_u32(const void *p) {
+  return __hip_atomic_load((const uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ int ldc_i32(const int *p) { return (int)ldc_u32(p); }
+__device__ __forceinline__ float ldc_f32(const float *p) { return __uint_as_float(ldc_u32(p)); }
+__device__ __forceinline__ unsigned long long ldc_u64(const void *p) {
+  return __hip_atomic_load((const unsigned long long *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ u32x4 ldc_16B(const u32x4 *p) {
+  const unsigned long long a = ldc_u64(p), b = ldc_u64((const unsigned long long *)p + 1);
+  u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
+  return r;
+}
+__device__ __forceinline__ uint16_t ldc_u16(const uint16_t *p) {
+  const uintptr_t a = (uintptr_t)p;
+  const uint32_t w = ldc_u32((const void *)(a & ~(uintptr_t)3));
+  return (uint16_t)((a & 2) ? (w >> 16) : (w & 0xffffu));
+}
+
 // ----------------------------------------------------------------------------- grid barrier
 // Two-level barrier: workgroups of one XCD count arrivals in a counter that lives in that XCD's
 // L2; the last arriver of each XCD publishes one cross-XCD signal and waits for the other dies,
@@ -80,38 +108,58 @@ __device__ __forceinline__ bool spin_ok(MkSync *s, unsigned &spins, unsigned whe
   return true;
 }
 
-__device__ __forceinline__ bool grid_barrier(Ctx &c, int *sh_dead) {
+// arrive: this workgroup's outputs of the current stage are complete.  The last arriver of an XCD becomes
+// that XCD's leader for this epoch: it writes the die's L2 back (release) and posts the cross-XCD signal.
+__device__ __forceinline__ void barrier_arrive(Ctx &c) {
   MkSync *s = c.sync;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   c.epoch++;
   if (threadIdx.x == 0) {
-    const unsigned epoch = c.epoch;
-    unsigned spins = 0;
-    unsigned old = __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    if (old + 1 == (unsigned)c.quota * epoch) {
-      __hip_atomic_fetch_add(&s->global_ctr, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-      while (__hip_atomic_load(&s->global_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)c.nxcd * epoch &&
-             spin_ok(s, spins, epoch))
-        __builtin_amdgcn_s_sleep(1);
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      __hip_atomic_fetch_max(&s->local_flag[c.xcd][0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    } else {
-      // poll with a compare-and-swap that never succeeds: it executes in the L2 (never served by
-      // the CU's vector L1) and cannot be folded into a plain load by the compiler
-      while (true) {
-        unsigned expect = 0xFFFFFFFFu;
-        __hip_atomic_compare_exchange_strong(&s->local_flag[c.xcd][0], &expect, 0xFFFFFFFFu, __ATOMIC_RELAXED,
-                                             __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-        if (expect >= epoch || !spin_ok(s, spins, epoch)) break;
-        __builtin_amdgcn_s_sleep(1);
-      }
-      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    }
-    *sh_dead = (spins >= 1024u) ? (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+    const unsigned old = __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    c.leader = (old + 1 == (unsigned)c.quota * c.epoch);
+    if (c.leader) __hip_atomic_fetch_add(&s->global_ctr, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
   }
+  c.pending = true;
+}
+
+// wait: every workgroup of the grid has arrived at the current epoch.  Leaders poll the global counter and then
+// raise their die's flag; everyone else polls that flag with a compare-and-swap that never succeeds (it executes in
+// the L2, is never served from the CU's L1, and cannot be folded into a plain load by the compiler).
+__device__ __forceinline__ void barrier_poll(Ctx &c) {
+  // thread 0 only; the caller must follow with a workgroup barrier and barrier_done()
+  MkSync *s = c.sync;
+  const unsigned epoch = c.epoch;
+  unsigned spins = 0;
+  if (c.leader) {
+    while (__hip_atomic_load(&s->global_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)c.nxcd * epoch &&
+           spin_ok(s, spins, epoch))
+      __builtin_amdgcn_s_sleep(1);
+    __hip_atomic_fetch_max(&s->local_flag[c.xcd][0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  } else {
+    while (true) {
+      unsigned expect = 0xFFFFFFFFu;
+      __hip_atomic_compare_exchange_strong(&s->local_flag[c.xcd][0], &expect, 0xFFFFFFFFu, __ATOMIC_RELAXED,
+                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+      if (expect >= epoch || !spin_ok(s, spins, epoch)) break;
+      __builtin_amdgcn_s_sleep(1);
+    }
+  }
+  *c.sh_dead = (spins >= 1024u) ? (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
+}
+
+// bookkeeping after the workgroup barrier that follows barrier_poll
+__device__ __forceinline__ void barrier_done(Ctx &c) {
+  c.pending = false;
+  c.dead = c.dead || (*c.sh_dead != 0);
+  c.t_wait = (long long)wall_clock64();
+}
+
+__device__ __forceinline__ void barrier_wait(Ctx &c) {
+  if (!c.pending) return;
+  if (threadIdx.x == 0) barrier_poll(c);
   __syncthreads();
-  return *sh_dead != 0;
+  barrier_done(c);
 }
 
 // ----------------------------------------------------------------------------- scheduler
@@ -241,16 +289,20 @@ __device__ __forceinline__ const u32x4 *weight_row(const MkWeight &w, int r, int
 }
 
 // ----------------------------------------------------------------------------- stages
+// Every stage function posts barrier_wait(c) itself, after any work that does not depend on the previous
+// stage (weight prefetch), and the main loop posts barrier_arrive(c) when the function returns.
+
 // Gather embedding rows.  Reference task: tasks/ampere/embedding.cuh:42-72.
-__device__ void stage_embed(const MkStage &st, const Ctx &c, const MkRuntime &rt, int M) {
+__device__ void stage_embed(const MkStage &st, Ctx &c, const MkRuntime &rt, int M) {
+  barrier_wait(c);
   const int k8 = st.k / 8;
   for (int t = c.vid; t < M; t += c.G) {
     long long id;
     if (st.flags & MK_F_EMBED_FROM_TOKENS) {
-      const int req = rt.request_ids[rt.tok_slot[t]];
-      id = rt.tokens[(long long)req * rt.max_seq + rt.tok_pos[t]];
+      const int req = ldc_i32(&rt.request_ids[ldc_i32(&rt.tok_slot[t])]);
+      id = (long long)ldc_u64(&rt.tokens[(long long)req * rt.max_seq + ldc_i32(&rt.tok_pos[t])]);
     } else {
-      id = ((const long long *)st.in)[t];
+      id = (long long)ldc_u64((const long long *)st.in + t);
     }
     const u32x4 *src = (const u32x4 *)st.w.seg[0] + (size_t)(id < 0 ? 0 : id) * k8;
     u32x4 *dst = (u32x4 *)st.out + (size_t)t * (st.ld_out / 8);
@@ -271,8 +323,10 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 // RMSNorm of full rows, one workgroup per token row (used when an iteration has several tokens;
 // single-token iterations fuse the norm into the consuming linear).  y = bf16((x * r) * w) with
 // r = rsqrt(mean(x^2) + eps) in fp32.  Reference task: tasks/mi300/rmsnorm_mi300.cuh:37-188.
-__device__ void stage_norm(const MkStage &st, const Ctx &c, int M, char *smem) {
+__device__ void stage_norm(const MkStage &st, Ctx &c, int M, char *smem) {
+  barrier_wait(c);
   float *red = (float *)smem;
+  uint32_t *xs = (uint32_t *)(smem + 1024);
   const int k2 = st.k / 2;
   for (int t = c.vid; t < M; t += c.G) {
     const uint32_t *x = (const uint32_t *)st.in + (size_t)t * (st.ld_in / 2);
@@ -280,54 +334,233 @@ __device__ void stage_norm(const MkStage &st, const Ctx &c, int M, char *smem) {
     uint32_t *y = (uint32_t *)st.out + (size_t)t * (st.ld_out / 2);
     float ss = 0.f;
     for (int i = threadIdx.x; i < k2; i += MK_THREADS) {
-      const uint32_t u = x[i];
+      const uint32_t u = ldc_u32(x + i);
+      xs[i] = u;
       ss += bf_lo(u) * bf_lo(u) + bf_hi(u) * bf_hi(u);
     }
     ss = block_sum(ss, red);
     const float r = rsqrtf(ss / (float)st.k + st.eps);
     for (int i = threadIdx.x; i < k2; i += MK_THREADS) {
-      const uint32_t u = x[i], g = w[i];
+      const uint32_t u = xs[i], g = w[i];
       y[i] = pack2((bf_lo(u) * r) * bf_lo(g), (bf_hi(u) * r) * bf_hi(g));
     }
+    __syncthreads();
   }
 }
 
 __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + __expf(-g)) * u; }
 
-// Single-token linear: out[n] = bf16(sum_k W[n,k] * x[k] (+ res[n])), optionally with the RMSNorm of x
-// fused in front and with the SwiGLU epilogue fused behind.  The weight matrix is streamed from HBM
-// exactly once with 128-bit loads, one 1 KB row segment per wavefront instruction; x lives in LDS as
-// packed bf16 and the products run on v_dot2_f32_bf16 with fp32 accumulation.
-// Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
-// (tasks/mi300/gang_linear_mi300.cuh:359-576).
-__device__ void stage_linear_m1(const MkStage &st, const Ctx &c, char *smem) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
-  const int K = st.k, k2 = K / 2, k8 = K / 8;
-  uint32_t *xs = (uint32_t *)smem;
-  float *red = (float *)(smem + 64 * 1024);
-  const uint32_t *xin = (const uint32_t *)st.in;
+// Stage the single input row of a one-token linear in LDS as packed bf16, applying the fused RMSNorm when the
+// stage asks for it (virtual workgroup 0 also stores the normalised row, which is the norm task's output tensor).
+__device__ __forceinline__ void stage_x_m1(const MkStage &st, const Ctx &c, uint32_t *xs, float *red) {
+  const int tid = threadIdx.x, k4 = st.k / 4;
+  const unsigned long long *xin = (const unsigned long long *)st.in;
+  unsigned long long *xs2 = (unsigned long long *)xs;
   if (st.flags & MK_F_NORM) {
     float ss = 0.f;
-    for (int i = tid; i < k2; i += MK_THREADS) {
-      const uint32_t u = xin[i];
-      xs[i] = u;
-      ss += bf_lo(u) * bf_lo(u) + bf_hi(u) * bf_hi(u);
+    for (int i = tid; i < k4; i += MK_THREADS) {
+      const unsigned long long u = ldc_u64(xin + i);
+      xs2[i] = u;
+      const uint32_t a = (uint32_t)u, b = (uint32_t)(u >> 32);
+      ss += bf_lo(a) * bf_lo(a) + bf_hi(a) * bf_hi(a) + bf_lo(b) * bf_lo(b) + bf_hi(b) * bf_hi(b);
     }
     ss = block_sum(ss, red);
-    const float r = rsqrtf(ss / (float)K + st.eps);
+    const float r = rsqrtf(ss / (float)st.k + st.eps);
     const uint32_t *nw = (const uint32_t *)st.norm_w;
     uint32_t *no = (c.vid == 0) ? (uint32_t *)st.norm_out : nullptr;
-    for (int i = tid; i < k2; i += MK_THREADS) {
+    for (int i = tid; i < st.k / 2; i += MK_THREADS) {
       const uint32_t u = xs[i], g = nw[i];
       const uint32_t y = pack2((bf_lo(u) * r) * bf_lo(g), (bf_hi(u) * r) * bf_hi(g));
       xs[i] = y;
       if (no) no[i] = y;
     }
   } else {
-    for (int i = tid; i < k2; i += MK_THREADS) xs[i] = xin[i];
+    for (int i = tid; i < k4; i += MK_THREADS) xs2[i] = ldc_u64(xin + i);
   }
   __syncthreads();
+}
 
+// Same staging done by ONE wavefront (the control wavefront of a tuned single-token linear): lane l owns the
+// 16-byte segments l, l+64, ... of the row, the sum of squares is a wavefront reduction, no workgroup barrier inside.
+template <int KL>
+__device__ __forceinline__ void stage_x_m1_wave(const MkStage &st, const Ctx &c, uint32_t *xs, int lane) {
+  const u32x4 *xin = (const u32x4 *)st.in;
+  u32x4 *xs4 = (u32x4 *)xs;
+  u32x4 v[KL];
+#pragma unroll
+  for (int kc = 0; kc < KL; kc++) v[kc] = ldc_16B(xin + kc * 64 + lane);
+  if (st.flags & MK_F_NORM) {
+    float ss = 0.f;
+#pragma unroll
+    for (int kc = 0; kc < KL; kc++) {
+#pragma unroll
+      for (int e = 0; e < 4; e++) {
+        const uint32_t u = v[kc][e];
+        ss += bf_lo(u) * bf_lo(u) + bf_hi(u) * bf_hi(u);
+      }
+    }
+    ss = wave_sum(ss);
+    const float r = rsqrtf(ss / (float)(KL * 512) + st.eps);
+    const u32x4 *nw = (const u32x4 *)st.norm_w;
+    u32x4 *no = (c.vid == 0) ? (u32x4 *)st.norm_out : nullptr;
+#pragma unroll
+    for (int kc = 0; kc < KL; kc++) {
+      const u32x4 g = nw[kc * 64 + lane];
+      u32x4 y;
+#pragma unroll
+      for (int e = 0; e < 4; e++) y[e] = pack2((bf_lo(v[kc][e]) * r) * bf_lo(g[e]), (bf_hi(v[kc][e]) * r) * bf_hi(g[e]));
+      xs4[kc * 64 + lane] = y;
+      if (no) no[kc * 64 + lane] = y;
+    }
+  } else {
+#pragma unroll
+    for (int kc = 0; kc < KL; kc++) xs4[kc * 64 + lane] = v[kc];
+  }
+}
+
+// Single-token linear: out[n] = bf16(sum_k W[n,k] * x[k] (+ res[n])), optionally with the RMSNorm of x
+// fused in front and with the SwiGLU epilogue fused behind.  The weight matrix is streamed from HBM
+// exactly once with 128-bit loads, one 1 KB row segment per wavefront instruction; x lives in LDS as
+// packed bf16 and the products run on v_dot2_f32_bf16 with fp32 accumulation.
+//
+// Wavefront roles: wavefront 0 is the control wavefront -- it polls the grid barrier, then loads, normalises and
+// publishes x -- while wavefronts 1..3 stream weight rows.  A wavefront's vector loads return in order, so a
+// wavefront that has weight loads in flight cannot observe the barrier before they land; keeping the poll on a
+// wavefront without weight loads lets the weight prefetch and the barrier overlap.
+// KL = K/512 row segments per lane; per worker wavefront the first NPF rows are prefetched straight into its LDS
+// ring and the next R rows into registers, all BEFORE the previous stage is known to be complete (weights do not
+// depend on it), so the HBM pipe stays busy across the grid barrier; each register slot is refilled once consumed.
+// Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
+// (tasks/mi300/gang_linear_mi300.cuh:359-576).
+template <int KL, int R, bool SILU>
+__device__ void stage_linear_m1_t(const MkStage &st, Ctx &c, char *smem) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  constexpr int K8 = KL * 64;
+  constexpr int NW = MK_WAVES - 1;                         // worker wavefronts
+  constexpr int PF_BYTES = (MK_PF_BYTES / NW) & ~1023;     // LDS ring per worker
+  constexpr int NPF = PF_BYTES / (KL * 1024);              // rows per worker prefetched straight into LDS
+  uint32_t *xs = (uint32_t *)smem;
+  const bool ctrl = wave == 0;
+  const int ww = ctrl ? 0 : wave - 1;
+  char *pf_base = smem + MK_PF_OFFSET + ww * PF_BYTES;
+  const u32x4 *pf = (const u32x4 *)pf_base;
+  const int n_out = SILU ? st.n / 2 : st.n;
+  const int nwaves = c.G * NW;
+  const int rpw = (n_out + nwaves - 1) / nwaves;
+  const int r0 = __builtin_amdgcn_readfirstlane((c.vid * NW + ww) * rpw);
+  const int r1 = min(n_out, r0 + rpw);
+  const int nw = ctrl ? 0 : max(0, r1 - r0) * (SILU ? 2 : 1);  // weight rows this wavefront streams
+  const int half = st.silu_half;
+  auto rowptr = [&](int i) -> const u32x4 * {
+    int vr;
+    if (SILU) {
+      const int o = r0 + (i >> 1);
+      const int g = o / half;
+      vr = g * 2 * half + (o - g * half) + ((i & 1) ? half : 0);
+    } else {
+      vr = r0 + i;
+    }
+    return weight_row(st.w, vr, K8) + lane;
+  };
+  const int npf = min(NPF, nw);
+  u32x4 buf[R][KL];
+  if (!ctrl) {
+    for (int j = 0; j < npf; j++) {
+      const u32x4 *p = rowptr(j);
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++)
+        __builtin_amdgcn_global_load_lds((const void *)(p + kc * 64), (__attribute__((address_space(3))) void *)(pf_base + (j * KL + kc) * 1024), 16, 0, 0);
+    }
+#pragma unroll
+    for (int j = 0; j < R; j++)
+      if (npf + j < nw) {
+        const u32x4 *p = rowptr(npf + j);
+#pragma unroll
+        for (int kc = 0; kc < KL; kc++) buf[j][kc] = ldg_stream(p + kc * 64);
+      }
+  } else {
+    if (c.pending && tid == 0) barrier_poll(c);
+    stage_x_m1_wave<KL>(st, c, xs, lane);
+  }
+  __syncthreads();
+  barrier_done(c);
+  if (ctrl) return;
+  // residual values of this wavefront's rows, one per lane, fetched once up front
+  float resv = 0.f;
+  if ((st.flags & MK_F_RES) && r0 + lane < r1) resv = bf2f(ldc_u16((const uint16_t *)st.res + r0 + lane));
+  const u32x4 *xs4 = (const u32x4 *)xs;
+  u32x4 xr[KL <= 8 ? KL : 1];
+  if (KL <= 8) {
+#pragma unroll
+    for (int kc = 0; kc < (KL <= 8 ? KL : 1); kc++) xr[kc] = xs4[kc * 64 + lane];
+  }
+  uint16_t *out = (uint16_t *)st.out;
+  float gate = 0.f, outv = 0.f;
+  int obase = 0;  // outputs [obase, obase+64) of this wavefront are collected in lanes before being stored
+  auto finish_row = [&](int idx, float a) {
+    a = wave_sum(a);
+    int o;
+    float v;
+    bool have = true;
+    if (SILU) {
+      o = idx >> 1;
+      if ((idx & 1) == 0) {
+        gate = a;
+        have = false;
+      }
+      v = silu_mul(gate, a);
+    } else {
+      o = idx;
+      v = a + __shfl(resv, o & 63, 64);
+    }
+    if (have) {
+      if (o - obase >= 64) {
+        out[r0 + obase + lane] = (uint16_t)f2bf(outv);
+        obase += 64;
+      }
+      if (lane == o - obase) outv = v;
+    }
+  };
+  // LDS ring rows: wait for the direct-to-LDS loads (issued first, so they are the oldest in the queue)
+  if (npf > 0) {
+    if ((st.flags & MK_F_RES) || nw - npf < R) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R * KL) : "memory");  // all but the R*KL youngest (register) loads
+  }
+  for (int i = 0; i < npf; i++) {
+    float a = 0.f;
+#pragma unroll
+    for (int kc = 0; kc < KL; kc++) a = dot8(pf[(i * KL + kc) * 64 + lane], KL <= 8 ? xr[KL <= 8 ? kc : 0] : xs4[kc * 64 + lane], a);
+    finish_row(i, a);
+  }
+  for (int i = npf; i < nw; i += R) {
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      if (i + j < nw) {
+        float a = 0.f;
+#pragma unroll
+        for (int kc = 0; kc < KL; kc++) a = dot8(buf[j][kc], KL <= 8 ? xr[KL <= 8 ? kc : 0] : xs4[kc * 64 + lane], a);
+        if (i + j + R < nw) {
+          const u32x4 *p = rowptr(i + j + R);
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) buf[j][kc] = ldg_stream(p + kc * 64);
+        }
+        finish_row(i + j, a);
+      }
+    }
+  }
+  const int n_o = max(0, r1 - r0);
+  if (obase + lane < n_o) out[r0 + obase + lane] = (uint16_t)f2bf(outv);
+}
+
+// Generic single-token linear for reduction lengths that are not a multiple of 512 or have no tuned
+// instantiation: same arithmetic, no cross-barrier prefetch.
+__device__ void stage_linear_m1_generic(const MkStage &st, Ctx &c, char *smem) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int K = st.k, k8 = K / 8;
+  uint32_t *xs = (uint32_t *)smem;
+  float *red = (float *)(smem + MK_RED_OFFSET);
+  barrier_wait(c);
+  stage_x_m1(st, c, xs, red);
   const bool silu = st.flags & MK_F_SILU;
   const int n_out = silu ? st.n / 2 : st.n;
   const int nwaves = c.G * MK_WAVES;
@@ -337,67 +570,54 @@ __device__ void stage_linear_m1(const MkStage &st, const Ctx &c, char *smem) {
   const u32x4 *xs4 = (const u32x4 *)xs;
   uint16_t *out = (uint16_t *)st.out;
   const uint16_t *res = (const uint16_t *)st.res;
-  if (silu) {
-    const int half = st.silu_half;
-    for (int r = r0; r < r1; r++) {
+  for (int r = r0; r < r1; r++) {
+    float v;
+    if (silu) {
+      const int half = st.silu_half;
       const int vr = (r / half) * 2 * half + (r % half);
       const u32x4 *wg = weight_row(st.w, vr, k8);
       const u32x4 *wu = weight_row(st.w, vr + half, k8);
       float ag = 0.f, au = 0.f;
 #pragma unroll 4
       for (int kc = lane; kc < k8; kc += 64) {
-        const u32x4 a = ldg_stream(wg + kc);
-        const u32x4 b = ldg_stream(wu + kc);
         const u32x4 x = xs4[kc];
-        ag = dot8(a, x, ag);
-        au = dot8(b, x, au);
+        ag = dot8(ldg_stream(wg + kc), x, ag);
+        au = dot8(ldg_stream(wu + kc), x, au);
       }
-      ag = wave_sum(ag);
-      au = wave_sum(au);
-      if (lane == 0) out[r] = (uint16_t)f2bf(silu_mul(ag, au));
-    }
-  } else {
-    int r = r0;
-    for (; r + 1 < r1; r += 2) {
-      const u32x4 *w0 = weight_row(st.w, r, k8);
-      const u32x4 *w1 = weight_row(st.w, r + 1, k8);
-      float a0 = 0.f, a1 = 0.f;
-#pragma unroll 4
-      for (int kc = lane; kc < k8; kc += 64) {
-        const u32x4 a = ldg_stream(w0 + kc);
-        const u32x4 b = ldg_stream(w1 + kc);
-        const u32x4 x = xs4[kc];
-        a0 = dot8(a, x, a0);
-        a1 = dot8(b, x, a1);
-      }
-      a0 = wave_sum(a0);
-      a1 = wave_sum(a1);
-      if (lane == 0) {
-        if (st.flags & MK_F_RES) {
-          a0 += bf2f(res[r]);
-          a1 += bf2f(res[r + 1]);
-        }
-        out[r] = (uint16_t)f2bf(a0);
-        out[r + 1] = (uint16_t)f2bf(a1);
-      }
-    }
-    for (; r < r1; r++) {
+      v = silu_mul(wave_sum(ag), wave_sum(au));
+    } else {
       const u32x4 *w0 = weight_row(st.w, r, k8);
       float a0 = 0.f;
 #pragma unroll 4
       for (int kc = lane; kc < k8; kc += 64) a0 = dot8(ldg_stream(w0 + kc), xs4[kc], a0);
-      a0 = wave_sum(a0);
-      if (lane == 0) {
-        if (st.flags & MK_F_RES) a0 += bf2f(res[r]);
-        out[r] = (uint16_t)f2bf(a0);
-      }
+      v = wave_sum(a0);
+      if (st.flags & MK_F_RES) v += bf2f(ldc_u16(res + r));
     }
+    if (lane == 0) out[r] = (uint16_t)f2bf(v);
+  }
+}
+
+__device__ void stage_linear_m1(const MkStage &st, Ctx &c, char *smem) {
+  const bool silu = st.flags & MK_F_SILU;
+  if (st.k == 4096) {
+    if (silu) stage_linear_m1_t<8, 4, true>(st, c, smem);
+    else stage_linear_m1_t<8, 4, false>(st, c, smem);
+  } else if (st.k == 12288 && !silu) {
+    stage_linear_m1_t<24, 2, false>(st, c, smem);
+  } else if (st.k == 2048) {
+    if (silu) stage_linear_m1_t<4, 4, true>(st, c, smem);
+    else stage_linear_m1_t<4, 4, false>(st, c, smem);
+  } else if (st.k == 1024 && !silu) {
+    stage_linear_m1_t<2, 4, false>(st, c, smem);
+  } else {
+    stage_linear_m1_generic(st, c, smem);
   }
 }
 
 // Standalone SwiGLU over interleaved [gate ; up] groups (used when the graph keeps the
 // gate/up linear and the activation apart).  Reference task: tasks/mi300/silu_mul_mi300.cuh:42-184.
-__device__ void stage_silu_mul(const MkStage &st, const Ctx &c, int M) {
+__device__ void stage_silu_mul(const MkStage &st, Ctx &c, int M) {
+  barrier_wait(c);
   const int n = st.n, half = st.silu_half;
   const uint16_t *in = (const uint16_t *)st.in;
   uint16_t *out = (uint16_t *)st.out;
@@ -406,7 +626,7 @@ __device__ void stage_silu_mul(const MkStage &st, const Ctx &c, int M) {
     const int t = i / n, j = i - t * n;
     const int g = j / half, jj = j - g * half;
     const uint16_t *row = in + (size_t)t * st.ld_in + (size_t)g * 2 * half;
-    out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(silu_mul(bf2f(row[jj]), bf2f(row[half + jj])));
+    out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(silu_mul(bf2f(ldc_u16(row + jj)), bf2f(ldc_u16(row + half + jj))));
   }
 }
 
@@ -415,7 +635,7 @@ __device__ void stage_silu_mul(const MkStage &st, const Ctx &c, int M) {
 // rotation, as in the reference (tasks/mi300/kv_cache_update_mi300.cuh:129-182).
 __device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst, const uint16_t *nw, const uint16_t *cos_row,
                                               const uint16_t *sin_row, int flags, float eps, int lane) {
-  float x0 = bf2f(src[lane]), x1 = bf2f(src[lane + 64]);
+  float x0 = bf2f(ldc_u16(src + lane)), x1 = bf2f(ldc_u16(src + lane + 64));
   if (flags & MK_F_QK_NORM) {
     const float ss = wave_sum(x0 * x0 + x1 * x1);
     const float r = rsqrtf(ss * (1.f / 128.f) + eps);
@@ -443,7 +663,8 @@ __device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst
 // paged_attention_minimal_decode (tasks/mi300/paged_attention_decode_minimal_mi300.cuh:100-371),
 // gang_attention_split_kv_kernel (tasks/mi300/gang_attention_mi300.cuh:49-153).
 template <int QPK>
-__device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt, int M, char *smem) {
+__device__ void stage_attn(const MkStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
+  barrier_wait(c);
   constexpr int D = 128;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int j16 = lane & 15, gg = wave * 4 + (lane >> 4);
@@ -464,13 +685,13 @@ __device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt,
   for (int u = c.vid; u < n_units; u += c.G) {
     const int item = u / cmax, cidx = u - item * cmax;
     const int t = item / nkv, h = item - t * nkv;
-    const int p = rt.tok_pos[t], L = p + 1;
-    int C = (L + 31) / 32;
+    const int p = ldc_i32(&rt.tok_pos[t]), L = p + 1;
+    int C = (L + 63) / 64;  // at least 64 positions (4 per lane group) per chunk
     C = C > cmax ? cmax : C;
     if (cidx >= C) continue;
     const int start = (int)(((long long)L * cidx) / C), end = (int)(((long long)L * (cidx + 1)) / C);
-    const int slot = rt.tok_slot[t], t0 = rt.tok_first[t], p0 = rt.tok_pos[t0];
-    const int *pages = rt.kv_indices + rt.kv_indptr[slot];
+    const int slot = ldc_i32(&rt.tok_slot[t]), t0 = ldc_i32(&rt.tok_first[t]), p0 = ldc_i32(&rt.tok_pos[t0]);
+    const int *pages = rt.kv_indices + ldc_i32(&rt.kv_indptr[slot]);
     const int new_lo = max(start, p0);                 // new positions handled here: [new_lo, end)
     const int n_new = end > new_lo ? end - new_lo : 0;
     __syncthreads();  // LDS reuse across units
@@ -485,15 +706,15 @@ __device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt,
         const uint16_t *src = (const uint16_t *)st.in + (size_t)tt * st.ld_in + (size_t)h * (QPK + 2) * D + QPK * D;
         prep_head_row(src, knew + j * D, (const uint16_t *)st.k_norm_w, (const uint16_t *)st.cos_tab + (size_t)pos * st.ld_cos,
                       (const uint16_t *)st.sin_tab + (size_t)pos * st.ld_cos, st.flags, st.eps, lane);
-        vnew[j * D + lane] = src[D + lane];
-        vnew[j * D + lane + 64] = src[D + lane + 64];
+        vnew[j * D + lane] = ldc_u16(src + D + lane);
+        vnew[j * D + lane + 64] = ldc_u16(src + D + lane + 64);
       }
     }
     __syncthreads();
     // the chunk that owns the newest position appends this token's K/V and publishes q
     if (cidx == C - 1) {
       const int j = p - new_lo;
-      const size_t rowi = (size_t)pages[p / ps] * ps + (p % ps);
+      const size_t rowi = (size_t)ldc_i32(&pages[p / ps]) * ps + (p % ps);
       uint32_t *kd = (uint32_t *)st.k_cache + (rowi * nkv + h) * (D / 2);
       uint32_t *vd = (uint32_t *)st.v_cache + (rowi * nkv + h) * (D / 2);
       if (tid < 64) kd[tid] = ((const uint32_t *)(knew + j * D))[tid];
@@ -530,10 +751,20 @@ __device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt,
       }
     };
     const int cend = min(end, p0);
-    for (int pos = start + gg; pos < cend; pos += 16) {
-      const size_t rowi = (size_t)pages[pos / ps] * ps + (pos % ps);
+    int pos = start + gg;
+    // two positions per group in flight
+    for (; pos + 16 < cend; pos += 32) {
+      const size_t rowa = (size_t)ldc_i32(&pages[pos / ps]) * ps + (pos % ps);
+      const size_t rowb = (size_t)ldc_i32(&pages[(pos + 16) / ps]) * ps + ((pos + 16) % ps);
+      const size_t offa = (rowa * nkv + h) * (D / 8) + j16, offb = (rowb * nkv + h) * (D / 8) + j16;
+      const u32x4 ka = ldc_16B(kc + offa), va = ldc_16B(vc + offa), kb = ldc_16B(kc + offb), vb = ldc_16B(vc + offb);
+      process(ka, va);
+      process(kb, vb);
+    }
+    for (; pos < cend; pos += 16) {
+      const size_t rowi = (size_t)ldc_i32(&pages[pos / ps]) * ps + (pos % ps);
       const size_t off = (rowi * nkv + h) * (D / 8) + j16;
-      process(kc[off], vc[off]);
+      process(ldc_16B(kc + off), ldc_16B(vc + off));
     }
     for (int j = gg; j < n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
     // ---- phase C: merge the 16 groups through LDS
@@ -578,24 +809,37 @@ __device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt,
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(&rt.attn_cnt[item], 1u, __ATOMIC_ACQ_REL, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned old = __hip_atomic_fetch_add(&rt.attn_cnt[item], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         const int last = (old == (unsigned)(C - 1));
         if (last) __hip_atomic_store(&rt.attn_cnt[item], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         *sflag = last;
       }
       __syncthreads();
       if (*sflag) {
+        // all chunk partials are read with independent device-scope loads, eight chunks in flight per thread
         const float *ip = rt.attn_part + (size_t)item * cmax * QPK * (D + 2);
         for (int o = tid; o < QPK * D; o += MK_THREADS) {
           const int hh = o >> 7, d = o & 127;
-          float mx = -INFINITY;
-          for (int cc = 0; cc < C; cc++) mx = fmaxf(mx, ip[((size_t)cc * QPK + hh) * (D + 2) + D]);
-          float ls = 0.f, os = 0.f;
-          for (int cc = 0; cc < C; cc++) {
-            const float *pp = ip + ((size_t)cc * QPK + hh) * (D + 2);
-            const float wgt = __builtin_amdgcn_exp2f(pp[D] - mx);
-            ls += pp[D + 1] * wgt;
-            os += pp[d] * wgt;
+          float mx = -INFINITY, ls = 0.f, os = 0.f;
+          for (int c0 = 0; c0 < C; c0 += 8) {
+            float mv[8], lv[8], ov[8];
+#pragma unroll
+            for (int j = 0; j < 8; j++) {
+              const int cc = min(c0 + j, C - 1);
+              const float *pp = ip + ((size_t)cc * QPK + hh) * (D + 2);
+              mv[j] = ldc_f32(pp + D);
+              lv[j] = ldc_f32(pp + D + 1);
+              ov[j] = ldc_f32(pp + d);
+            }
+#pragma unroll
+            for (int j = 0; j < 8; j++)
+              if (c0 + j < C) {
+                const float mn = fmaxf(mx, mv[j]);
+                const float a = __builtin_amdgcn_exp2f(mx - mn), b = __builtin_amdgcn_exp2f(mv[j] - mn);
+                ls = ls * a + lv[j] * b;
+                os = os * a + ov[j] * b;
+                mx = mn;
+              }
           }
           orow[o] = (uint16_t)f2bf(os / ls);
         }
@@ -606,11 +850,13 @@ __device__ void stage_attn(const MkStage &st, const Ctx &c, const MkRuntime &rt,
 
 // Greedy sampling, stage 1: every workgroup scans a contiguous slice of each token's logits and keeps
 // (max, lowest index attaining it).  Reference task: tasks/mi300/argmax_mi300.cuh:78-127.
-__device__ void stage_argmax_partial(const MkStage &st, const Ctx &c, int M, char *smem) {
+__device__ void stage_argmax_partial(const MkStage &st, Ctx &c, int M, char *smem) {
+  barrier_wait(c);
   float *sv = (float *)smem;
   int *si = (int *)(smem + 1024);
   const int n = st.n;
-  const int per = (n + c.G - 1) / c.G;
+  int per = (n + c.G - 1) / c.G;
+  per = (per + 1) & ~1;  // even, so slices start on a dword
   const int c0 = c.vid * per, c1 = min(n, c0 + per);
   float *pv = (float *)st.aux0;
   int *pi = (int *)st.aux1;
@@ -619,11 +865,16 @@ __device__ void stage_argmax_partial(const MkStage &st, const Ctx &c, int M, cha
     const uint16_t *row = (const uint16_t *)st.in + (size_t)t * st.ld_in;
     float best = -INFINITY;
     int bi = 0x7fffffff;
-    for (int i = c0 + threadIdx.x; i < c1; i += MK_THREADS) {
-      const float v = bf2f(row[i]);
-      if (v > best) {
-        best = v;
+    for (int i = c0 + 2 * (int)threadIdx.x; i < c1; i += 2 * MK_THREADS) {
+      const uint32_t w = ldc_u32(row + i);
+      const float v0 = bf_lo(w), v1 = bf_hi(w);
+      if (v0 > best) {
+        best = v0;
         bi = i;
+      }
+      if (i + 1 < c1 && v1 > best) {
+        best = v1;
+        bi = i + 1;
       }
     }
 #pragma unroll
@@ -655,7 +906,8 @@ __device__ void stage_argmax_partial(const MkStage &st, const Ctx &c, int M, cha
 
 // Greedy sampling, stage 2: one wavefront per token reduces the per-workgroup partials.
 // Reference task: tasks/mi300/argmax_mi300.cuh:129-158.
-__device__ void stage_argmax_reduce(const MkStage &st, const Ctx &c, int M) {
+__device__ void stage_argmax_reduce(const MkStage &st, Ctx &c, int M) {
+  barrier_wait(c);
   const float *pv = (const float *)st.aux0;
   const int *pi = (const int *)st.aux1;
   long long *out = (long long *)st.out;
@@ -664,8 +916,8 @@ __device__ void stage_argmax_reduce(const MkStage &st, const Ctx &c, int M) {
     float best = -INFINITY;
     int bi = 0x7fffffff;
     for (int i = lane; i < c.G; i += 64) {
-      const float v = pv[t * c.G + i];
-      const int ix = pi[t * c.G + i];
+      const float v = ldc_f32(&pv[t * c.G + i]);
+      const int ix = ldc_i32(&pi[t * c.G + i]);
       if (v > best || (v == best && ix < bi)) {
         best = v;
         bi = ix;
@@ -695,6 +947,11 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.sync = rt.sync;
   c.xcd = xcc_id();
   c.epoch = 0;
+  c.pending = false;
+  c.leader = false;
+  c.dead = false;
+  c.t_wait = 0;
+  c.sh_dead = &sh_bcast[3];
   // ---- XCD discovery: rank of this workgroup inside its die, dies in use, workgroups per die
   if (threadIdx.x == 0) {
     MkSync *s = rt.sync;
@@ -712,51 +969,67 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     sh_bcast[0] = before + (int)rank;
     sh_bcast[1] = nx;
     sh_bcast[2] = (int)__hip_atomic_load(&s->xcd_count[c.xcd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    sh_bcast[3] = (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
   c.vid = sh_bcast[0];
   c.nxcd = sh_bcast[1];
   c.quota = sh_bcast[2];
+  c.dead = sh_bcast[3] != 0;
   __syncthreads();
 
-  for (int it = 0; it < max_iters; it++) {
+  for (int it = 0; it < max_iters && !c.dead; it++) {
     // ---- scheduler step on one thread of virtual workgroup 0, published through the barrier
-    if (run_scheduler && c.vid == 0 && threadIdx.x == 0) {
-      const int ntok = mk_prepare_next_batch(rt, (int *)smem);
-      if (ntok == 0) rt.sched->finished = 1;
-      else rt.sched->iterations++;
-      if (rt.timing && rt.sched->iterations <= rt.timing_cap) rt.timing[rt.sched->iterations] = (long long)wall_clock64();
+    if (run_scheduler) {
+      barrier_wait(c);  // the previous iteration's sampled tokens are complete
+      if (c.vid == 0 && threadIdx.x == 0) {
+        const int ntok = mk_prepare_next_batch(rt, (int *)smem);
+        if (ntok == 0) rt.sched->finished = 1;
+        else rt.sched->iterations++;
+        if (rt.timing && rt.sched->iterations <= rt.timing_cap) rt.timing[rt.sched->iterations] = (long long)wall_clock64();
+      }
+      barrier_arrive(c);
     }
-    bool dead = false;
-    if (run_scheduler) dead = grid_barrier(c, &sh_bcast[3]);
-    if (threadIdx.x == 0) sh_bcast[0] = rt.sched->num_tokens;
+    barrier_wait(c);
+    if (threadIdx.x == 0) sh_bcast[0] = ldc_i32(&rt.sched->num_tokens);
     __syncthreads();
     const int M = sh_bcast[0];
     __syncthreads();
-    if (M == 0 || dead) break;
+    if (M == 0 || c.dead) break;
 
-    for (int s = 0; s < rt.num_stages && !dead; s++) {
+    for (int s = 0; s < rt.num_stages && !c.dead; s++) {
       const MkStage &st = rt.stages[s];
       const int op = st.op, flags = st.flags;
       if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
+      const long long t_in = (long long)wall_clock64();
       switch (op) {
         case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
         case MK_OP_LINEAR:
           if (M == 1) stage_linear_m1(st, c, smem);
+          else barrier_wait(c);
           break;
         case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
         case MK_OP_ATTN:
           if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4>(st, c, rt, M, smem);
           else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8>(st, c, rt, M, smem);
+          else barrier_wait(c);
           break;
         case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, M, smem); break;
         case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, M); break;
-        default: break;
+        default: barrier_wait(c); break;
       }
-      dead = grid_barrier(c, &sh_bcast[3]);
+      const long long t_out = (long long)wall_clock64();
+      barrier_arrive(c);
+      if (threadIdx.x == 0 && rt.stage_prof) {
+        long long *pr = rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + s);
+        pr[0] = t_in;
+        pr[1] = c.t_wait;
+        pr[2] = t_out;
+        pr[3] = (long long)wall_clock64();
+      }
     }
-    if (dead) break;
   }
+  barrier_wait(c);  // drain: nobody leaves while another workgroup may still poll
   if (c.vid == 0 && threadIdx.x == 0 && rt.timing) rt.timing[0] = (long long)wall_clock64();
 }

@@ -17,7 +17,14 @@
 #define MK_MAX_TOKENS 64      // max tokens per iteration supported by the kernels
 #define MK_ATTN_MAX_CHUNKS 32 // split-KV fan-out limit per (token, kv head)
 #define MK_MAX_NEW_PER_REQ 8  // prefill tokens per request per iteration (reference: MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
-#define MK_LDS_BYTES (96 * 1024)  // dynamic LDS per workgroup; > 80 KB pins one workgroup per CU
+// LDS map of one workgroup (dynamic, > 80 KB pins one workgroup per CU):
+//   [0, 24 KB)      input row(s) of the running stage / attention scratch (attention may run on into the ring)
+//   [24 KB, 25 KB)  reduction scratch
+//   [32 KB, 128 KB) weight prefetch rings of the worker wavefronts, filled by direct-to-LDS loads across the grid barrier
+#define MK_RED_OFFSET (24 * 1024)
+#define MK_PF_OFFSET (32 * 1024)
+#define MK_PF_BYTES (96 * 1024)
+#define MK_LDS_BYTES (128 * 1024)
 
 enum MkOp {
   MK_OP_NONE = 0,
@@ -129,6 +136,7 @@ struct MkRuntime {
   // attention split-KV workspace
   float *attn_part;     // [units][qpk][head_dim + 2]
   unsigned *attn_cnt;   // [max_tokens * num_kv_heads]
-  long long *timing;    // optional [2 + 2*max] wall-clock ticks per iteration
+  long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end
   int timing_cap, pad0;
+  long long *stage_prof; // [workgroups][num_stages][4] ticks of the last iteration: entry, wait done, exit, arrived
 };

@@ -22,7 +22,7 @@ EXPORTED_SYMBOLS = [
     "mk_graph_create", "mk_graph_destroy", "mk_tensor_attach", "mk_tensor_new", "mk_tensor_shuffle",
     "mk_tensor_num_dims", "mk_tensor_dim", "mk_tensor_ptr", "mk_add_task", "mk_generate_task_graph",
     "mk_compile", "mk_init_requests", "mk_launch", "mk_launch_steps", "mk_enqueue_steps", "mk_wait",
-    "mk_run_once", "mk_get_stats", "mk_describe_program", "mk_last_error", "mk_version",
+    "mk_run_once", "mk_get_stats", "mk_get_stage_profile", "mk_describe_program", "mk_last_error", "mk_version",
 ]
 
 
@@ -109,6 +109,7 @@ def load():
     i32p = ctypes.POINTER(ctypes.c_int32)
     lib.mk_run_once.argtypes = [vp, vp, ci, i32p, i32p, i32p]
     lib.mk_get_stats.argtypes = [vp, ctypes.POINTER(MkStats)]
+    lib.mk_get_stage_profile.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_int64), ci]
     lib.mk_describe_program.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p)]
     lib.mk_last_error.restype = ctypes.c_char_p
     lib.mk_version.restype = ctypes.c_char_p

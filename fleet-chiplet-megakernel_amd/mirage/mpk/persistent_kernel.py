@@ -526,6 +526,19 @@ class PersistentKernel:
         _capi.check(self._lib.mk_get_stats(self._handle, ctypes.byref(st)))
         return {name: getattr(st, name) for name, _ in st._fields_}
 
+    def stage_profile(self, workgroup: int = 0, raw: bool = False):
+        """Per-stage timing of the last iteration on one virtual workgroup: list of (description, entered,
+        barrier_satisfied, work_done, arrived) in microseconds relative to that workgroup's first stage (raw=True:
+        100 MHz ticks, comparable across workgroups; 0 = stage skipped)."""
+        n = self.stats()["num_stages"]
+        buf = (ctypes.c_int64 * (4 * max(1, n)))()
+        got = _capi.check(self._lib.mk_get_stage_profile(self._handle, int(workgroup), buf, n))
+        desc = self.describe_program().splitlines()
+        if raw:
+            return [(desc[i], *[int(buf[4 * i + k]) for k in range(4)]) for i in range(got)]
+        t0 = min(buf[4 * i] for i in range(got) if buf[4 * i] > 0) if got else 0
+        return [(desc[i], *[(buf[4 * i + k] - t0) * 0.01 if buf[4 * i] > 0 else -1.0 for k in range(4)]) for i in range(got)]
+
     def finalize(self):
         assert not self.__finalized__
         if self._handle is not None:

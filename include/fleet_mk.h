@@ -144,6 +144,11 @@ typedef struct mk_stats {
   double last_launch_ms;   /* HIP-event time of the last launch's kernel, on the stream it ran on */
 } mk_stats;
 int mk_get_stats(mk_graph *g, mk_stats *out);
+/* Device-side stage timing of the LAST decode iteration, as seen by virtual workgroup `workgroup`: for each stage four
+ * 100 MHz wall-clock ticks {entered, previous stage's barrier satisfied, work done, arrival posted}.  Returns the number
+ * of stages written (<= max_stages).  Counterpart of the reference's MPK_ENABLE_EVENT_TIMING ring
+ * (persistent_kernel.cuh:1299-1307,2412-2429). */
+int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages);
 /* Stage listing (one line per stage) for debugging and tests; owned by the handle. */
 int mk_describe_program(mk_graph *g, const char **text_out);
 
