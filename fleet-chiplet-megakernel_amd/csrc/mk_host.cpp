@@ -227,6 +227,7 @@ int lower_linear(mk_graph *g, size_t &i) {
   st.op = MK_OP_LINEAR;
   st.k = (int)tin.dims[1];
   if (st.k % 8) return fail(MK_EINVAL, "task '%s': reduction length %d must be a multiple of 8", lt.name.c_str(), st.k);
+  if (g->cfg.max_num_batched_tokens > 1 && st.k % 32) return fail(MK_EINVAL, "task '%s': reduction length %d must be a multiple of 32 when more than one token is batched", lt.name.c_str(), st.k);
   int64_t rows;
   int half;
   int rc = resolve_weight(g, w_id, st.k, &st.w, &rows, &half);
@@ -293,6 +294,7 @@ int lower_linear(mk_graph *g, size_t &i) {
     st.ld_in = (int)nx.strides[0];
     st.norm_w = nw.ptr;
     st.norm_out = no.ptr;
+    st.ld_norm = (int)no.strides[0];
   }
   g->stages.push_back(st);
   g->stage_desc.push_back(fmt("LINEAR%s%s%s %s x %s -> %s n=%d k=%d segs=%d", (st.flags & MK_F_NORM) ? "+norm" : "", (st.flags & MK_F_RES) ? "+res" : "",

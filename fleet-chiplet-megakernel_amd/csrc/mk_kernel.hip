@@ -14,6 +14,8 @@
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
 typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
+typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
+typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define MK_SPIN_LIMIT (1u << 24)
 
@@ -614,6 +616,118 @@ __device__ void stage_linear_m1(const MkStage &st, Ctx &c, char *smem) {
   }
 }
 
+
+// Multi-token linear on the matrix cores: out[m, n] = bf16(sum_k x[m,k] * W[n,k] (+ res[m,n])) for 2..64 token rows,
+// optional SwiGLU epilogue.  A workgroup owns a contiguous range of 16-row weight tiles and ALL token rows, so every
+// weight byte is still read from HBM exactly once; its four wavefronts split K and are reduced through LDS.  One
+// v_mfma_f32_16x16x32_bf16 consumes a 16(n) x 32(k) weight fragment (one 16-byte load per lane, 64 contiguous bytes per
+// weight row) against a 32(k) x 16(m) activation fragment that comes from the L2-resident activation rows.
+// Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
+// (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
+template <int MT>
+__device__ void stage_linear_mfma(const MkStage &st, Ctx &c, int M, char *smem) {
+  constexpr int TG = 6;  // weight tiles per K sweep
+  barrier_wait(c);
+  // activations were produced by other workgroups: invalidate this CU's L1 once, then use cached loads so the rows
+  // are shared through the XCD's L2
+  if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  __syncthreads();
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int lr = lane & 15, lg = lane >> 4;
+  const bool silu = st.flags & MK_F_SILU;
+  const int K = st.k, k8 = K / 8;
+  const int n_out = silu ? st.n / 2 : st.n;
+  const int ntiles = (n_out + 15) / 16;  // output tiles of 16 columns
+  const int t_begin = (int)(((long long)c.vid * ntiles) / c.G), t_end = (int)(((long long)(c.vid + 1) * ntiles) / c.G);
+  const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
+  const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
+  const int kq = ((K / 32 + MK_WAVES - 1) / MK_WAVES) * 32;  // K slice per wavefront, multiple of 32
+  const int kbeg = min(K, wave * kq), kend = min(K, kbeg + kq);
+  const int half = st.silu_half;
+  const int otg = silu ? TG / 2 : TG;  // output tiles per sweep
+  f32x4 *red = (f32x4 *)smem;           // [waves][TG][MT][64]
+  const uint16_t *xrow[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) xrow[mt] = x + (size_t)min(mt * 16 + lr, M - 1) * ldx + lg * 8;
+
+  for (int ot0 = t_begin; ot0 < t_end; ot0 += otg) {
+    const int not_ = min(otg, t_end - ot0);       // output tiles in this sweep
+    const int nt = silu ? 2 * not_ : not_;        // weight tiles in this sweep
+    const uint16_t *wrow[TG];
+#pragma unroll
+    for (int t = 0; t < TG; t++) {
+      const int ot = ot0 + (silu ? (t >> 1) : t);
+      int o = min(ot * 16 + lr, n_out - 1);       // output column owned by this lane's weight row
+      int vr = o;
+      if (silu) {
+        const int g = o / half;
+        vr = g * 2 * half + (o - g * half) + ((t & 1) ? half : 0);
+      }
+      wrow[t] = (const uint16_t *)weight_row(st.w, vr, k8) + lg * 8;
+    }
+    f32x4 acc[TG][MT];
+#pragma unroll
+    for (int t = 0; t < TG; t++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+#pragma unroll 2
+    for (int k = kbeg; k < kend; k += 32) {
+      bf16x8 a[TG], b[MT];
+#pragma unroll
+      for (int t = 0; t < TG; t++)
+        if (t < nt) a[t] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k));
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) b[mt] = *(const bf16x8 *)(xrow[mt] + k);
+#pragma unroll
+      for (int t = 0; t < TG; t++)
+        if (t < nt) {
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[mt], acc[t][mt], 0, 0, 0);
+        }
+    }
+    __syncthreads();  // previous sweep's epilogue has finished reading LDS
+#pragma unroll
+    for (int t = 0; t < TG; t++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) red[((wave * TG + t) * MT + mt) * 64 + lane] = acc[t][mt];
+    __syncthreads();
+    // epilogue: entry (output tile u, token tile mt, lane slot l) -> 4 consecutive output columns of one token row
+    const int entries = not_ * MT * 64;
+    for (int e = tid; e < entries; e += MK_THREADS) {
+      const int l = e & 63, mt = (e >> 6) % MT, u = (e >> 6) / MT;
+      const int m = mt * 16 + (l & 15);
+      const int n0 = (ot0 + u) * 16 + (l >> 4) * 4;
+      f32x4 v, v2;
+      if (silu) {
+        v = red[((0 * TG + 2 * u) * MT + mt) * 64 + l];
+        v2 = red[((0 * TG + 2 * u + 1) * MT + mt) * 64 + l];
+#pragma unroll
+        for (int w = 1; w < MK_WAVES; w++) {
+          v += red[((w * TG + 2 * u) * MT + mt) * 64 + l];
+          v2 += red[((w * TG + 2 * u + 1) * MT + mt) * 64 + l];
+        }
+      } else {
+        v = red[((0 * TG + u) * MT + mt) * 64 + l];
+#pragma unroll
+        for (int w = 1; w < MK_WAVES; w++) v += red[((w * TG + u) * MT + mt) * 64 + l];
+      }
+      if (m < M) {
+        uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
+        const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
+#pragma unroll
+        for (int i = 0; i < 4; i++) {
+          const int n = n0 + i;
+          if (n < n_out) {
+            float r = silu ? silu_mul(v[i], v2[i]) : v[i];
+            if (st.flags & MK_F_RES) r += bf2f(rrow[n]);
+            orow[n] = (uint16_t)f2bf(r);
+          }
+        }
+      }
+    }
+  }
+}
+
 // Standalone SwiGLU over interleaved [gate ; up] groups (used when the graph keeps the
 // gate/up linear and the activation apart).  Reference task: tasks/mi300/silu_mul_mi300.cuh:42-184.
 __device__ void stage_silu_mul(const MkStage &st, Ctx &c, int M) {
@@ -1007,7 +1121,10 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
         case MK_OP_LINEAR:
           if (M == 1) stage_linear_m1(st, c, smem);
-          else barrier_wait(c);
+          else if (M <= 16) stage_linear_mfma<1>(st, c, M, smem);
+          else if (M <= 32) stage_linear_mfma<2>(st, c, M, smem);
+          else if (M <= 48) stage_linear_mfma<3>(st, c, M, smem);
+          else stage_linear_mfma<4>(st, c, M, smem);
           break;
         case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
         case MK_OP_ATTN:

@@ -78,7 +78,7 @@ struct MkStage {
   const void *q_norm_w, *k_norm_w, *cos_tab, *sin_tab;
   void *q_ws;
   int num_q_heads, num_kv_heads, head_dim, ld_qws;
-  int ld_cos, pad2;
+  int ld_cos, ld_norm;  // ld_norm: leading dimension of norm_out
   float sm_scale_log2;  // log2(e) / sqrt(head_dim)
   int pad3;
   // argmax

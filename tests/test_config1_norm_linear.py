@@ -56,3 +56,43 @@ def test_norm_linear_bs1(gang, H, N):
     st = mpk.stats()
     assert st["num_xcds"] == 8 and st["aborted"] == 0
     mpk.finalize()
+
+
+@pytest.mark.parametrize("M", [2, 5, 16, 17, 33, 64])
+@pytest.mark.parametrize("H,N,res", [(4096, 4096, True), (1024, 3008, False), (12288, 512, True)])
+def test_norm_linear_multi_token(M, H, N, res):
+    """Multi-token rows take the MFMA path (norm as its own stage, linear with optional residual)."""
+    import mirage as mi
+    from oracle.qwen3_ref import linear_k, rmsnorm_k
+    g = torch.Generator().manual_seed(M * 7 + N)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    nw = (1.0 + 0.02 * torch.randn(H, generator=g)).to(torch.bfloat16)
+    W = (0.02 * torch.randn(N, H, generator=g)).to(torch.bfloat16)
+    r = torch.randn(M, N, generator=g).to(torch.bfloat16)
+    B = 64
+    meta = make_meta(1, 64, B, B, B)
+    mpk = make_mpk(meta, 64, B, B, B, 64, mode="onepass")
+    pad = lambda t: torch.cat([t, torch.zeros(B - t.shape[0], t.shape[1], dtype=t.dtype)]).cuda()
+    xd, nwd, Wd, rd = pad(x), nw.cuda(), W.cuda(), pad(r)
+    tx, tnw, tW, tr = mpk.attach_input(xd, "x"), mpk.attach_input(nwd, "norm_w"), mpk.attach_input(Wd, "W"), mpk.attach_input(rd, "res")
+    tn = mpk.new_tensor((B, H), dtype=mi.bfloat16, name="norm_out")
+    ty = mpk.new_tensor((B, N), dtype=mi.bfloat16, name="y")
+    mpk.rmsnorm_layer(input=tx, weight=tnw, output=tn, grid_dim=(B, 1, 1), block_dim=(128, 1, 1))
+    if res:
+        mpk.linear_with_residual_layer(input=tn, weight=tW, residual=tr, output=ty, grid_dim=(N // 64, 1, 1), block_dim=(256, 1, 1))
+    else:
+        mpk.linear_layer(input=tn, weight=tW, output=ty, grid_dim=(N // 64, 1, 1), block_dim=(128, 1, 1))
+    mpk.compile()
+    mpk.run_once(list(range(M)), [0] * M)   # M requests with one token each
+    y = ty.to_torch().cpu()
+    n_gpu = tn.to_torch().cpu()
+    n_ref = rmsnorm_k(x, nw)
+    ulp_n, _ = bf16_ulp_diff(n_gpu[:M], n_ref)
+    assert ulp_n <= 1.0
+    y_ref = linear_k(n_gpu[:M], W, res=r if res else None)   # oracle fed with the GPU's own normalised rows
+    frac = float((y[:M].float() != y_ref.float()).float().mean())
+    ulp, mabs = bf16_ulp_diff(y[:M], y_ref, floor=1.0 / 16)
+    assert ulp <= 1.0 and frac < 0.02, f"{frac:.4f} of outputs differ, max {ulp} ulp ({mabs})"
+    assert float(y[M:].abs().sum()) == 0.0, "rows beyond the batch must not be written"
+    assert mpk.stats()["aborted"] == 0
+    mpk.finalize()

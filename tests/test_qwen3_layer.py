@@ -156,3 +156,19 @@ def test_v_append_exact_and_qkv_matches():
     qkv = res["qkv_gpu"][0].view(cfg.num_kv_heads, (cfg.num_q_heads // cfg.num_kv_heads) + 2, cfg.head_dim)
     v_new = qkv[:, -1, :]
     assert torch.equal(res["v_after"][pages[70 // ps], 70 % ps], v_new)
+
+
+@pytest.mark.parametrize("L_cached,n_new", [(0, 5), (0, 8), (70, 8), (300, 3), (63, 2)])
+def test_small_layer_prefill_chunks(L_cached, n_new):
+    """Several new tokens of one request in one pass (chunked prefill): causal attention inside the chunk, MFMA linears."""
+    from oracle.qwen3_ref import Qwen3Config
+    cfg = Qwen3Config(hidden_size=1024, num_q_heads=8, num_kv_heads=2, head_dim=128, intermediate_size=1536, num_layers=1)
+    res = _run_layer(cfg, L_cached, n_new, "fleet", seed=100 + L_cached + n_new)
+    _check(res, cfg, L_cached, n_new)
+
+
+def test_full_width_layer_prefill_chunk_mpk_mode():
+    from oracle.qwen3_ref import Qwen3Config
+    cfg = Qwen3Config(num_layers=1)
+    res = _run_layer(cfg, 40, 8, "mpk", seed=9)
+    _check(res, cfg, 40, 8)
