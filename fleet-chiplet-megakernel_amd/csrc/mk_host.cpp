@@ -10,6 +10,7 @@
 #include <math.h>
 #include <stdarg.h>
 #include <stdio.h>
+#include <stdlib.h>
 #include <string.h>
 
 #include <array>
@@ -93,7 +94,9 @@ struct mk_graph {
   std::vector<Tensor> tensors;
   std::vector<Task> tasks;
   bool compiled = false;
+  bool host_only = false;  // created with device < 0: records, validates, lowers and emits the task graph, never launches
   std::vector<void *> allocs;
+  std::vector<void *> host_allocs;
   std::vector<MkStage> stages;
   std::vector<std::string> stage_desc;
   MkRuntime h_rt;
@@ -117,6 +120,12 @@ namespace {
 
 int dev_alloc(mk_graph *g, void **out, size_t bytes, bool zero = true) {
   if (bytes == 0) bytes = 16;
+  if (g->host_only) {  // stand-in address: only its identity matters to the lowering
+    *out = malloc(16);
+    if (!*out) return fail(MK_EINVAL, "out of host memory");
+    g->host_allocs.push_back(*out);
+    return MK_OK;
+  }
   HIP_TRY(hipMalloc(out, bytes));
   g->allocs.push_back(*out);
   if (zero) HIP_TRY(hipMemset(*out, 0, bytes));
@@ -726,6 +735,17 @@ int mk_graph_create(const mk_config *cfg, mk_graph **out) {
     return fail(MK_EINVAL, "max_num_pages*page_size=%lld cannot hold one sequence of max_seq_length=%d", (long long)cfg->max_num_pages * cfg->page_size,
                 cfg->max_seq_length);
   if (cfg->max_num_pages > (MK_LDS_BYTES / 4)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 4);
+  if (cfg->device < 0) {
+    mk_graph *g = new mk_graph();
+    g->cfg = *cfg;
+    if (g->cfg.rms_eps == 0.f) g->cfg.rms_eps = 1e-6f;
+    g->host_only = true;
+    g->num_cus = 256;
+    g->G = cfg->num_workers > 0 ? cfg->num_workers : 256;
+    memset(&g->h_rt, 0, sizeof(g->h_rt));
+    *out = g;
+    return MK_OK;
+  }
   int ndev = 0;
   HIP_TRY(hipGetDeviceCount(&ndev));
   if (ndev < 1) return fail(MK_EHIP, "no HIP device visible: the megakernel has no CPU fallback");
@@ -753,6 +773,7 @@ int mk_graph_destroy(mk_graph *g) {
   if (!g) return MK_OK;
   if (g->launch_pending) (void)hipDeviceSynchronize();
   for (void *p : g->allocs) (void)hipFree(p);
+  for (void *p : g->host_allocs) free(p);
   if (g->ev0) (void)hipEventDestroy(g->ev0);
   if (g->ev1) (void)hipEventDestroy(g->ev1);
   delete g;
@@ -902,6 +923,7 @@ int mk_generate_task_graph(mk_graph *g, int num_gpus, int my_gpu_id, const char 
 int mk_compile(mk_graph *g) {
   if (!g) return fail(MK_EINVAL, "null argument");
   if (g->compiled) return fail(MK_ESTATE, "graph already compiled");
+  if (g->host_only) return fail(MK_ESTATE, "this graph was created without a device (device < 0): it can be lowered and described, not compiled");
   HIP_TRY(hipSetDevice(g->cfg.device));
   const mk_config &c = g->cfg;
   if (!c.step || !c.tokens || !c.input_tokens || !c.output_tokens || !c.prompt_lengths || !c.qo_indptr || !c.paged_kv_indptr || !c.paged_kv_indices ||
@@ -1085,6 +1107,10 @@ int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max
 
 int mk_describe_program(mk_graph *g, const char **text_out) {
   if (!g || !text_out) return fail(MK_EINVAL, "null argument");
+  if (!g->compiled) {
+    int rc = lower(g);
+    if (rc) return rc;
+  }
   *text_out = g->program_text.c_str();
   return MK_OK;
 }

@@ -94,8 +94,9 @@ class PersistentKernel:
         assert mt["paged_kv_last_page_len_buffer"].shape[0] == max_num_batched_requests
         assert mt["input_tokens"].numel() >= max_num_batched_tokens and mt["output_tokens"].numel() >= max_num_batched_tokens
         device = mt["tokens"].device
-        if device.type != "cuda":
-            raise RuntimeError("meta tensors must live on the GPU: the megakernel has no CPU path")
+        # CPU meta tensors give a host-only graph: layers can be recorded, validated, lowered and dumped as a task graph,
+        # but compile() / __call__ raise -- the megakernel has no CPU path
+        self.host_only = device.type != "cuda"
         self.device = device
         lib = _capi.load()
         cfg = _capi.MkConfig()
@@ -106,7 +107,7 @@ class PersistentKernel:
         cfg.max_num_pages = max_num_pages
         cfg.page_size = page_size
         cfg.total_num_requests = self.total_num_requests
-        cfg.device = device.index if device.index is not None else torch.cuda.current_device()
+        cfg.device = -1 if self.host_only else (device.index if device.index is not None else torch.cuda.current_device())
         cfg.eos_token_id = int(eos_token_id)
         cfg.rms_eps = 1e-6
         cfg.step = mt["step"].data_ptr()
@@ -134,8 +135,8 @@ class PersistentKernel:
             assert strides[d] == strides[d + 1] * dims[d + 1], f"{name}: only row-major tensors can be attached"
         assert name is not None
         dt = convert_torch_type_to_dtype(torch_tensor.dtype)
-        if torch_tensor.device.type != "cuda":
-            raise RuntimeError(f"{name}: attached tensors must live on the GPU")
+        if (torch_tensor.device.type != "cuda") != self.host_only:
+            raise RuntimeError(f"{name}: attached tensors must live on the same kind of device as the meta tensors")
         tid = _capi.check(self._lib.mk_tensor_attach(
             self._handle, ctypes.c_void_p(torch_tensor.data_ptr()), len(dims), _capi.int_array(dims, ctypes.c_int64),
             _capi.int_array(strides, ctypes.c_int64), dt.code, name.encode()))

@@ -54,7 +54,8 @@ typedef struct mk_config {
   int max_num_pages;
   int page_size;
   int total_num_requests;       /* rows of `tokens` */
-  int device;                   /* HIP device ordinal */
+  int device;                   /* HIP device ordinal; < 0 = host-only graph (record / validate / lower / emit the task
+                                   graph without a GPU; mk_compile and the launch calls then fail with MK_ESTATE) */
   int64_t eos_token_id;
   float rms_eps;                /* 0 => 1e-6, the constant baked into the reference kernels */
   int reserved0;

@@ -1,0 +1,184 @@
+"""CPU-only checks of the drop-in boundary: the shared library loads and exports every symbol include/fleet_mk.h declares,
+and the host side (graph recording, validation, lowering to the stage program, reference-schema task graph) behaves as
+the reference's host code does for this path -- without launching anything (host-only graphs, device = -1)."""
+import ctypes
+import json
+import os
+import re
+
+import pytest
+import torch
+
+import mirage as mi
+from mirage import _capi
+from helpers import make_meta
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def test_library_exports_every_declared_symbol():
+    header = open(os.path.join(ROOT, "include", "fleet_mk.h")).read()
+    declared = sorted(set(re.findall(r"\b(mk_[a-z_0-9]+)\s*\(", header)))
+    assert len(declared) >= 20
+    lib = _capi.load()
+    for sym in declared:
+        assert hasattr(lib, sym), f"libfleet_mk.so does not export {sym}"
+    assert set(declared) == set(_capi.EXPORTED_SYMBOLS)
+    assert b"gfx950" in lib.mk_version()
+
+
+def test_status_codes_and_error_strings():
+    lib = _capi.load()
+    assert lib.mk_graph_create(None, None) == _capi.MK_EINVAL
+    assert b"null" in lib.mk_last_error()
+    cfg = _capi.MkConfig()
+    cfg.device = -1
+    cfg.max_num_batched_tokens = 65  # above the kernel's limit
+    cfg.max_num_batched_requests, cfg.page_size, cfg.max_num_pages, cfg.max_seq_length = 1, 16, 4, 32
+    h = ctypes.c_void_p()
+    assert lib.mk_graph_create(ctypes.byref(cfg), ctypes.byref(h)) == _capi.MK_EINVAL
+    assert b"max_num_batched_tokens" in lib.mk_last_error()
+    cfg.max_num_batched_tokens = 1
+    cfg.max_num_pages, cfg.page_size, cfg.max_seq_length = 1, 16, 64  # one sequence does not fit in the page pool
+    assert lib.mk_graph_create(ctypes.byref(cfg), ctypes.byref(h)) == _capi.MK_EINVAL
+
+
+def _host_mpk(B=4, R=2, max_seq=64, pages=8, page_size=16, total=2):
+    meta = make_meta(total, max_seq, B, R, pages, device="cpu")
+    return mi.PersistentKernel(mode="offline", world_size=1, mpi_rank=0, num_workers=256, num_local_schedulers=0, num_remote_schedulers=0,
+                               max_seq_length=max_seq, max_num_batched_requests=R, max_num_batched_tokens=B, max_num_pages=pages,
+                               page_size=page_size, meta_tensors=meta, profiler_tensor=None, trace_name=None, spec_decode_config=None,
+                               use_cutlass_kernel=False, eos_token_id=2)
+
+
+def _t(mpk, name, *shape, dtype=torch.bfloat16):
+    return mpk.attach_input(torch.zeros(*shape, dtype=dtype), name)
+
+
+def test_constructor_contract():
+    meta = make_meta(2, 64, 4, 2, 8, device="cpu")
+    kw = dict(world_size=1, mpi_rank=0, num_workers=256, num_local_schedulers=0, num_remote_schedulers=0, max_seq_length=64,
+              max_num_batched_requests=2, max_num_batched_tokens=4, max_num_pages=8, page_size=16, meta_tensors=meta, profiler_tensor=None,
+              trace_name=None, spec_decode_config=None, use_cutlass_kernel=False)
+    with pytest.raises(ValueError, match="Invalid persistent kernel mode"):
+        mi.PersistentKernel(mode="bogus", **kw)
+    with pytest.raises(NotImplementedError):
+        mi.PersistentKernel(mode="offline", **{**kw, "world_size": 2})
+    bad = dict(meta)
+    bad["tokens"] = meta["tokens"].to(torch.int32)
+    with pytest.raises(AssertionError, match="tokens.dtype"):
+        mi.PersistentKernel(mode="offline", **{**kw, "meta_tensors": bad})
+    mpk = mi.PersistentKernel(mode="offline", **kw)
+    assert mpk.total_num_requests == 2 and mpk.target_cc == 94 and mpk.max_num_batched_tokens == 4
+    assert mi.mpk.spec_decode_class(None, ngram_size=3, spec_length=4) is None
+    with pytest.raises(NotImplementedError):
+        mi.mpk.spec_decode_class("promptlookup")
+
+
+def test_tensor_api_and_shape_errors():
+    mpk = _host_mpk()
+    x = _t(mpk, "x", 4, 1024)
+    assert x.num_dims == 2 and x.dim(0) == 4 and x.dim(1) == 1024
+    with pytest.raises(AssertionError):  # row-major only (persistent_kernel.py:473-474)
+        mpk.attach_input(torch.zeros(8, 4, dtype=torch.bfloat16).t(), "xt")
+    with pytest.raises(RuntimeError, match="Invalid io_category"):
+        mpk.new_tensor((4, 8), name="bad", io_category="host_tensor")
+    q, k, v = _t(mpk, "q", 1024, 1024), _t(mpk, "k", 256, 1024), _t(mpk, "v", 256, 1024)
+    qkv = mpk.shuffle_tensors([q, k, v], 0, 2, "qkv")
+    assert qkv.dim(0) == 1536 and qkv.dim(1) == 1024
+    with pytest.raises(_capi.MkError, match="not divisible"):
+        mpk.shuffle_tensors([q, k, v], 0, 3, "qkv3")
+    with pytest.raises(AssertionError):
+        mpk.shuffle_tensors([q, k], 1, 2, "dim1")
+    # unknown task names are rejected when registered, like Graph::register_task (src/kernel/graph.cc:844-847)
+    with pytest.raises(_capi.MkError, match="Unsupported task name"):
+        mpk._task("definitely_not_a_task", (1, 1, 1), (128, 1, 1), [(x, (-1, -1, -1), -1)])
+    with pytest.raises(NotImplementedError):
+        mpk.allreduce_layer()
+
+
+def test_lowering_fuses_norm_and_swiglu_and_attention():
+    mpk = _host_mpk(B=4, R=2)
+    H, I, nq, nkv, D = 1024, 1536, 8, 2, 128
+    ids = _t(mpk, "ids", 4, 1, dtype=torch.int64)
+    emb, x = _t(mpk, "emb", 100, H), mpk.new_tensor((4, H), name="x")
+    nw, n = _t(mpk, "nw", H), mpk.new_tensor((4, H), name="n")
+    q, k, v = _t(mpk, "q", nq * D, H), _t(mpk, "k", nkv * D, H), _t(mpk, "v", nkv * D, H)
+    qkv_w = mpk.shuffle_tensors([q, k, v], 0, nkv, "qkv_w")
+    qkv = mpk.new_tensor((4, (nq + 2 * nkv) * D), name="qkv")
+    kc, vc = _t(mpk, "kc", 8, 16, nkv, D), _t(mpk, "vc", 8, 16, nkv, D)
+    qn, kn = _t(mpk, "qn", D), _t(mpk, "kn", D)
+    cos, sin = _t(mpk, "cos", 64, D), _t(mpk, "sin", 64, D)
+    qws, att, lse = mpk.new_tensor((4, nq * D), name="qws"), mpk.new_tensor((4, nq * D), name="att"), mpk.new_tensor((4, nq), dtype=mi.float32, name="lse")
+    wo, x1 = _t(mpk, "wo", H, nq * D), mpk.new_tensor((4, H), name="x1")
+    wg, wu = _t(mpk, "wg", I, H), _t(mpk, "wu", I, H)
+    gu = mpk.shuffle_tensors([wg, wu], 0, I // 128, "gu")
+    mid, act = mpk.new_tensor((4, 2 * I), name="mid"), mpk.new_tensor((4, I), name="act")
+    wd, x2 = _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="x2")
+    lm, logits = _t(mpk, "lm", 1000, H), mpk.new_tensor((4, 1000), name="logits")
+    pv, pi = mpk.new_tensor((4, 8), name="pv"), mpk.new_tensor((4, 8), dtype=mi.int64, name="pi")
+    out = _t(mpk, "out", 4, 1, dtype=torch.int64)
+    mpk.embed_layer(input=ids, weight=emb, output=x, grid_dim=(1, 1, 1), block_dim=(128, 1, 1), input_source=1)
+    mpk.rmsnorm_layer(input=x, weight=nw, output=n, grid_dim=(4, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_layer(input=n, weight=qkv_w, output=qkv, grid_dim=(24, 1, 1), block_dim=(128, 1, 1))
+    mpk.kv_cache_update_layer(input=qkv, k_cache=kc, v_cache=vc, q_norm=qn, k_norm=kn, cos_pos_embed=cos, sin_pos_embed=sin, q_workspace=qws,
+                              grid_dim=(2, nkv, 1), block_dim=(256, 1, 1))
+    mpk.paged_attention_ck_fmha_layer(q_workspace=qws, k_cache=kc, v_cache=vc, o_acc=att, lse_acc=lse, attention_params=(nq, 1, 2),
+                                      grid_dim=(2, nkv, 1), block_dim=(256, 1, 1))
+    mpk.linear_with_residual_layer(input=att, weight=wo, residual=x, output=x1, grid_dim=(16, 1, 1), block_dim=(256, 1, 1))
+    mpk.rmsnorm_layer(input=x1, weight=nw, output=n, grid_dim=(4, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_layer(input=n, weight=gu, output=mid, grid_dim=(48, 1, 1), block_dim=(128, 1, 1))
+    mpk.silu_mul_layer(input=mid, output=act, grid_dim=(I // 128, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_with_residual_layer(input=act, weight=wd, residual=x1, output=x2, grid_dim=(16, 1, 1), block_dim=(256, 1, 1))
+    mpk.rmsnorm_layer(input=x2, weight=nw, output=n, grid_dim=(4, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_layer(input=n, weight=lm, output=logits, grid_dim=(8, 1, 1), block_dim=(128, 1, 1))
+    mpk.argmax_partial_layer(input=logits, output=(pv, pi), grid_dim=(8, 1, 1), block_dim=(128, 1, 1))
+    mpk.argmax_reduce_layer(input=(pv, pi), output=out, grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
+    prog = [l.split(None, 1)[1] for l in mpk.describe_program().splitlines()]
+    kinds = [l.split()[0] for l in prog]
+    assert kinds == ["EMBED", "NORM[multi-token", "LINEAR+norm", "ATTN", "LINEAR+res", "NORM[multi-token", "LINEAR+norm+silu", "LINEAR+res",
+                     "NORM[multi-token", "LINEAR+norm", "ARGMAX_PARTIAL", "ARGMAX_REDUCE"]
+    assert "segs=3" in prog[2] and "segs=2" in prog[6] and "-> act" in prog[6]  # shuffled views resolved, activation folded in
+    # reference-shaped task graph: tasks = 2 + sum of grid sizes; first/last events as in runtime.cc:176-182,590-595
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    n_tasks = 2 + 1 + 4 + 24 + 4 + 4 + 16 + 4 + 48 + 12 + 16 + 4 + 8 + 8 + 1
+    assert len(tg["all_tasks"]) == n_tasks
+    assert tg["all_tasks"][0]["task_type"] == 0 and tg["all_tasks"][1]["task_type"] == 10
+    assert tg["all_events"][0]["event_type"] == 911 and tg["all_events"][1]["event_type"] == 903 and tg["all_events"][-1]["event_type"] == 910
+    assert tg["all_events"][1]["first_task_id"] == 2 and tg["all_events"][1]["last_task_id"] == n_tasks
+    lin = [t for t in tg["all_tasks"] if t["task_type"] == 120]
+    assert lin[1]["inputs"][1]["base_ptr"] == "qkv_w" and lin[1]["inputs"][1]["dims"] == [64, 1024]  # 1536 rows over 24 blocks
+    assert lin[1]["inputs"][1]["offset"] == 64 * 1024 * 2 and lin[1]["outputs"][0]["offset"] == 64 * 2
+    for key in ("trigger_event", "dependent_event", "request_id", "expert_offset", "kv_idx", "merge_task_offset", "n_tile_start", "n_tile_count"):
+        assert key in lin[0]
+    with pytest.raises(_capi.MkError, match="one GPU"):
+        mpk.kn_graph.generate_task_graph(2, 1)
+    with pytest.raises(_capi.MkError, match="without a device"):
+        mpk.compile()
+
+
+def test_lowering_rejects_bad_graphs():
+    mpk = _host_mpk()
+    x, W = _t(mpk, "x", 4, 1024), _t(mpk, "W", 512, 1000)
+    y = mpk.new_tensor((4, 512), name="y")
+    mpk.linear_layer(input=x, weight=W, output=y, grid_dim=(8, 1, 1), block_dim=(128, 1, 1))
+    with pytest.raises(_capi.MkError, match="expected 1024"):
+        mpk.describe_program()
+    mpk2 = _host_mpk()
+    x, W = _t(mpk2, "x", 2, 1024), _t(mpk2, "W", 512, 1024)  # fewer rows than max_num_batched_tokens
+    y = mpk2.new_tensor((4, 512), name="y")
+    mpk2.linear_layer(input=x, weight=W, output=y, grid_dim=(8, 1, 1), block_dim=(128, 1, 1))
+    with pytest.raises(_capi.MkError, match="max_num_batched_tokens"):
+        mpk2.describe_program()
+    mpk3 = _host_mpk()
+    qkv = _t(mpk3, "qkv", 4, 12 * 64)
+    kc, vc = _t(mpk3, "kc", 8, 16, 2, 64), _t(mpk3, "vc", 8, 16, 2, 64)
+    o, lse, qws = mpk3.new_tensor((4, 512), name="o"), mpk3.new_tensor((4, 8), dtype=mi.float32, name="lse"), mpk3.new_tensor((4, 512), name="qws")
+    mpk3.gang_paged_attention_split_kv_layer(input=qkv, k_cache=kc, v_cache=vc, q_norm=None, k_norm=None, cos_pos_embed=None, sin_pos_embed=None,
+                                             lse=lse, output=o, q_workspace=qws, attention_params=(8, 1, 512))
+    with pytest.raises(_capi.MkError, match="head_dim 64"):
+        mpk3.describe_program()
+    mpk4 = _host_mpk()
+    with pytest.raises(AssertionError, match="divisible"):  # gang layers need N divisible by 8 * tile_n (persistent_kernel.py:1595-1599)
+        mpk4.gang_linear_layer(input=_t(mpk4, "x", 4, 1024), weight=_t(mpk4, "W", 1000, 1024), output=mpk4.new_tensor((4, 1000), name="y"),
+                               tile_n=64, output_stride=1000)
