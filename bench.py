@@ -89,6 +89,7 @@ def main():
     ap.add_argument("--prompt-length", type=int, default=80)
     ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true", help="also run one 1 GiB device-to-device copy (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the decode megakernel on ONE GPU; --gpus must be 1 "
@@ -106,6 +107,12 @@ def main():
     shape = Qwen3Shape(num_layers=args.layers)
     B, K, W, P = args.batch, args.steps, args.warmup, args.prompt_length
     max_seq = max(1200, P + W + K + 2)
+    if args.calib_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
     weights = random_weights(shape, seed=0)
     dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
     prompts = [torch.randint(0, shape.vocab_size, (P,), generator=torch.Generator().manual_seed(r)) for r in range(B)]
@@ -149,9 +156,12 @@ def main():
                      "traffic": None, "kernel": "mk_persistent_kernel", "kernel_ms_per_launch": round(kernel_ms, 3),
                      "algorithmic_bytes_per_launch": bytes_total},
     }
+    dec.mpk.finalize()
+    del dec, weights
+    torch.cuda.synchronize()
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(shape)
-    print(json.dumps(out))
+    print(json.dumps(out), flush=True)
 
 
 if __name__ == "__main__":

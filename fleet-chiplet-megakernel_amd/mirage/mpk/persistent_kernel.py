@@ -548,6 +548,9 @@ class PersistentKernel:
         self.__finalized__ = True
 
     def __del__(self):
+        import sys
+        if sys.is_finalizing():  # the HIP runtime may already be gone at interpreter shutdown: leave the memory to the OS
+            return
         try:
             if not self.__finalized__:
                 self.finalize()
