@@ -23,11 +23,12 @@ HIPCC_FLAGS = [
 ]
 
 
-def build(verbose: bool = True) -> str:
+def build(verbose: bool = True, defines=(), out: str = None) -> str:
     hipcc = shutil.which("hipcc") or "/opt/rocm/bin/hipcc"
     if not os.path.exists(hipcc):
         raise RuntimeError("hipcc not found: the megakernel library cannot be built")
-    cmd = [hipcc] + HIPCC_FLAGS + [os.path.join(CSRC, "fleet_mk.hip"), "-o", LIB]
+    lib = out or LIB
+    cmd = [hipcc] + HIPCC_FLAGS + ["-D" + d for d in defines] + [os.path.join(CSRC, "fleet_mk.hip"), "-o", lib]
     if verbose:
         print(" ".join(cmd), flush=True)
     res = subprocess.run(cmd, cwd=CSRC, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
@@ -36,7 +37,7 @@ def build(verbose: bool = True) -> str:
         raise RuntimeError("hipcc failed:\n" + out)
     if verbose and out.strip():
         print(out)
-    return LIB
+    return lib
 
 
 if __name__ == "__main__":

@@ -19,15 +19,28 @@ typedef float f32x4 __attribute__((ext_vector_type(4)));
 
 #define MK_SPIN_LIMIT (1u << 24)
 
+// prefetch depth of the single-token linear: LDS ring bytes per workgroup and register rows per worker wavefront
+#ifndef MK_TUNE_PF_BYTES
+#define MK_TUNE_PF_BYTES 0  // measured: the ring does not pay once the poll sits on the control wavefront
+#endif
+#ifndef MK_TUNE_R8
+#define MK_TUNE_R8 4
+#endif
+#ifndef MK_TUNE_R24
+#define MK_TUNE_R24 2
+#endif
+
 struct Ctx {
   int vid;   // virtual workgroup id: xcd-major, so vids [x*quota, (x+1)*quota) share an L2
   int G;     // workgroups in the grid
   int xcd;   // XCC_ID of the CU this workgroup landed on
   int quota; // workgroups on this XCD
   int nxcd;  // XCDs that received at least one workgroup
+  unsigned quotas[8];  // workgroups on each of the first 8 XCD ids (0 = unused)
+  int xi;     // index of this XCD among the XCDs in use
+  int rank;   // rank of this workgroup inside its XCD
   unsigned epoch;
   bool pending;  // an arrive has been posted that no wait has consumed yet
-  bool leader;   // (thread 0 only) this workgroup was the last of its XCD to arrive
   bool dead;     // the watchdog fired somewhere: unwind
   long long t_wait;  // (profiling) tick at which the last barrier_wait completed
   int *sh_dead;
@@ -65,7 +78,7 @@ __device__ __forceinline__ float group16_sum(float v) {
 }
 __device__ __forceinline__ unsigned xcc_id() {
   // HW_REG_XCC_ID (id 20), bits [3:0]
-  return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 15u;
+  return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 7u;  // MI355X: 8 XCDs
 }
 __device__ __forceinline__ u32x4 ldg_stream(const u32x4 *p) { return __builtin_nontemporal_load(p); }
 
@@ -93,10 +106,9 @@ __device__ __forceinline__ uint16_t ldc_u16(const uint16_t *p) {
 }
 
 // ----------------------------------------------------------------------------- grid barrier
-// Two-level barrier: workgroups of one XCD count arrivals in a counter that lives in that XCD's
-// L2; the last arriver of each XCD publishes one cross-XCD signal and waits for the other dies,
-// then releases its own die through an L2-local flag.  Replaces the reference's per-event
-// two-level counters (persistent_kernel.cuh:1214-1284).
+// Stage barrier with one arrival counter per XCD (each in its own 128-byte line, so a die's arrivals meet in that
+// die's L2 and only completed lines travel between dies).  Replaces the reference's per-event two-level counters
+// (persistent_kernel.cuh:1214-1284).
 __device__ __forceinline__ bool spin_ok(MkSync *s, unsigned &spins, unsigned where) {
   ++spins;
   if ((spins & 1023u) == 0) {
@@ -110,42 +122,34 @@ __device__ __forceinline__ bool spin_ok(MkSync *s, unsigned &spins, unsigned whe
   return true;
 }
 
-// arrive: this workgroup's outputs of the current stage are complete.  The last arriver of an XCD becomes
-// that XCD's leader for this epoch: it writes the die's L2 back (release) and posts the cross-XCD signal.
+// arrive: this workgroup's outputs of the current stage are complete: write them back (agent-scope release) and
+// count the arrival in the counter of this workgroup's XCD (one 128-byte line per die, so the 32 arrivals of a die meet
+// in that die's L2).  Nothing is returned, so nobody waits on the atomic.
 __device__ __forceinline__ void barrier_arrive(Ctx &c) {
   MkSync *s = c.sync;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   __syncthreads();
   c.epoch++;
-  if (threadIdx.x == 0) {
-    const unsigned old = __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    c.leader = (old + 1 == (unsigned)c.quota * c.epoch);
-    if (c.leader) __hip_atomic_fetch_add(&s->global_ctr, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-  }
+  if (threadIdx.x == 0) __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
   c.pending = true;
 }
 
-// wait: every workgroup of the grid has arrived at the current epoch.  Leaders poll the global counter and then
-// raise their die's flag; everyone else polls that flag with a compare-and-swap that never succeeds (it executes in
-// the L2, is never served from the CU's L1, and cannot be folded into a plain load by the compiler).
+// poll (thread 0 only): the barrier is complete when every die's counter has reached quota x epoch.  The eight
+// counters are read with independent device-scope loads (one round trip per poll), so completion is seen two hops
+// after the last arrival (atomic -> load) instead of going through a leader and a broadcast flag.
 __device__ __forceinline__ void barrier_poll(Ctx &c) {
-  // thread 0 only; the caller must follow with a workgroup barrier and barrier_done()
   MkSync *s = c.sync;
   const unsigned epoch = c.epoch;
   unsigned spins = 0;
-  if (c.leader) {
-    while (__hip_atomic_load(&s->global_ctr, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)c.nxcd * epoch &&
-           spin_ok(s, spins, epoch))
-      __builtin_amdgcn_s_sleep(1);
-    __hip_atomic_fetch_max(&s->local_flag[c.xcd][0], epoch, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-  } else {
-    while (true) {
-      unsigned expect = 0xFFFFFFFFu;
-      __hip_atomic_compare_exchange_strong(&s->local_flag[c.xcd][0], &expect, 0xFFFFFFFFu, __ATOMIC_RELAXED,
-                                           __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-      if (expect >= epoch || !spin_ok(s, spins, epoch)) break;
-      __builtin_amdgcn_s_sleep(1);
-    }
+  while (true) {
+    unsigned v[8];
+#pragma unroll
+    for (int x = 0; x < 8; x++) v[x] = __hip_atomic_load(&s->local_ctr[x][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    bool ok = true;
+#pragma unroll
+    for (int x = 0; x < 8; x++) ok = ok && (v[x] >= c.quotas[x] * epoch);
+    if (ok || !spin_ok(s, spins, epoch)) break;
+    __builtin_amdgcn_s_sleep(1);
   }
   *c.sh_dead = (spins >= 1024u) ? (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
 }
@@ -295,7 +299,7 @@ __device__ __forceinline__ const u32x4 *weight_row(const MkWeight &w, int r, int
 // stage (weight prefetch), and the main loop posts barrier_arrive(c) when the function returns.
 
 // Gather embedding rows.  Reference task: tasks/ampere/embedding.cuh:42-72.
-__device__ void stage_embed(const MkStage &st, Ctx &c, const MkRuntime &rt, int M) {
+__device__ __forceinline__ void stage_embed(const MkStage &st, Ctx &c, const MkRuntime &rt, int M) {
   barrier_wait(c);
   const int k8 = st.k / 8;
   for (int t = c.vid; t < M; t += c.G) {
@@ -325,7 +329,7 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 // RMSNorm of full rows, one workgroup per token row (used when an iteration has several tokens;
 // single-token iterations fuse the norm into the consuming linear).  y = bf16((x * r) * w) with
 // r = rsqrt(mean(x^2) + eps) in fp32.  Reference task: tasks/mi300/rmsnorm_mi300.cuh:37-188.
-__device__ void stage_norm(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_norm(const MkStage &st, Ctx &c, int M, char *smem) {
   barrier_wait(c);
   float *red = (float *)smem;
   uint32_t *xs = (uint32_t *)(smem + 1024);
@@ -435,11 +439,11 @@ __device__ __forceinline__ void stage_x_m1_wave(const MkStage &st, const Ctx &c,
 // Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:359-576).
 template <int KL, int R, bool SILU>
-__device__ void stage_linear_m1_t(const MkStage &st, Ctx &c, char *smem) {
+__device__ __forceinline__ void stage_linear_m1_t(const MkStage &st, Ctx &c, char *smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   constexpr int K8 = KL * 64;
   constexpr int NW = MK_WAVES - 1;                         // worker wavefronts
-  constexpr int PF_BYTES = (MK_PF_BYTES / NW) & ~1023;     // LDS ring per worker
+  constexpr int PF_BYTES = (MK_TUNE_PF_BYTES / NW) & ~1023;  // LDS ring per worker (0 = ring disabled)
   constexpr int NPF = PF_BYTES / (KL * 1024);              // rows per worker prefetched straight into LDS
   uint32_t *xs = (uint32_t *)smem;
   const bool ctrl = wave == 0;
@@ -556,7 +560,7 @@ __device__ void stage_linear_m1_t(const MkStage &st, Ctx &c, char *smem) {
 
 // Generic single-token linear for reduction lengths that are not a multiple of 512 or have no tuned
 // instantiation: same arithmetic, no cross-barrier prefetch.
-__device__ void stage_linear_m1_generic(const MkStage &st, Ctx &c, char *smem) {
+__device__ __forceinline__ void stage_linear_m1_generic(const MkStage &st, Ctx &c, char *smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
   const int K = st.k, k8 = K / 8;
   uint32_t *xs = (uint32_t *)smem;
@@ -599,13 +603,13 @@ __device__ void stage_linear_m1_generic(const MkStage &st, Ctx &c, char *smem) {
   }
 }
 
-__device__ void stage_linear_m1(const MkStage &st, Ctx &c, char *smem) {
+__device__ __forceinline__ void stage_linear_m1(const MkStage &st, Ctx &c, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
   if (st.k == 4096) {
-    if (silu) stage_linear_m1_t<8, 4, true>(st, c, smem);
-    else stage_linear_m1_t<8, 4, false>(st, c, smem);
+    if (silu) stage_linear_m1_t<8, MK_TUNE_R8, true>(st, c, smem);
+    else stage_linear_m1_t<8, MK_TUNE_R8, false>(st, c, smem);
   } else if (st.k == 12288 && !silu) {
-    stage_linear_m1_t<24, 2, false>(st, c, smem);
+    stage_linear_m1_t<24, MK_TUNE_R24, false>(st, c, smem);
   } else if (st.k == 2048) {
     if (silu) stage_linear_m1_t<4, 4, true>(st, c, smem);
     else stage_linear_m1_t<4, 4, false>(st, c, smem);
@@ -625,7 +629,7 @@ __device__ void stage_linear_m1(const MkStage &st, Ctx &c, char *smem) {
 // Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
 template <int MT>
-__device__ void stage_linear_mfma(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_linear_mfma(const MkStage &st, Ctx &c, int M, char *smem) {
   constexpr int TG = 6;  // weight tiles per K sweep
   barrier_wait(c);
   // activations were produced by other workgroups: invalidate this CU's L1 once, then use cached loads so the rows
@@ -730,7 +734,7 @@ __device__ void stage_linear_mfma(const MkStage &st, Ctx &c, int M, char *smem) 
 
 // Standalone SwiGLU over interleaved [gate ; up] groups (used when the graph keeps the
 // gate/up linear and the activation apart).  Reference task: tasks/mi300/silu_mul_mi300.cuh:42-184.
-__device__ void stage_silu_mul(const MkStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_silu_mul(const MkStage &st, Ctx &c, int M) {
   barrier_wait(c);
   const int n = st.n, half = st.silu_half;
   const uint16_t *in = (const uint16_t *)st.in;
@@ -777,7 +781,7 @@ __device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst
 // paged_attention_minimal_decode (tasks/mi300/paged_attention_decode_minimal_mi300.cuh:100-371),
 // gang_attention_split_kv_kernel (tasks/mi300/gang_attention_mi300.cuh:49-153).
 template <int QPK>
-__device__ void stage_attn(const MkStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
+__device__ __forceinline__ void stage_attn(const MkStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
   barrier_wait(c);
   constexpr int D = 128;
   const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
@@ -964,7 +968,7 @@ __device__ void stage_attn(const MkStage &st, Ctx &c, const MkRuntime &rt, int M
 
 // Greedy sampling, stage 1: every workgroup scans a contiguous slice of each token's logits and keeps
 // (max, lowest index attaining it).  Reference task: tasks/mi300/argmax_mi300.cuh:78-127.
-__device__ void stage_argmax_partial(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_argmax_partial(const MkStage &st, Ctx &c, int M, char *smem) {
   barrier_wait(c);
   float *sv = (float *)smem;
   int *si = (int *)(smem + 1024);
@@ -1020,7 +1024,7 @@ __device__ void stage_argmax_partial(const MkStage &st, Ctx &c, int M, char *sme
 
 // Greedy sampling, stage 2: one wavefront per token reduces the per-workgroup partials.
 // Reference task: tasks/mi300/argmax_mi300.cuh:129-158.
-__device__ void stage_argmax_reduce(const MkStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_argmax_reduce(const MkStage &st, Ctx &c, int M) {
   barrier_wait(c);
   const float *pv = (const float *)st.aux0;
   const int *pi = (const int *)st.aux1;
@@ -1055,6 +1059,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
                                                                                 int run_scheduler) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int sh_bcast[4];
+  __shared__ int sh_quota[10];
   const MkRuntime rt = *rtp;
   Ctx c;
   c.G = gridDim.x;
@@ -1062,7 +1067,6 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.xcd = xcc_id();
   c.epoch = 0;
   c.pending = false;
-  c.leader = false;
   c.dead = false;
   c.t_wait = 0;
   c.sh_dead = &sh_bcast[3];
@@ -1074,12 +1078,18 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     unsigned spins = 0;
     while (__hip_atomic_load(&s->init_ctr, __ATOMIC_ACQUIRE, __HIP_MEMORY_SCOPE_AGENT) < (unsigned)c.G && spin_ok(s, spins, 0xFFFF0000u))
       __builtin_amdgcn_s_sleep(1);
-    int nx = 0, before = 0;
+    int nx = 0, before = 0, xi = 0;
     for (int i = 0; i < MK_MAX_XCD; i++) {
       const unsigned n = __hip_atomic_load(&s->xcd_count[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       nx += n > 0;
-      if (i < c.xcd) before += (int)n;
+      if (i < c.xcd) {
+        before += (int)n;
+        xi += n > 0;
+      }
     }
+    sh_quota[8] = xi;
+    sh_quota[9] = (int)rank;
+    for (int i = 0; i < 8; i++) sh_quota[i] = (int)__hip_atomic_load(&s->xcd_count[i], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     sh_bcast[0] = before + (int)rank;
     sh_bcast[1] = nx;
     sh_bcast[2] = (int)__hip_atomic_load(&s->xcd_count[c.xcd], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -1090,6 +1100,9 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.nxcd = sh_bcast[1];
   c.quota = sh_bcast[2];
   c.dead = sh_bcast[3] != 0;
+  for (int i = 0; i < 8; i++) c.quotas[i] = (unsigned)sh_quota[i];
+  c.xi = sh_quota[8];
+  c.rank = sh_quota[9];
   __syncthreads();
 
   for (int it = 0; it < max_iters && !c.dead; it++) {

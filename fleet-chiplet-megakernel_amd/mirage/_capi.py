@@ -8,7 +8,8 @@ import ctypes
 import os
 
 _HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(os.path.dirname(_HERE), "libfleet_mk.so")
+# FLEET_MK_LIB selects another build of the same library (used to compare tuning variants)
+LIB_PATH = os.environ.get("FLEET_MK_LIB") or os.path.join(os.path.dirname(_HERE), "libfleet_mk.so")
 
 MK_OK = 0
 MK_EINVAL = -1
