@@ -389,6 +389,178 @@ int lower_attention(mk_graph *g, size_t &i) {
   return MK_OK;
 }
 
+
+bool is_moe_linear(const std::string &n) {
+  return n == "moe_w13_linear_mi300" || n == "moe_w2_linear_mi300" || n == "gang_moe_w13_linear_mi300" || n == "gang_moe_w2_linear_mi300";
+}
+
+// dims 0 and 1 of a [tokens, topk, width] tensor must form one contiguous run of rows
+bool rows_contiguous_3d(const Tensor &t) { return t.ndims == 3 && t.strides[2] == 1 && t.strides[0] == t.dims[1] * t.strides[1]; }
+
+// Router: moe_topk_softmax_mi300 [logits, topk_weight, routing_indices, mask].  When the per-expert linear that consumes
+// the routing follows directly, single-token iterations route inside that linear and this stage runs for multi-token
+// iterations only.
+int lower_moe_topk(mk_graph *g, size_t &i, bool *inline_next) {
+  const Task &t = g->tasks[i];
+  if (t.ops.size() != 4) return fail(MK_EINVAL, "%s expects 4 operands", t.name.c_str());
+  const Tensor &lg = g->tensors[t.ops[0]], &tw = g->tensors[t.ops[1]], &ri = g->tensors[t.ops[2]], &mk = g->tensors[t.ops[3]];
+  const int B = g->cfg.max_num_batched_tokens;
+  if (lg.ndims != 2 || lg.dtype != MK_DT_BF16 || lg.dims[0] < B) return fail(MK_EINVAL, "%s: logits must be [tokens, experts] bf16", t.name.c_str());
+  const int E = (int)lg.dims[1];
+  if (E < 1 || E > MK_MOE_MAX_EXPERTS) return fail(MK_EUNSUPPORTED, "%s: %d experts (max %d)", t.name.c_str(), E, MK_MOE_MAX_EXPERTS);
+  if (tw.ndims != 2 || tw.dtype != MK_DT_F32 || tw.dims[0] < B || tw.strides[1] != 1) return fail(MK_EINVAL, "%s: routing weights must be [tokens, topk] fp32", t.name.c_str());
+  const int topk = (int)tw.dims[1];
+  if (topk < 1 || topk > MK_MOE_MAX_TOPK || topk > E) return fail(MK_EUNSUPPORTED, "%s: top-%d of %d experts (max %d)", t.name.c_str(), topk, E, MK_MOE_MAX_TOPK);
+  if (ri.ndims != 2 || ri.dtype != MK_DT_I32 || ri.dims[0] != E || ri.dims[1] < B || ri.strides[1] != 1)
+    return fail(MK_EINVAL, "%s: routing indices must be [experts, tokens] int32", t.name.c_str());
+  if (mk.dtype != MK_DT_I32 || mk.elems() < (size_t)E + 1) return fail(MK_EINVAL, "%s: mask must hold experts+1 int32", t.name.c_str());
+  if (i + 1 >= g->tasks.size() || !is_moe_linear(g->tasks[i + 1].name) || g->tasks[i + 1].ops.size() != 5 || g->tasks[i + 1].ops[2] != t.ops[2] ||
+      g->tasks[i + 1].ops[3] != t.ops[3])
+    return fail(MK_EUNSUPPORTED, "%s must be followed by the per-expert linear that consumes its routing table (it publishes the active-expert mask)", t.name.c_str());
+  *inline_next = g->tensors[g->tasks[i + 1].ops[0]].ndims == 2;
+  MkStage st;
+  memset(&st, 0, sizeof(st));
+  st.op = MK_OP_MOE_TOPK;
+  if (*inline_next) st.flags |= MK_F_ONLY_MULTI;
+  st.moe_logits = lg.ptr;
+  st.ld_logits = (int)lg.strides[0];
+  st.moe_topk_w = (float *)tw.ptr;
+  st.ld_topk_w = (int)tw.strides[0];
+  st.moe_routing = (int *)ri.ptr;
+  st.ld_routing = (int)ri.strides[0];
+  st.moe_mask = (int *)mk.ptr;
+  st.num_experts = E;
+  st.topk = topk;
+  g->stages.push_back(st);
+  g->stage_desc.push_back(fmt("MOE_TOPK%s %s -> %s,%s experts=%d topk=%d", *inline_next ? "[multi-token only]" : "", lg.name.c_str(), tw.name.c_str(), ri.name.c_str(), E, topk));
+  i++;
+  return MK_OK;
+}
+
+// Per-expert linear [input, weight[E,N,K], routing_indices, mask, output[tokens,topk,N]]; input is [tokens, K] (every
+// slot of a token sees the same row: W13) or [tokens, topk, K] (W2).  A directly following moe_silu_mul / moe_mul_sum_add
+// over its output becomes the epilogue.
+int lower_moe_linear(mk_graph *g, size_t &i, const MkStage *router) {
+  const Task &t = g->tasks[i];
+  if (t.ops.size() != 5) return fail(MK_EINVAL, "%s expects 5 operands", t.name.c_str());
+  const Tensor &x = g->tensors[t.ops[0]], &w = g->tensors[t.ops[1]], &ri = g->tensors[t.ops[2]], &mk = g->tensors[t.ops[3]], &y = g->tensors[t.ops[4]];
+  const int B = g->cfg.max_num_batched_tokens;
+  if (w.ndims != 3 || w.dtype != MK_DT_BF16 || !w.ptr || w.strides[2] != 1 || w.strides[1] != w.dims[2] || w.strides[0] != w.dims[1] * w.dims[2])
+    return fail(MK_EINVAL, "%s: weight '%s' must be a contiguous [experts, rows, k] bf16 tensor", t.name.c_str(), w.name.c_str());
+  const int E = (int)w.dims[0], N = (int)w.dims[1], K = (int)w.dims[2];
+  if (E > MK_MOE_MAX_EXPERTS) return fail(MK_EUNSUPPORTED, "%s: %d experts (max %d)", t.name.c_str(), E, MK_MOE_MAX_EXPERTS);
+  if (K % 8 || K > 4096) return fail(MK_EUNSUPPORTED, "%s: k=%d must be a multiple of 8 and at most 4096", t.name.c_str(), K);
+  if (ri.ndims != 2 || ri.dtype != MK_DT_I32 || ri.dims[0] != E || ri.dims[1] < B || ri.strides[1] != 1)
+    return fail(MK_EINVAL, "%s: routing indices must be [experts, tokens] int32", t.name.c_str());
+  if (mk.dtype != MK_DT_I32 || mk.elems() < (size_t)E + 1) return fail(MK_EINVAL, "%s: mask must hold experts+1 int32", t.name.c_str());
+  if (!rows_contiguous_3d(y) || y.dtype != MK_DT_BF16 || y.dims[0] < B || y.dims[2] < N) return fail(MK_EINVAL, "%s: output must be [tokens, topk, %d] bf16", t.name.c_str(), N);
+  const int topk = (int)y.dims[1];
+  if (topk < 1 || topk > MK_MOE_MAX_TOPK) return fail(MK_EUNSUPPORTED, "%s: topk=%d (max %d)", t.name.c_str(), topk, MK_MOE_MAX_TOPK);
+  MkStage st;
+  memset(&st, 0, sizeof(st));
+  st.op = MK_OP_MOE_LINEAR;
+  st.n = N;
+  st.k = K;
+  st.num_experts = E;
+  st.topk = topk;
+  st.w.nseg = 1;
+  st.w.seg[0] = w.ptr;
+  st.w.seg_rows[0] = st.w.group_rows = E * N;
+  st.moe_routing = (int *)ri.ptr;
+  st.ld_routing = (int)ri.strides[0];
+  st.moe_mask = (int *)mk.ptr;
+  st.in = x.ptr;
+  if (x.dtype != MK_DT_BF16 || x.dims[0] < B) return fail(MK_EINVAL, "%s: input must be bf16 with at least %d token rows", t.name.c_str(), B);
+  if (x.ndims == 2) {
+    if (x.dims[1] != K || x.strides[1] != 1) return fail(MK_EINVAL, "%s: input must be [tokens, %d]", t.name.c_str(), K);
+    st.ld_in = (int)x.strides[0];
+  } else if (x.ndims == 3) {
+    if (x.dims[1] != topk || x.dims[2] != K || x.strides[2] != 1) return fail(MK_EINVAL, "%s: input must be [tokens, %d, %d]", t.name.c_str(), topk, K);
+    st.ld_in = (int)x.strides[0];
+    st.ld_in_slot = (int)x.strides[1];
+  } else {
+    return fail(MK_EINVAL, "%s: input must be 2-D or 3-D", t.name.c_str());
+  }
+  if ((st.ld_in % 8) || (st.ld_in_slot % 8)) return fail(MK_EINVAL, "%s: input rows must be 16-byte aligned", t.name.c_str());
+  st.out = y.ptr;
+  st.ld_out = (int)y.strides[0];
+  st.ld_out_slot = (int)y.strides[1];
+  if (router) {
+    st.flags |= MK_F_MOE_INLINE_TOPK;
+    st.moe_logits = router->moe_logits;
+    st.ld_logits = router->ld_logits;
+    st.moe_topk_w = router->moe_topk_w;
+    st.ld_topk_w = router->ld_topk_w;
+    if (router->topk != topk || router->num_experts != E) return fail(MK_EINVAL, "%s: router has %d experts / top-%d, linear has %d / %d", t.name.c_str(), router->num_experts, router->topk, E, topk);
+  }
+  size_t consumed = 1;
+  std::string extra;
+  const Task *nx = i + 1 < g->tasks.size() ? &g->tasks[i + 1] : nullptr;
+  if (nx && nx->name == "moe_silu_mul" && nx->ops.size() == 2 && nx->ops[0] == t.ops[4] && N % 2 == 0) {
+    const Tensor &o = g->tensors[nx->ops[1]];
+    if (!rows_contiguous_3d(o) || o.dtype != MK_DT_BF16 || o.dims[0] < B || o.dims[1] != topk || o.dims[2] != N / 2)
+      return fail(MK_EINVAL, "moe_silu_mul: output must be [tokens, %d, %d] bf16", topk, N / 2);
+    st.flags |= MK_F_SILU;
+    st.out2 = o.ptr;
+    st.ld_out2 = (int)o.strides[0];
+    st.ld_out2_slot = (int)o.strides[1];
+    consumed = 2;
+    extra = "+silu -> " + o.name;
+  } else if (nx && nx->name == "moe_mul_sum_add_mi300" && nx->ops.size() == 4 && nx->ops[0] == t.ops[4] && x.ndims == 3) {
+    // fused for single-token iterations; the combine stage emitted by lower_moe_combine covers the others
+    const Tensor &tw = g->tensors[nx->ops[1]], &r = g->tensors[nx->ops[2]], &o = g->tensors[nx->ops[3]];
+    if (tw.ndims != 2 || tw.dtype != MK_DT_F32 || tw.dims[1] != topk || tw.strides[1] != 1 || r.ndims != 2 || o.ndims != 2 || r.dims[1] < N || o.dims[1] < N ||
+        r.dtype != MK_DT_BF16 || o.dtype != MK_DT_BF16)
+      return fail(MK_EINVAL, "moe_mul_sum_add_mi300: shapes do not match the expert outputs");
+    st.flags |= MK_F_MOE_COMBINE;
+    st.moe_topk_w = (float *)tw.ptr;
+    st.ld_topk_w = (int)tw.strides[0];
+    st.res = r.ptr;
+    st.ld_res = (int)r.strides[0];
+    st.out2 = o.ptr;
+    st.ld_out2 = (int)o.strides[0];
+    extra = "+combine(single token) -> " + o.name;
+  }
+  g->stages.push_back(st);
+  g->stage_desc.push_back(fmt("MOE_LINEAR%s %s x %s -> %s experts=%d topk=%d n=%d k=%d%s", router ? "+route(single token)" : "", x.name.c_str(), w.name.c_str(), y.name.c_str(), E,
+                              topk, N, K, extra.c_str()));
+  g->weight_bytes += (int64_t)topk * N * K * 2;  // bytes a single-token iteration streams
+  i += consumed;
+  return MK_OK;
+}
+
+// moe_mul_sum_add_mi300 [expert outputs [tokens,topk,n], routing weights [tokens,topk], residual, output]
+int lower_moe_combine(mk_graph *g, size_t &i, bool fused_single) {
+  const Task &t = g->tasks[i];
+  if (t.ops.size() != 4) return fail(MK_EINVAL, "%s expects 4 operands", t.name.c_str());
+  const Tensor &x = g->tensors[t.ops[0]], &tw = g->tensors[t.ops[1]], &r = g->tensors[t.ops[2]], &o = g->tensors[t.ops[3]];
+  const int B = g->cfg.max_num_batched_tokens;
+  if (x.ndims != 3 || x.dtype != MK_DT_BF16 || x.strides[2] != 1 || x.dims[0] < B) return fail(MK_EINVAL, "%s: input must be [tokens, topk, n] bf16", t.name.c_str());
+  const int topk = (int)x.dims[1], N = (int)x.dims[2];
+  if (tw.ndims != 2 || tw.dtype != MK_DT_F32 || tw.dims[1] != topk || tw.strides[1] != 1 || tw.dims[0] < B) return fail(MK_EINVAL, "%s: weights must be [tokens, %d] fp32", t.name.c_str(), topk);
+  if (r.ndims != 2 || o.ndims != 2 || r.dims[1] < N || o.dims[1] < N || r.dtype != MK_DT_BF16 || o.dtype != MK_DT_BF16 || r.dims[0] < B || o.dims[0] < B)
+    return fail(MK_EINVAL, "%s: residual/output must be [tokens, >=%d] bf16", t.name.c_str(), N);
+  MkStage st;
+  memset(&st, 0, sizeof(st));
+  st.op = MK_OP_MOE_COMBINE;
+  if (fused_single) st.flags |= MK_F_ONLY_MULTI;
+  st.n = N;
+  st.topk = topk;
+  st.in = x.ptr;
+  st.ld_in = (int)x.strides[0];
+  st.ld_in_slot = (int)x.strides[1];
+  st.moe_topk_w = (float *)tw.ptr;
+  st.ld_topk_w = (int)tw.strides[0];
+  st.res = r.ptr;
+  st.ld_res = (int)r.strides[0];
+  st.out = o.ptr;
+  st.ld_out = (int)o.strides[0];
+  g->stages.push_back(st);
+  g->stage_desc.push_back(fmt("MOE_COMBINE%s %s * %s + %s -> %s n=%d topk=%d", fused_single ? "[multi-token only]" : "", x.name.c_str(), tw.name.c_str(), r.name.c_str(), o.name.c_str(), N, topk));
+  i++;
+  return MK_OK;
+}
+
 int lower(mk_graph *g) {
   g->stages.clear();
   g->stage_desc.clear();
@@ -464,6 +636,40 @@ int lower(mk_graph *g) {
     } else if (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300") {
       int rc = lower_attention(g, i);
       if (rc) return rc;
+    } else if (t.name == "moe_topk_softmax_mi300") {
+      bool inline_next = false;
+      int rc = lower_moe_topk(g, i, &inline_next);
+      if (rc) return rc;
+      const MkStage router = g->stages.back();
+      rc = lower_moe_linear(g, i, inline_next ? &router : nullptr);
+      if (rc) return rc;
+    } else if (is_moe_linear(t.name)) {
+      int rc = lower_moe_linear(g, i, nullptr);
+      if (rc) return rc;
+    } else if (t.name == "moe_mul_sum_add_mi300") {
+      const bool fused = !g->stages.empty() && g->stages.back().op == MK_OP_MOE_LINEAR && (g->stages.back().flags & MK_F_MOE_COMBINE) &&
+                         g->stages.back().out == g->tensors[t.ops.empty() ? 0 : t.ops[0]].ptr;
+      int rc = lower_moe_combine(g, i, fused);
+      if (rc) return rc;
+    } else if (t.name == "moe_silu_mul") {
+      if (t.ops.size() != 2) return fail(MK_EINVAL, "moe_silu_mul expects 2 operands");
+      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[t.ops[1]];
+      if (!rows_contiguous_3d(x) || !rows_contiguous_3d(o) || x.dims[2] != 2 * o.dims[2] || x.dims[1] != o.dims[1] || x.dtype != MK_DT_BF16 || o.dtype != MK_DT_BF16)
+        return fail(MK_EINVAL, "moe_silu_mul shapes mismatch");
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_SILU_MUL;
+      st.n = (int)o.dims[2];
+      st.silu_half = st.n;  // [gate ; up] halves of every (token, slot) row
+      st.groups = 1;
+      st.topk = (int)x.dims[1];
+      st.in = x.ptr;
+      st.ld_in = (int)x.strides[1];
+      st.out = o.ptr;
+      st.ld_out = (int)o.strides[1];
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("SILU_MUL(moe) %s -> %s n=%d rows/token=%d", x.name.c_str(), o.name.c_str(), st.n, st.topk));
+      i++;
     } else if (t.name == "argmax_partial") {
       if (t.ops.size() != 3) return fail(MK_EINVAL, "argmax_partial expects 3 operands");
       if (i + 1 >= g->tasks.size() || g->tasks[i + 1].name != "argmax_reduce" || g->tasks[i + 1].ops.size() != 3)
@@ -526,7 +732,8 @@ int task_type_id(const std::string &n) {
       {"gang_attn_split_kv_mi300", 138}, {"kv_cache_update_mi300", 140}, {"paged_attention_ck_fmha_split_kv_mi300", 141},
       {"gang_linear_silu_mi300", 142}, {"linear_silu_mi300", 182}, {"splitk_linear_mi300", 129}, {"gang_splitk_linear_res_mi300", 144},
       {"gang_linear_n_tiling_mi300", 147}, {"gang_linear_res_n_tiling_mi300", 148}, {"gang_linear_msplit_mi300", 183},
-      {"gang_linear_res_msplit_mi300", 184}};
+      {"gang_linear_res_msplit_mi300", 184}, {"moe_w13_linear_mi300", 170}, {"moe_w2_linear_mi300", 171}, {"moe_topk_softmax_mi300", 172},
+      {"moe_mul_sum_add_mi300", 173}, {"gang_moe_w13_linear_mi300", 174}, {"gang_moe_w2_linear_mi300", 175}, {"moe_silu_mul", 118}};
   auto it = ids.find(n);
   return it == ids.end() ? 0 : it->second;
 }
@@ -903,7 +1110,8 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
   bool a, b;
   int c;
   static const char *known[] = {"embedding", "rmsnorm", "gang_rmsnorm_mi300", "silu_mul", "gang_attn_split_kv_mi300", "kv_cache_update_mi300",
-                                "paged_attention_ck_fmha_split_kv_mi300", "argmax_partial", "argmax_reduce"};
+                                "paged_attention_ck_fmha_split_kv_mi300", "argmax_partial", "argmax_reduce", "moe_topk_softmax_mi300", "moe_w13_linear_mi300",
+                                "moe_w2_linear_mi300", "gang_moe_w13_linear_mi300", "gang_moe_w2_linear_mi300", "moe_silu_mul", "moe_mul_sum_add_mi300"};
   bool ok = linear_kind(t.name, &a, &b, &c);
   for (auto k : known) ok = ok || t.name == k;
   if (!ok) return fail(MK_EUNSUPPORTED, "Unsupported task name: %s", task_name);

@@ -739,12 +739,351 @@ __device__ __forceinline__ void stage_silu_mul(const MkStage &st, Ctx &c, int M)
   const int n = st.n, half = st.silu_half;
   const uint16_t *in = (const uint16_t *)st.in;
   uint16_t *out = (uint16_t *)st.out;
-  const int total = M * n;
+  const int total = M * (st.topk > 0 ? st.topk : 1) * n;  // MoE: topk rows per token, contiguous
   for (int i = c.vid * MK_THREADS + threadIdx.x; i < total; i += c.G * MK_THREADS) {
     const int t = i / n, j = i - t * n;
     const int g = j / half, jj = j - g * half;
     const uint16_t *row = in + (size_t)t * st.ld_in + (size_t)g * 2 * half;
     out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(silu_mul(bf2f(ldc_u16(row + jj)), bf2f(ldc_u16(row + half + jj))));
+  }
+}
+
+// ----------------------------------------------------------------------------- mixture of experts
+// Routing lists of one workgroup, kept in the LDS region above MK_PF_OFFSET.
+struct MoeLds {
+  int r[MK_MOE_MAX_EXPERTS];          // single-token routing: 1 + slot per expert
+  int act_e[MK_MOE_MAX_EXPERTS];      // expert id of each active expert
+  int pair_off[MK_MOE_MAX_EXPERTS + 4];  // first (token, slot) pair of each active expert; [n_act] = number of pairs
+  int pair_ts[MK_MAX_TOKENS * MK_MOE_MAX_TOPK];  // token | slot << 8
+  int n_act;
+  int wtot[2][MK_WAVES];
+  float w[MK_MOE_MAX_TOPK];           // single-token routing weights by slot
+};
+
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+  return v;
+}
+
+// Route one token with one wavefront: fp32 softmax over all experts, `topk` rounds of arg-max (equal probabilities
+// go to the lower expert id), weights renormalised by the sum of the selected probabilities.  Lane l owns experts
+// l, l+64, ...: sel[j] becomes 1 + slot for a selected expert l + 64 j, 0 otherwise; lane s < topk returns the weight
+// and expert of slot s.  Reference task: tasks/mi300/moe_topk_softmax_mi300.cuh:100-213.
+__device__ __forceinline__ void moe_route_wave(const uint16_t *logits, int E, int topk, int lane, int sel[4], float &w_slot, int &e_slot) {
+  float p[4];
+  float mx = -3.0e38f;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    const int e = j * 64 + lane;
+    p[j] = e < E ? bf2f(ldc_u16(logits + e)) : -3.0e38f;
+    mx = fmaxf(mx, p[j]);
+    sel[j] = 0;
+  }
+  mx = wave_max(mx);
+  float sum = 0.f;
+#pragma unroll
+  for (int j = 0; j < 4; j++) {
+    p[j] = (j * 64 + lane < E) ? expf(p[j] - mx) : 0.f;
+    sum += p[j];
+  }
+  const float inv = 1.f / wave_sum(sum);
+#pragma unroll
+  for (int j = 0; j < 4; j++) p[j] = (j * 64 + lane < E) ? p[j] * inv : -1.f;
+  float tot = 0.f;
+  w_slot = 0.f;
+  e_slot = 0;
+  for (int s = 0; s < topk; s++) {
+    float bv = p[0];
+    int be = lane;
+#pragma unroll
+    for (int j = 1; j < 4; j++)
+      if (p[j] > bv) {
+        bv = p[j];
+        be = j * 64 + lane;
+      }
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) {
+      const float ov = __shfl_xor(bv, o, 64);
+      const int oe = __shfl_xor(be, o, 64);
+      if (ov > bv || (ov == bv && oe < be)) {
+        bv = ov;
+        be = oe;
+      }
+    }
+    tot += bv;
+    if (lane == s) {
+      w_slot = bv;
+      e_slot = be;
+    }
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (j * 64 + lane == be) {
+        sel[j] = s + 1;
+        p[j] = -10000.f;
+      }
+  }
+  w_slot *= 1.f / tot;
+}
+
+// Router stage for multi-token iterations: one wavefront per token writes the routing weights and the token's
+// column of the routing table.  Columns of tokens that are not part of the iteration are left alone.
+__device__ __forceinline__ void stage_moe_topk(const MkStage &st, Ctx &c, int M) {
+  barrier_wait(c);
+  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int E = st.num_experts;
+  for (int t = c.vid * MK_WAVES + wave; t < M; t += c.G * MK_WAVES) {
+    int sel[4];
+    float w;
+    int e;
+    moe_route_wave((const uint16_t *)st.moe_logits + (size_t)t * st.ld_logits, E, st.topk, lane, sel, w, e);
+    if (lane < st.topk) st.moe_topk_w[(size_t)t * st.ld_topk_w + lane] = w;
+#pragma unroll
+    for (int j = 0; j < 4; j++)
+      if (j * 64 + lane < E) st.moe_routing[(size_t)(j * 64 + lane) * st.ld_routing + t] = sel[j];
+  }
+}
+
+// Build the active-expert list and the (token, slot) pairs of every active expert from the routing table.
+// Single-token iterations keep slot order (active expert s is the expert of slot s); multi-token iterations list
+// experts in ascending id with their tokens in ascending order.
+__device__ __forceinline__ void moe_build_lists(const MkStage &st, MoeLds *L, int M, bool r_in_lds) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int E = st.num_experts;
+  if (M == 1) {
+    if (tid <= st.topk) {  // slot s is "active expert" s; a slot no expert claims (caller-written table) stays empty
+      L->act_e[tid] = -1;
+      L->pair_off[tid] = tid;
+      L->pair_ts[tid] = tid << 8;
+    }
+    if (tid == 0) L->n_act = st.topk;
+    __syncthreads();
+    if (tid < E) {
+      const int r = r_in_lds ? L->r[tid] : ldc_i32(st.moe_routing + (size_t)tid * st.ld_routing);
+      if (r > 0 && r <= st.topk) L->act_e[r - 1] = tid;
+    }
+    __syncthreads();
+    return;
+  }
+  int cnt = 0;
+  if (tid < E)
+    for (int t = 0; t < M; t++) {
+      const int r = ldc_i32(st.moe_routing + (size_t)tid * st.ld_routing + t);
+      cnt += r > 0 && r <= st.topk;
+    }
+  int sc = cnt, sa = cnt > 0;  // inclusive scans inside the wavefront
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int vc = __shfl_up(sc, o, 64), va = __shfl_up(sa, o, 64);
+    if (lane >= o) {
+      sc += vc;
+      sa += va;
+    }
+  }
+  if (lane == 63) {
+    L->wtot[0][wave] = sc;
+    L->wtot[1][wave] = sa;
+  }
+  __syncthreads();
+  int bc = 0, ba = 0;
+  for (int w = 0; w < wave; w++) {
+    bc += L->wtot[0][w];
+    ba += L->wtot[1][w];
+  }
+  const int off = bc + sc - cnt, ai = ba + sa - (cnt > 0);
+  if (cnt > 0) {
+    L->act_e[ai] = tid;
+    L->pair_off[ai] = off;
+    int i = off;
+    for (int t = 0; t < M; t++) {
+      const int r = ldc_i32(st.moe_routing + (size_t)tid * st.ld_routing + t);
+      if (r > 0 && r <= st.topk && i < MK_MAX_TOKENS * MK_MOE_MAX_TOPK) L->pair_ts[i++] = t | ((r - 1) << 8);
+    }
+  }
+  if (tid == MK_THREADS - 1) {
+    L->n_act = ba + sa;
+    L->pair_off[ba + sa] = bc + sc;
+  }
+  __syncthreads();
+}
+
+// Per-expert linear over the active experts: y[t, slot, :] = W[e(t,slot)] x(t, slot), one weight row (or one
+// [gate ; up] row pair) per wavefront step, each row read once and applied to every token routed to its expert.
+// Work units (active expert, row) are dealt out in contiguous runs per wavefront; the rows of the next R units are
+// in flight in registers while a unit is reduced.  Optional epilogues: SwiGLU (gate and up rounded to bf16 first, as
+// the separate activation task of the reference sees them) and, for a single token, the weighted sum over the
+// slots plus residual, accumulated in slot order in fp32 from the bf16-rounded expert outputs.
+// KL = 16-byte row segments per lane (K <= 512 KL).
+// Reference tasks: moe_linear_kernel_mi300 (tasks/mi300/moe_linear_mi300.cuh:53-295), silu_mul_task_impl,
+// mul_sum_add_mi300_task_impl (tasks/mi300/moe_mul_sum_add_mi300.cuh:31-55).
+template <int KL, int R, bool SILU>
+__device__ __forceinline__ void stage_moe_linear_t(const MkStage &st, Ctx &c, int M, char *smem) {
+  constexpr int NROW = SILU ? 2 : 1;
+  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  MoeLds *L = (MoeLds *)(smem + MK_PF_OFFSET);
+  const int k8 = st.k / 8;
+  const bool combine = !SILU && (st.flags & MK_F_MOE_COMBINE) && M == 1;
+  const bool inline_topk = (st.flags & MK_F_MOE_INLINE_TOPK) && M == 1;
+  barrier_wait(c);
+  if (M > 1) {  // activation rows are read with cached loads below: drop stale lines of this CU's L1 first
+    if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __syncthreads();
+  }
+  if (inline_topk) {
+    if (wave == 0) {
+      int sel[4];
+      float w;
+      int e;
+      moe_route_wave((const uint16_t *)st.moe_logits, st.num_experts, st.topk, lane, sel, w, e);
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (j * 64 + lane < st.num_experts) {
+          L->r[j * 64 + lane] = sel[j];
+          if (c.vid == 0) st.moe_routing[(size_t)(j * 64 + lane) * st.ld_routing] = sel[j];
+        }
+      if (lane < st.topk) {
+        L->w[lane] = w;
+        if (c.vid == 0) st.moe_topk_w[lane] = w;
+      }
+    }
+    __syncthreads();
+  } else if (combine && tid < st.topk) {
+    L->w[tid] = ldc_f32(st.moe_topk_w + tid);
+  }
+  moe_build_lists(st, L, M, inline_topk);
+  const int n_act = L->n_act;
+  if (c.vid == 0 && st.moe_mask) {  // publish the active-expert list (its order is unspecified in the reference)
+    for (int i = tid; i < st.num_experts; i += MK_THREADS) st.moe_mask[i] = i < n_act ? L->act_e[i] : -1;
+    if (tid == 0) st.moe_mask[st.num_experts] = n_act;
+  }
+  // single token: stage the input row(s) in LDS (one row, or one row per slot)
+  const int nslot_in = st.ld_in_slot ? st.topk : 1;
+  const bool x_lds = M == 1 && (size_t)nslot_in * st.k * 2 <= (size_t)MK_RED_OFFSET;
+  u32x4 *xs4 = (u32x4 *)smem;
+  if (x_lds) {
+    for (int i = tid; i < nslot_in * k8; i += MK_THREADS) {
+      const int s = i / k8, o = i - s * k8;
+      xs4[i] = ldc_16B((const u32x4 *)((const uint16_t *)st.in + (size_t)s * st.ld_in_slot) + o);
+    }
+    __syncthreads();
+  }
+  const int NR = SILU ? st.n / 2 : st.n;  // units per expert
+  const int nwaves = c.G * MK_WAVES, gw = c.vid * MK_WAVES + wave;
+  int U, upw;
+  if (combine) {  // token-major: the n_act units of one output row are consecutive and stay in one wavefront
+    U = NR * n_act;
+    upw = ((NR + nwaves - 1) / nwaves) * n_act;
+  } else {
+    U = n_act * NR;
+    upw = (U + nwaves - 1) / nwaves;
+  }
+  const int u0 = min(U, gw * upw), u1 = min(U, u0 + upw);
+  const u32x4 *W = (const u32x4 *)st.w.seg[0];
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  u32x4 buf[R][NROW][KL];
+  auto load_unit = [&](int u, u32x4 (&b)[NROW][KL]) {
+    int a, j;
+    if (combine) {
+      j = u / n_act;
+      a = u - j * n_act;
+    } else {
+      a = u / NR;
+      j = u - a * NR;
+    }
+    const int ei = L->act_e[a];
+    const size_t e = (size_t)max(ei, 0);
+#pragma unroll
+    for (int h = 0; h < NROW; h++) {
+      const u32x4 *p = W + (e * st.n + (size_t)(j + h * NR)) * k8;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) b[h][kc] = (ei >= 0 && kc * 64 + lane < k8) ? ldg_stream(p + kc * 64 + lane) : zero;
+    }
+  };
+#pragma unroll
+  for (int jj = 0; jj < R; jj++)
+    if (u0 + jj < u1) load_unit(u0 + jj, buf[jj]);
+  uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
+  float comb = 0.f;
+  for (int i = u0; i < u1; i += R) {
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) {
+      const int u = i + jj;
+      if (u < u1) {
+        int a, j;
+        if (combine) {
+          j = u / n_act;
+          a = u - j * n_act;
+        } else {
+          a = u / NR;
+          j = u - a * NR;
+        }
+        const int p0 = L->pair_off[a], p1 = L->act_e[a] >= 0 ? L->pair_off[a + 1] : p0;
+        if (combine && a == 0) comb = bf2f(ldc_u16((const uint16_t *)st.res + j));
+        for (int p = p0; p < p1; p++) {
+          const int ts = L->pair_ts[p], tok = ts & 255, slot = ts >> 8;
+          const u32x4 *x = x_lds ? xs4 + (st.ld_in_slot ? slot * k8 : 0)
+                                 : (const u32x4 *)((const uint16_t *)st.in + (size_t)tok * st.ld_in + (size_t)slot * st.ld_in_slot);
+          float acc[NROW];
+#pragma unroll
+          for (int h = 0; h < NROW; h++) acc[h] = 0.f;
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) {
+            u32x4 xv = zero;
+            if (kc * 64 + lane < k8) xv = (x_lds || M > 1) ? x[kc * 64 + lane] : ldc_16B(x + kc * 64 + lane);
+#pragma unroll
+            for (int h = 0; h < NROW; h++) acc[h] = dot8(buf[jj][h][kc], xv, acc[h]);
+          }
+#pragma unroll
+          for (int h = 0; h < NROW; h++) acc[h] = wave_sum(acc[h]);
+          uint16_t *y = out + (size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot;
+          if (SILU) {
+            const uint32_t g = f2bf(acc[0]), up = f2bf(acc[NROW - 1]);
+            if (lane == 0) {
+              y[j] = (uint16_t)g;
+              y[j + NR] = (uint16_t)up;
+              out2[(size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
+            }
+          } else {
+            const uint32_t v = f2bf(acc[0]);
+            if (lane == 0) y[j] = (uint16_t)v;
+            if (combine) comb = fmaf(bf2f((uint16_t)v), L->w[slot], comb);
+          }
+        }
+        if (combine && a == n_act - 1 && lane == 0) out2[j] = (uint16_t)f2bf(comb);
+        if (u + R < u1) load_unit(u + R, buf[jj]);
+      }
+    }
+  }
+}
+
+__device__ __forceinline__ void stage_moe_linear(const MkStage &st, Ctx &c, int M, char *smem) {
+  const bool silu = st.flags & MK_F_SILU;
+  if (st.k <= 1024) {
+    if (silu) stage_moe_linear_t<2, 4, true>(st, c, M, smem);
+    else stage_moe_linear_t<2, 6, false>(st, c, M, smem);
+  } else if (st.k <= 2048) {
+    if (silu) stage_moe_linear_t<4, 3, true>(st, c, M, smem);
+    else stage_moe_linear_t<4, 4, false>(st, c, M, smem);
+  } else {
+    if (silu) stage_moe_linear_t<8, 1, true>(st, c, M, smem);
+    else stage_moe_linear_t<8, 2, false>(st, c, M, smem);
+  }
+}
+
+// Weighted sum of the expert outputs plus residual for multi-token iterations:
+// out[t, :] = bf16(res[t, :] + sum_k w[t, k] * y[t, k, :]), fp32, slots in order.
+// Reference task: mul_sum_add_mi300_task_impl (tasks/mi300/moe_mul_sum_add_mi300.cuh:31-55).
+__device__ __forceinline__ void stage_moe_combine(const MkStage &st, Ctx &c, int M) {
+  barrier_wait(c);
+  const int n = st.n, total = M * n;
+  const uint16_t *in = (const uint16_t *)st.in, *res = (const uint16_t *)st.res;
+  uint16_t *out = (uint16_t *)st.out;
+  for (int i = c.vid * MK_THREADS + threadIdx.x; i < total; i += c.G * MK_THREADS) {
+    const int t = i / n, j = i - t * n;
+    float s = bf2f(ldc_u16(res + (size_t)t * st.ld_res + j));
+    for (int k = 0; k < st.topk; k++)
+      s = fmaf(bf2f(ldc_u16(in + (size_t)t * st.ld_in + (size_t)k * st.ld_in_slot + j)), ldc_f32(st.moe_topk_w + (size_t)t * st.ld_topk_w + k), s);
+    out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(s);
   }
 }
 
@@ -1145,6 +1484,9 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
           else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8>(st, c, rt, M, smem);
           else barrier_wait(c);
           break;
+        case MK_OP_MOE_TOPK: stage_moe_topk(st, c, M); break;
+        case MK_OP_MOE_LINEAR: stage_moe_linear(st, c, M, smem); break;
+        case MK_OP_MOE_COMBINE: stage_moe_combine(st, c, M); break;
         case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, M, smem); break;
         case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, M); break;
         default: barrier_wait(c); break;

@@ -35,6 +35,9 @@ enum MkOp {
   MK_OP_ATTN = 5,
   MK_OP_ARGMAX_PARTIAL = 6,
   MK_OP_ARGMAX_REDUCE = 7,
+  MK_OP_MOE_TOPK = 8,     // router softmax -> top-k -> renormalise, one wavefront per token
+  MK_OP_MOE_LINEAR = 9,   // per-expert linear over the active experts (W13 with optional SwiGLU, W2)
+  MK_OP_MOE_COMBINE = 10, // out = res + sum_k w[t,k] * x[t,k,:]
 };
 
 enum MkStageFlags {
@@ -45,7 +48,12 @@ enum MkStageFlags {
   MK_F_ROPE = 16,        // ATTN: rotate-half RoPE on q and k
   MK_F_ONLY_MULTI = 32,  // stage runs only when the iteration has more than one token
   MK_F_EMBED_FROM_TOKENS = 64,  // EMBED: ids come from tokens[req, step+j] instead of input_tokens
+  MK_F_MOE_INLINE_TOPK = 128,   // MOE_LINEAR: a single-token iteration routes inside this stage (the MOE_TOPK stage before it is multi-token only)
+  MK_F_MOE_COMBINE = 256,       // MOE_LINEAR: a single-token iteration also forms res + sum_k w_k * y_k (the MOE_COMBINE stage after it is multi-token only)
 };
+
+#define MK_MOE_MAX_EXPERTS 256  // one thread per expert when the routing lists are built
+#define MK_MOE_MAX_TOPK 16
 
 // A (possibly shuffled) weight matrix [rows, k] bf16.  Virtual row r of a shuffled
 // tensor lives in source `seg` at a row computed from the group structure, so no
@@ -83,6 +91,18 @@ struct MkStage {
   int pad3;
   // argmax
   void *aux0, *aux1;
+  // mixture of experts.  MOE_LINEAR: x(t,slot) = in + t*ld_in + slot*ld_in_slot, expert e's weights are rows
+  // [e*n, (e+1)*n) of w.seg[0], y(t,slot,row) = out + t*ld_out + slot*ld_out_slot + row; with MK_F_SILU rows
+  // [0,n/2) are gate and [n/2,n) up, and out2(t,slot,j) receives silu(gate_j)*up_j; with MK_F_MOE_COMBINE out2 is
+  // the [tokens, n] result of the weighted sum.
+  const void *moe_logits;  // [tokens, num_experts] bf16 router logits (ld_logits)
+  float *moe_topk_w;       // [tokens, topk] fp32 renormalised routing weights (ld_topk_w)
+  int *moe_routing;        // [num_experts, tokens] int32: 1 + top-k slot of the expert for that token, 0 = not routed
+  int *moe_mask;           // [num_experts + 1] int32: ids of the active experts, then their count at [num_experts]
+  void *out2;
+  int num_experts, topk, ld_logits, ld_topk_w;
+  int ld_routing, ld_in_slot, ld_out_slot, ld_out2;
+  int ld_out2_slot, pad4, pad5, pad6;
 };
 
 // Hierarchical barrier state.  One 128-byte line per counter so that XCD-local

@@ -1,4 +1,4 @@
-"""Qwen3 dense decode driver on the MI355X megakernel.
+"""Qwen3 decode driver (dense Qwen3-8B shape and mixture-of-experts Qwen3-30B-A3B shape) on the MI355X megakernel.
 
 Builds the per-layer task graph through the PersistentKernel API the same way the reference driver
 does (demo/qwen3/demo.py:314-1169), in either of its two README configurations:
@@ -8,6 +8,10 @@ does (demo/qwen3/demo.py:314-1169), in either of its two README configurations:
   (USE_GANG=1 USE_CK_FMHA=1 USE_FUSED_SILU=1, demo.py:556-1113);
 * mode="mpk": rmsnorm -> linear -> kv_cache_update -> paged_attention_ck_fmha -> linear_with_residual ->
   rmsnorm -> linear -> silu_mul -> linear_with_residual (the non-gang path with separate activation).
+
+With Qwen3Shape.num_experts > 0 the MLP is the reference's mixture-of-experts sequence (demo/qwen3/demo_30B_A3B.py:
+675-754): router linear -> top-k softmax routing -> W13 per-expert linear -> SwiGLU -> W2 per-expert linear -> weighted
+sum + residual ("fleet": the gang_moe_* layers, "mpk": the moe_* layers with explicit grids).
 
 Both lower to the same stage program.  Weights are random-init (there is no checkpoint loader here);
 the CLI prints decode ms/token measured over decode iterations only.
@@ -32,12 +36,27 @@ class Qwen3Shape:
     num_layers: int = 36
     vocab_size: int = 151936
     rope_theta: float = 1e6
+    num_experts: int = 0           # > 0: mixture-of-experts MLP
+    num_experts_per_tok: int = 0
+    moe_intermediate_size: int = 0
 
-    def weight_bytes_per_token(self):
-        """bf16 weight bytes one decode step streams (all linears + LM head)."""
+    @staticmethod
+    def qwen3_30b_a3b(num_layers: int = 48):
+        """Qwen3-30B-A3B: 48 layers, hidden 2048, 32 q / 4 kv heads, 128 experts, top-8, expert width 768."""
+        return Qwen3Shape(hidden_size=2048, num_q_heads=32, num_kv_heads=4, head_dim=128, intermediate_size=0, num_layers=num_layers,
+                          num_experts=128, num_experts_per_tok=8, moe_intermediate_size=768)
+
+    def weight_bytes_per_token(self, distinct_experts: int = None):
+        """bf16 weight bytes one decode step streams (all linears + LM head).  For the mixture-of-experts shape the
+        expert term counts `distinct_experts` experts per layer (default: top-k, i.e. one token)."""
         H, I = self.hidden_size, self.intermediate_size
         qkv = (self.num_q_heads + 2 * self.num_kv_heads) * self.head_dim * H
-        per_layer = qkv + self.num_q_heads * self.head_dim * H + 2 * I * H + H * I
+        if self.num_experts > 0:
+            ne = self.num_experts_per_tok if distinct_experts is None else distinct_experts
+            mlp = self.num_experts * H + ne * 3 * self.moe_intermediate_size * H
+        else:
+            mlp = 2 * I * H + H * I
+        per_layer = qkv + self.num_q_heads * self.head_dim * H + mlp
         return 2 * (self.num_layers * per_layer + self.vocab_size * H)
 
     def kv_bytes_per_position(self):
@@ -59,10 +78,16 @@ def random_weights(shape: Qwen3Shape, seed: int = 0, device="cuda"):
     ones = lambda n: torch.ones(n, dtype=torch.bfloat16, device=device)
     w = {"embed": lin(shape.vocab_size, H), "layers": []}
     for _ in range(shape.num_layers):
-        w["layers"].append({
-            "input_norm": ones(H), "q_proj": lin(shape.num_q_heads * D, H), "k_proj": lin(shape.num_kv_heads * D, H),
-            "v_proj": lin(shape.num_kv_heads * D, H), "q_norm": ones(D), "k_norm": ones(D), "o_proj": lin(H, shape.num_q_heads * D),
-            "post_norm": ones(H), "gate_proj": lin(I, H), "up_proj": lin(I, H), "down_proj": lin(H, I)})
+        lw = {"input_norm": ones(H), "q_proj": lin(shape.num_q_heads * D, H), "k_proj": lin(shape.num_kv_heads * D, H),
+              "v_proj": lin(shape.num_kv_heads * D, H), "q_norm": ones(D), "k_norm": ones(D), "o_proj": lin(H, shape.num_q_heads * D),
+              "post_norm": ones(H)}
+        if shape.num_experts > 0:
+            E, MI = shape.num_experts, shape.moe_intermediate_size
+            # packed per expert as the reference driver does (demo/qwen3/demo_30B_A3B.py:376-420): [gate ; up] rows
+            lw.update({"router": lin(E, H), "gate_up_proj": lin(E * 2 * MI, H).view(E, 2 * MI, H), "down_proj": lin(E * H, MI).view(E, H, MI)})
+        else:
+            lw.update({"gate_proj": lin(I, H), "up_proj": lin(I, H), "down_proj": lin(H, I)})
+        w["layers"].append(lw)
     w["final_norm"] = ones(H)
     w["lm_head"] = lin(shape.vocab_size, H)
     return w
@@ -144,9 +169,22 @@ class Qwen3Decoder:
         q_ws = new("ck_fmha_q_workspace", nq * D)
         lse_acc = new("ck_fmha_lse_acc", nq, mi.float32)
         attn_proj_out = new("attn_proj_out", H)
-        mlp_mid = new("mlp_mid", 2 * I)
-        silu_mul_out = new("silu_mul_out", I)
-        mlp_out = new("mlp_out", H)
+        moe = s.num_experts > 0
+        if moe:
+            E, topk, MI = s.num_experts, s.num_experts_per_tok, s.moe_intermediate_size
+            new3 = lambda name, cols: mpk.new_tensor(dims=(B, topk, cols), dtype=mi.bfloat16, name=name, io_category="cuda_tensor")
+            moe_gate_out = new("moe_gate_out", E)
+            moe_topk_weight = new("moe_topk_weight", topk, mi.float32)
+            moe_routing_indices = mpk.new_tensor(dims=(E, B), dtype=mi.int32, name="moe_routing_indices", io_category="cuda_tensor")
+            moe_mask = mpk.new_tensor(dims=(E + 1,), dtype=mi.int32, name="moe_mask", io_category="cuda_tensor")
+            mlp_mid, silu_mul_out, mlp_out = new3("mlp_mid", 2 * MI), new3("silu_mul_out", MI), new3("mlp_out", H)
+            mlp_weighted_sum_out = new("mlp_weighted_sum_out", H)
+            t.update(moe_gate_out=moe_gate_out, moe_topk_weight=moe_topk_weight, moe_routing_indices=moe_routing_indices, moe_mask=moe_mask,
+                     mlp_weighted_sum_out=mlp_weighted_sum_out)
+        else:
+            mlp_mid = new("mlp_mid", 2 * I)
+            silu_mul_out = new("silu_mul_out", I)
+            mlp_out = new("mlp_out", H)
         argmax_in = new("argmax_in", s.vocab_size)
         argmax_tasks = mpk.num_workers if s.vocab_size % mpk.num_workers == 0 else 1
         for cand in (240, 256, 128, 64, 32, 16, 8, 4, 2):
@@ -204,6 +242,32 @@ class Qwen3Decoder:
                 mpk.linear_with_residual_layer(input=attn_out, weight=w_o, residual=x, output=proj_out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1))
             x = proj_out
             w_norm2 = mpk.attach_input(lw["post_norm"], f"layer_{i}_post_attn_layernorm")
+            if moe:
+                # demo/qwen3/demo_30B_A3B.py:675-754
+                w_router = mpk.attach_input(lw["router"], f"layer_{i}_moe_gate")
+                w_gatedup = mpk.attach_input(lw["gate_up_proj"], f"layer_{i}_experts_gate_up_proj")
+                w_down = mpk.attach_input(lw["down_proj"], f"layer_{i}_experts_down_proj")
+                norm(x, w_norm2)
+                mpk.linear_layer(input=rmsnorm_out, weight=w_router, output=moe_gate_out, grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+                mpk.moe_topk_softmax_routing_layer(input=moe_gate_out, output=(moe_topk_weight, moe_routing_indices, moe_mask),
+                                                   grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+                if gang:
+                    mpk.gang_moe_w13_linear_layer(input=rmsnorm_out, weight=w_gatedup, moe_routing_indices=moe_routing_indices,
+                                                  moe_mask=moe_mask, output=mlp_mid)
+                else:
+                    mpk.moe_w13_linear_layer(input=rmsnorm_out, weight=w_gatedup, moe_routing_indices=moe_routing_indices, moe_mask=moe_mask,
+                                             output=mlp_mid, grid_dim=(10, w_gatedup.dim(1) // 64, 1), block_dim=(256, 1, 1))
+                mpk.moe_silu_mul_layer(input=mlp_mid, output=silu_mul_out, grid_dim=(B, topk, 1), block_dim=(256, 1, 1))
+                if gang:
+                    mpk.gang_moe_w2_linear_layer(input=silu_mul_out, weight=w_down, moe_routing_indices=moe_routing_indices, moe_mask=moe_mask,
+                                                 output=mlp_out)
+                else:
+                    mpk.moe_w2_linear_layer(input=silu_mul_out, weight=w_down, moe_routing_indices=moe_routing_indices, moe_mask=moe_mask,
+                                            output=mlp_out, grid_dim=(8, w_down.dim(1) // 64, 1), block_dim=(256, 1, 1))
+                mpk.moe_mul_sum_add_layer(input=mlp_out, weight=moe_topk_weight, residual=x, output=mlp_weighted_sum_out,
+                                          grid_dim=(B, max(1, H // 256), 1), block_dim=(256, 1, 1))
+                x = mlp_weighted_sum_out
+                continue
             w_gate = mpk.attach_input(lw["gate_proj"], f"layer_{i}_gate_proj")
             w_up = mpk.attach_input(lw["up_proj"], f"layer_{i}_up_proj")
             groups = (2 * I) // 256
@@ -265,8 +329,9 @@ def main():
     ap.add_argument("--page-size", type=int, default=4096)
     ap.add_argument("--num-layers", type=int, default=36)
     ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
+    ap.add_argument("--model", choices=["qwen3-8b", "qwen3-30b-a3b"], default="qwen3-8b")
     args = ap.parse_args()
-    shape = Qwen3Shape(num_layers=args.num_layers)
+    shape = Qwen3Shape(num_layers=args.num_layers) if args.model == "qwen3-8b" else Qwen3Shape.qwen3_30b_a3b(min(args.num_layers, 48))
     B = args.max_num_batched_tokens
     R = args.max_num_batched_requests or B
     max_seq = min(args.max_seq_length, args.prompt_length + args.max_new_tokens + 1)

@@ -9,6 +9,8 @@ whole generation.  Nothing here computes: without libfleet_mk.so and a gfx950 de
 import ctypes
 import math
 
+import sys
+
 import torch
 
 from .. import _capi
@@ -252,6 +254,87 @@ class PersistentKernel:
         self._task("splitk_linear_res_atomic_mi300", grid_dim, block_dim,
                    [(input, (-1, 1, -1), 1), (weight, (0, 1, -1), 1), (residual, (1, -1, -1), -1), (workspace, (1, -1, -1), -1),
                     (done_counter, (0, -1, -1), -1), (output, (1, -1, -1), -1)], [k_splits])
+
+    def splitk_linear_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1437.  Lowered like linear_layer: the MI355X stage never splits K across workgroups."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("splitk_linear_mi300", grid_dim, block_dim,
+                   [(input, (-1, 1, -1), 1), (weight, (0, 1, -1), 1), (output, (1, 0, -1), -1)])
+
+    # ------------------------------------------------------------------ mixture-of-experts layers
+    def moe_topk_softmax_routing_layer(self, input: DTensor, output: tuple, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1203.  fp32 softmax over all experts -> top-k (ties to the lower expert id) -> renormalise.
+        Unlike the reference task (moe_topk_softmax_mi300.cuh:116-122) the router logits are left intact."""
+        assert input.num_dims == 2  # (batch_size, num_experts)
+        assert len(output) == 3
+        moe_topk_weight, moe_routing_indices, moe_masks = output
+        assert moe_topk_weight.num_dims == 2  # (batch_size, num_experts_per_tok)
+        assert moe_routing_indices.num_dims == 2  # (num_experts, batch_size)
+        assert moe_masks.num_dims == 1  # (num_experts + 1)
+        self._task("moe_topk_softmax_mi300", grid_dim, block_dim,
+                   [(input, (0, -1, -1), -1), (moe_topk_weight, (0, -1, -1), -1), (moe_routing_indices, _REPL, -1), (moe_masks, _REPL, -1)])
+
+    def _moe_linear(self, name, input, weight, moe_routing_indices, moe_mask, output, grid_dim, block_dim, in_forloop, params=()):
+        assert weight.num_dims == 3  # (num_experts, output_size, reduction_size)
+        assert moe_routing_indices.num_dims == 2  # (num_experts, batch_size)
+        assert moe_mask.num_dims == 1  # (num_experts + 1)
+        assert output.num_dims == 3  # (batch_size, num_experts_per_tok, output_size)
+        self._task(name, grid_dim, block_dim,
+                   [(input, _REPL, in_forloop), (weight, (-1, 1, -1), 2), (moe_routing_indices, _REPL, -1), (moe_mask, _REPL, -1),
+                    (output, (-1, 2, -1), -1)], params)
+
+    def moe_w13_linear_layer(self, input: DTensor, weight: DTensor, moe_routing_indices: DTensor, moe_mask: DTensor, output: DTensor,
+                             grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1229.  output[t, slot, :] = weight[expert(t, slot)] @ input[t]."""
+        assert input.num_dims == 2  # (batch_size, hidden_size)
+        self._moe_linear("moe_w13_linear_mi300", input, weight, moe_routing_indices, moe_mask, output, grid_dim, block_dim, 1)
+
+    def moe_silu_mul_layer(self, input: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1262.  Rows are [gate ; up] halves per (token, slot)."""
+        assert input.num_dims == 3  # (batch_size, num_experts_per_tok, 2 * intermediate_size)
+        assert output.num_dims == 3  # (batch_size, num_experts_per_tok, intermediate_size)
+        self._task("moe_silu_mul", grid_dim, block_dim, [(input, (0, 1, -1), -1), (output, (0, 1, -1), -1)])
+
+    def moe_w2_linear_layer(self, input: DTensor, weight: DTensor, moe_routing_indices: DTensor, moe_mask: DTensor, output: DTensor,
+                            grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1278.  output[t, slot, :] = weight[expert(t, slot)] @ input[t, slot]."""
+        assert input.num_dims == 3  # (batch_size, num_experts_per_tok, intermediate_size)
+        self._moe_linear("moe_w2_linear_mi300", input, weight, moe_routing_indices, moe_mask, output, grid_dim, block_dim, 2)
+
+    def _gang_moe_params(self, weight, k_multiple, per_token):
+        batch_size = self.max_num_batched_tokens
+        num_experts, output_size, reduction_size = weight.dim(0), weight.dim(1), weight.dim(2)
+        tile_n = 64
+        assert output_size % tile_n == 0, f"output_size {output_size} not divisible by {tile_n}"
+        assert reduction_size % k_multiple == 0, f"K={reduction_size} not divisible by {k_multiple}"
+        n_tiles = output_size // tile_n
+        tiles_per_expert = n_tiles * batch_size if per_token else max(1, batch_size // 16) * n_tiles
+        max_experts_per_xcd = (num_experts + 7) // 8
+        total_tiles_per_xcd = max_experts_per_xcd * tiles_per_expert
+        assert total_tiles_per_xcd <= 65535, f"total_tiles_per_xcd={total_tiles_per_xcd} exceeds uint16_t (bs={batch_size})"
+        return [tiles_per_expert, max_experts_per_xcd, total_tiles_per_xcd]
+
+    def gang_moe_w13_linear_layer(self, input: DTensor, weight: DTensor, moe_routing_indices: DTensor, moe_mask: DTensor, output: DTensor,
+                                  block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1311.  Same stage as moe_w13_linear_layer."""
+        assert input.num_dims == 2
+        self._moe_linear("gang_moe_w13_linear_mi300", input, weight, moe_routing_indices, moe_mask, output, (8, 1, 1), block_dim, 1,
+                         self._gang_moe_params(weight, 256, False))
+
+    def gang_moe_w2_linear_layer(self, input: DTensor, weight: DTensor, moe_routing_indices: DTensor, moe_mask: DTensor, output: DTensor,
+                                 block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1361.  Same stage as moe_w2_linear_layer."""
+        assert input.num_dims == 3
+        self._moe_linear("gang_moe_w2_linear_mi300", input, weight, moe_routing_indices, moe_mask, output, (8, 1, 1), block_dim, 2,
+                         self._gang_moe_params(weight, 128, True))
+
+    def moe_mul_sum_add_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1411.  output = residual + sum_k weight[t, k] * input[t, k, :] in fp32."""
+        assert input.num_dims == 3  # (batch_size, num_experts_per_tok, hidden_size)
+        assert weight.num_dims == 2  # (batch_size, num_experts_per_tok)
+        assert residual.num_dims == 2 and output.num_dims == 2
+        self._task("moe_mul_sum_add_mi300", grid_dim, block_dim,
+                   [(input, (0, 2, -1), -1), (weight, (0, -1, -1), -1), (residual, (0, 1, -1), -1), (output, (0, 1, -1), -1)])
 
     def _gang_params(self, weight, tile_n, output_stride, m_tiles, wg, out_rows=None):
         batch_size = self.max_num_batched_tokens
@@ -547,9 +630,8 @@ class PersistentKernel:
             self._handle = None
         self.__finalized__ = True
 
-    def __del__(self):
-        import sys
-        if sys.is_finalizing():  # the HIP runtime may already be gone at interpreter shutdown: leave the memory to the OS
+    def __del__(self, _is_finalizing=sys.is_finalizing):
+        if _is_finalizing():  # the HIP runtime may already be gone at interpreter shutdown: leave the memory to the OS
             return
         try:
             if not self.__finalized__:

@@ -25,6 +25,13 @@ force on small shapes and invariants (scale invariance, RoPE as a complex rotati
 attention, permutation invariance, planted argmax) -- the reference holds no golden vectors for this
 path.  What stays "parity unpinned": the exact summation order inside the reference's ck_tile GEMM
 pipelines (third-party, absent from the tree); both restatements accumulate in fp32 like it does.
+
+Mixture of experts (Qwen3-30B-A3B shape): moe_route_k / moe_mlp_k restate the reference's MoE task kernels
+(moe_topk_softmax_mi300.cuh, moe_linear_mi300.cuh, moe_mul_sum_add_mi300.cuh) and are pinned against float64
+softmax + torch.topk, planted ties, a dense float64 evaluation of the same experts, and the E=1 special case that
+reduces to the dense SwiGLU MLP.  moe_block_t restates HF transformers' Qwen3MoeSparseMoeBlock (third-party,
+pinned 4.57.1 in the reference's requirements, not importable here at that version): PARITY UNPINNED beyond
+agreeing with moe_mlp_k within bf16 tolerance.
 """
 import math
 from dataclasses import dataclass
@@ -47,6 +54,10 @@ class Qwen3Config:
     rope_theta: float = 1e6
     rms_eps: float = 1e-6
     max_positions: int = 4096
+    # mixture of experts (Qwen3-30B-A3B: 128 experts, top-8, expert width 768); num_experts == 0 -> dense SwiGLU MLP
+    num_experts: int = 0
+    num_experts_per_tok: int = 0
+    moe_intermediate_size: int = 0
 
     @property
     def q_size(self):
@@ -71,11 +82,20 @@ def make_layer_weights(cfg: Qwen3Config, gen: torch.Generator, norm_std: float =
             w = w + torch.randn(n, generator=gen, dtype=torch.float32) * norm_std
         return w.to(BF16)
 
-    return {
+    w = {
         "input_norm": norm(H), "q_proj": lin(cfg.q_size, H), "k_proj": lin(cfg.kv_size, H), "v_proj": lin(cfg.kv_size, H),
-        "q_norm": norm(D), "k_norm": norm(D), "o_proj": lin(H, cfg.q_size),
-        "post_norm": norm(H), "gate_proj": lin(I, H), "up_proj": lin(I, H), "down_proj": lin(H, I),
+        "q_norm": norm(D), "k_norm": norm(D), "o_proj": lin(H, cfg.q_size), "post_norm": norm(H),
     }
+    if cfg.num_experts > 0:
+        E, MI = cfg.num_experts, cfg.moe_intermediate_size
+        # expert tensors as the reference driver packs them (demo/qwen3/demo_30B_A3B.py:376-420):
+        # gate_up_proj [E, 2*MI, H] = [gate ; up] per expert, down_proj [E, H, MI]
+        w["router"] = lin(E, H)
+        w["gate_up_proj"] = (torch.randn(E, 2 * MI, H, generator=gen, dtype=torch.float32) * 0.02).to(BF16)
+        w["down_proj"] = (torch.randn(E, H, MI, generator=gen, dtype=torch.float32) * 0.02).to(BF16)
+    else:
+        w.update({"gate_proj": lin(I, H), "up_proj": lin(I, H), "down_proj": lin(H, I)})
+    return w
 
 
 def make_model_weights(cfg: Qwen3Config, seed: int = 0, norm_std: float = 0.0):
@@ -128,6 +148,84 @@ def linear_silu_k(x, Wg, Wu):
 
 def silu_mul_k(gate_bf16, up_bf16):
     return silu_mul_f32(gate_bf16.float(), up_bf16.float()).to(BF16)
+
+
+def moe_route_k(logits_bf16, topk: int):
+    """Router of the reference's MoE path (tasks/mi300/moe_topk_softmax_mi300.cuh:124-213): fp32 softmax over ALL
+    experts, `topk` rounds of arg-max where equal probabilities go to the lower expert id, weights renormalised by
+    the sum of the selected probabilities.  Returns (weights fp32 [T, topk], experts int64 [T, topk]) in slot order."""
+    x = logits_bf16.float()
+    p = torch.exp(x - x.max(-1, keepdim=True).values)
+    p = p * (1.0 / p.sum(-1, keepdim=True))
+    T, E = p.shape
+    w = torch.zeros(T, topk, dtype=torch.float32)
+    e = torch.zeros(T, topk, dtype=torch.int64)
+    q = p.clone()
+    for s in range(topk):
+        best = q.max(-1).values
+        idx = (q == best[:, None]).float().argmax(-1)  # first (lowest) index attaining the maximum
+        w[:, s], e[:, s] = best, idx
+        q[torch.arange(T), idx] = -10000.0
+    return w * (1.0 / w.sum(-1, keepdim=True)), e
+
+
+def moe_routing_tables(experts, num_experts: int):
+    """The routing table / mask tensors the reference's router task emits (moe_topk_softmax_mi300.cuh:176-229):
+    routing[e, t] = 1 + slot if expert e serves token t else 0; mask = ids of the active experts (any order) with
+    their count at index num_experts."""
+    T, topk = experts.shape
+    routing = torch.zeros(num_experts, T, dtype=torch.int32)
+    for t in range(T):
+        for s in range(topk):
+            routing[experts[t, s], t] = s + 1
+    active = sorted(set(experts.flatten().tolist()))
+    return routing, active
+
+
+def moe_mlp_k(h, x_res, gate_up, down, weights, experts):
+    """Kernel-order expert MLP + combine on T tokens.  h: normalised input [T, H] bf16; x_res: residual [T, H] bf16;
+    gate_up [E, 2I, H], down [E, H, I].  Rounding points follow the reference's task sequence
+    (demo/qwen3/demo_30B_A3B.py:697-754): W13 output [T, topk, 2I] rounded to bf16
+    (tasks/mi300/moe_linear_mi300.cuh:53-295), SwiGLU on those bf16 values -> bf16, W2 output [T, topk, H] rounded to
+    bf16, then out = bf16(res + sum_k w_k * y_k) accumulated in fp32 in slot order
+    (tasks/mi300/moe_mul_sum_add_mi300.cuh:41-54).  Returns (out, mid, act, y)."""
+    T, topk = experts.shape
+    I2 = gate_up.shape[1]
+    H = down.shape[1]
+    mid = torch.zeros(T, topk, I2, dtype=BF16)
+    act = torch.zeros(T, topk, I2 // 2, dtype=BF16)
+    y = torch.zeros(T, topk, H, dtype=BF16)
+    out = torch.zeros(T, H, dtype=BF16)
+    for t in range(T):
+        acc = x_res[t].float()
+        for s in range(topk):
+            e = int(experts[t, s])
+            mid[t, s] = (h[t].float() @ gate_up[e].float().t()).to(BF16)
+            act[t, s] = silu_mul_k(mid[t, s, :I2 // 2], mid[t, s, I2 // 2:])
+            y[t, s] = (act[t, s].float() @ down[e].float().t()).to(BF16)
+            acc = acc + y[t, s].float() * weights[t, s]
+        out[t] = acc.to(BF16)
+    return out, mid, act, y
+
+
+def moe_block_t(h, router, gate_up, down, topk: int):
+    """torch-order sparse MoE block = HF transformers 4.57.1 Qwen3MoeSparseMoeBlock.forward with norm_topk_prob=True
+    (third-party; restated from its published algorithm, PARITY UNPINNED): bf16 router linear, fp32 softmax, top-k,
+    renormalise, routing weights cast to bf16, per-expert SwiGLU MLP in bf16 scaled by the bf16 weight and
+    index-added into a bf16 buffer in ascending expert order."""
+    T, H = h.shape
+    logits = F.linear(h, router)
+    rw = F.softmax(logits, dim=1, dtype=torch.float)
+    rw, sel = torch.topk(rw, topk, dim=-1)
+    rw = (rw / rw.sum(dim=-1, keepdim=True)).to(h.dtype)
+    out = torch.zeros(T, H, dtype=h.dtype)
+    I = gate_up.shape[1] // 2
+    for e in sorted(set(sel.flatten().tolist())):
+        tok, slot = torch.where(sel == e)
+        cur = h[tok]
+        y = F.linear(F.silu(F.linear(cur, gate_up[e, :I])) * F.linear(cur, gate_up[e, I:]), down[e])
+        out.index_add_(0, tok, (y * rw[tok, slot, None]).to(h.dtype))
+    return out
 
 
 def head_norm_rope_k(x, w, cos_row, sin_row, eps=1e-6, qk_norm=True, rope=True):
@@ -212,6 +310,9 @@ class Qwen3Oracle:
             a = torch.stack([attention_k(q[t], cache.k[li, :pos0 + t + 1], cache.v[li, :pos0 + t + 1]) for t in range(T)])
             x = linear_k(a.view(T, nq * D), W["o_proj"], res=x)
             h = rmsnorm_k(x, W["post_norm"], cfg.rms_eps)
+            if cfg.num_experts > 0:
+                wts, exp = moe_route_k(linear_k(h, W["router"]), cfg.num_experts_per_tok)
+                return moe_mlp_k(h, x, W["gate_up_proj"], W["down_proj"], wts, exp)[0]
             m = linear_silu_k(h, W["gate_proj"], W["up_proj"])
             return linear_k(m, W["down_proj"], res=x)
         # torch order
@@ -233,6 +334,8 @@ class Qwen3Oracle:
         a = a.permute(1, 0, 2).reshape(T, nq * D)
         x = x + F.linear(a, W["o_proj"])
         h = rmsnorm_t(x, W["post_norm"])
+        if cfg.num_experts > 0:
+            return x + moe_block_t(h, W["router"], W["gate_up_proj"], W["down_proj"], cfg.num_experts_per_tok)
         m = F.silu(F.linear(h, W["gate_proj"])) * F.linear(h, W["up_proj"])
         return x + F.linear(m, W["down_proj"])
 

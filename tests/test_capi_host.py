@@ -182,3 +182,66 @@ def test_lowering_rejects_bad_graphs():
     with pytest.raises(AssertionError, match="divisible"):  # gang layers need N divisible by 8 * tile_n (persistent_kernel.py:1595-1599)
         mpk4.gang_linear_layer(input=_t(mpk4, "x", 4, 1024), weight=_t(mpk4, "W", 1000, 1024), output=mpk4.new_tensor((4, 1000), name="y"),
                                tile_n=64, output_stride=1000)
+
+
+def _moe_graph(mpk, B, gang, fused_order=True):
+    H, E, topk, MI = 512, 16, 4, 128
+    x, n = mpk.new_tensor((B, H), name="x"), mpk.new_tensor((B, H), name="n")
+    nw, wr = _t(mpk, "nw", H), _t(mpk, "router", E, H)
+    w13, w2 = _t(mpk, "w13", E, 2 * MI, H), _t(mpk, "w2", E, H, MI)
+    gate = mpk.new_tensor((B, E), name="gate")
+    tw = mpk.new_tensor((B, topk), dtype=mi.float32, name="topk_w")
+    ri = mpk.new_tensor((E, B), dtype=mi.int32, name="routing")
+    mask = mpk.new_tensor((E + 1,), dtype=mi.int32, name="mask")
+    mid, act, y = mpk.new_tensor((B, topk, 2 * MI), name="mid"), mpk.new_tensor((B, topk, MI), name="act"), mpk.new_tensor((B, topk, H), name="y")
+    out = mpk.new_tensor((B, H), name="out")
+    mpk.rmsnorm_layer(input=x, weight=nw, output=n, grid_dim=(B, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_layer(input=n, weight=wr, output=gate, grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+    mpk.moe_topk_softmax_routing_layer(input=gate, output=(tw, ri, mask), grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+    if gang:
+        mpk.gang_moe_w13_linear_layer(input=n, weight=w13, moe_routing_indices=ri, moe_mask=mask, output=mid)
+    else:
+        mpk.moe_w13_linear_layer(input=n, weight=w13, moe_routing_indices=ri, moe_mask=mask, output=mid, grid_dim=(10, 2 * MI // 64, 1), block_dim=(256, 1, 1))
+    mpk.moe_silu_mul_layer(input=mid, output=act, grid_dim=(B, topk, 1), block_dim=(256, 1, 1))
+    if gang:
+        mpk.gang_moe_w2_linear_layer(input=act, weight=w2, moe_routing_indices=ri, moe_mask=mask, output=y)
+    else:
+        mpk.moe_w2_linear_layer(input=act, weight=w2, moe_routing_indices=ri, moe_mask=mask, output=y, grid_dim=(8, H // 64, 1), block_dim=(256, 1, 1))
+    mpk.moe_mul_sum_add_layer(input=y, weight=tw, residual=x, output=out, grid_dim=(B, H // 256, 1), block_dim=(256, 1, 1))
+    return dict(E=E, topk=topk, MI=MI, H=H)
+
+
+@pytest.mark.parametrize("gang", [False, True])
+def test_lowering_of_mixture_of_experts_layers(gang):
+    """The reference's MoE sequence (demo/qwen3/demo_30B_A3B.py:675-754) lowers to router linear, top-k stage (multi-token only),
+    W13 with routing + SwiGLU folded in, W2 with the combine folded in for single tokens, and a multi-token combine stage."""
+    mpk = _host_mpk(B=4, R=2)
+    d = _moe_graph(mpk, 4, gang)
+    prog = [l.split(None, 1)[1] for l in mpk.describe_program().splitlines()]
+    kinds = [l.split()[0] for l in prog]
+    assert kinds == ["NORM[multi-token", "LINEAR+norm", "MOE_TOPK[multi-token", "MOE_LINEAR+route(single", "MOE_LINEAR", "MOE_COMBINE[multi-token"]
+    assert "+silu -> act" in prog[3] and "n=256 k=512" in prog[3] and "+combine(single token) -> out" in prog[4] and "n=512 k=128" in prog[4]
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    types = {t["task_type"] for t in tg["all_tasks"]}
+    # runtime_header.h:141-146 task ids
+    assert ({174, 175} if gang else {170, 171}) <= types and {172, 173, 118} <= types
+
+
+def test_lowering_rejects_bad_moe_graphs():
+    mpk = _host_mpk(B=2, R=2)
+    H, E, topk = 256, 8, 2
+    gate = mpk.new_tensor((2, E), name="gate")
+    tw = mpk.new_tensor((2, topk), dtype=mi.float32, name="tw")
+    ri = mpk.new_tensor((E, 2), dtype=mi.int32, name="ri")
+    mask = mpk.new_tensor((E + 1,), dtype=mi.int32, name="mask")
+    mpk.moe_topk_softmax_routing_layer(input=gate, output=(tw, ri, mask), grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+    with pytest.raises(_capi.MkError, match="must be followed by the per-expert linear"):
+        mpk.describe_program()
+    mpk = _host_mpk(B=2, R=2)
+    n, w = mpk.new_tensor((2, H), name="n"), _t(mpk, "w", E, 64, H + 8)
+    ri = mpk.new_tensor((E, 2), dtype=mi.int32, name="ri")
+    mask = mpk.new_tensor((E + 1,), dtype=mi.int32, name="mask")
+    y = mpk.new_tensor((2, topk, 64), name="y")
+    mpk.moe_w13_linear_layer(input=n, weight=w, moe_routing_indices=ri, moe_mask=mask, output=y, grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+    with pytest.raises(_capi.MkError, match=r"input must be \[tokens, 264\]"):
+        mpk.describe_program()

@@ -200,3 +200,77 @@ def test_model_orders_agree_and_prefill_equals_stepwise():
     other = prompt.clone()
     other[3:] = (other[3:] + 1) % cfg.vocab_size
     same(ok.forward(other, c4, 0)[:3], lk[:3])
+
+
+def test_moe_router_matches_float64_topk_and_tie_rule():
+    """moe_route_k against an independent float64 softmax + torch.topk + renormalise (the routing
+    tests/runtime_python/blackwell/sm100_moe/test_gate_topk.py:37-52 uses as its reference), plus what the closed form
+    fixes: weights sum to 1, planted probabilities come back, equal logits go to the lower expert id."""
+    from oracle.qwen3_ref import moe_route_k, moe_routing_tables
+    g = torch.Generator().manual_seed(0)
+    T, E, k = 16, 128, 8
+    # distinct logits so that top-k is unambiguous
+    logits = (torch.randperm(T * E, generator=g).view(T, E).float() / (T * E) * 8 - 4).to(torch.bfloat16)
+    logits = torch.stack([torch.unique(r)[torch.randperm(len(torch.unique(r)), generator=g)][:96] for r in logits])  # dedupe after bf16 rounding
+    E = logits.shape[1]
+    w, e = moe_route_k(logits, k)
+    p64 = torch.softmax(logits.double(), -1)
+    tv, ti = torch.topk(p64, k, dim=-1)
+    assert torch.equal(e, ti), "selected experts (in slot order = descending probability) differ from float64 top-k"
+    torch.testing.assert_close(w.double(), tv / tv.sum(-1, keepdim=True), rtol=1e-5, atol=0)
+    torch.testing.assert_close(w.sum(-1), torch.ones(T), rtol=1e-6, atol=0)
+    # planted probabilities: logits = log(p) for a known distribution -> weights = p_topk / sum(p_topk)
+    p = torch.tensor([[0.4, 0.05, 0.3, 0.05, 0.2]])
+    w2, e2 = moe_route_k(torch.log(p).to(torch.bfloat16), 2)
+    assert e2.tolist() == [[0, 2]]
+    torch.testing.assert_close(w2, torch.tensor([[0.4 / 0.7, 0.3 / 0.7]]), rtol=2e-2, atol=0)  # bf16 logits
+    # ties: all-equal logits select experts 0..k-1 in order with weight 1/k (moe_topk_softmax_mi300.cuh:152-176)
+    w3, e3 = moe_route_k(torch.zeros(2, 10, dtype=torch.bfloat16), 3)
+    assert e3.tolist() == [[0, 1, 2], [0, 1, 2]]
+    torch.testing.assert_close(w3, torch.full((2, 3), 1 / 3), rtol=1e-6, atol=0)
+    # a tie for the LAST slot only: the lower id wins, the higher is dropped
+    lg = torch.tensor([[1.0, 3.0, 2.0, 2.0, 0.0]]).to(torch.bfloat16)
+    _, e4 = moe_route_k(lg, 2)
+    assert e4.tolist() == [[1, 2]]
+    # routing table / active list as the reference's task emits them (routing[e, t] = slot + 1)
+    routing, active = moe_routing_tables(torch.tensor([[1, 2], [2, 4]]), 5)
+    assert routing.tolist() == [[0, 0], [1, 0], [2, 1], [0, 0], [0, 2]] and active == [1, 2, 4]
+
+
+def test_moe_mlp_against_dense_float64_and_single_expert_case():
+    """moe_mlp_k against a float64 evaluation of the definition out = res + sum_k w_k * W2[e_k] (silu(Wg[e_k] h) * (Wu[e_k] h))
+    (tests/runtime_python/test_moe_linear.py:33-61 builds the same per-expert reference), and the special case of one expert
+    with weight 1, which is the dense SwiGLU MLP."""
+    from oracle.qwen3_ref import linear_k, moe_block_t, moe_mlp_k, moe_route_k, silu_mul_k
+    g = torch.Generator().manual_seed(1)
+    T, H, E, I, k = 5, 64, 6, 32, 3
+    bf = torch.bfloat16
+    h = torch.randn(T, H, generator=g).to(bf)
+    res = torch.randn(T, H, generator=g).to(bf)
+    gu = (0.2 * torch.randn(E, 2 * I, H, generator=g)).to(bf)
+    dn = (0.2 * torch.randn(E, H, I, generator=g)).to(bf)
+    router = (0.3 * torch.randn(E, H, generator=g)).to(bf)
+    w, e = moe_route_k(linear_k(h, router), k)
+    out, mid, act, y = moe_mlp_k(h, res, gu, dn, w, e)
+    ref = res.double().clone()
+    for t in range(T):
+        for s in range(k):
+            ex = int(e[t, s])
+            a = h[t].double() @ gu[ex].double().t()
+            m = torch.nn.functional.silu(a[:I]) * a[I:]
+            ref[t] += float(w[t, s]) * (m @ dn[ex].double().t())
+    torch.testing.assert_close(out.double(), ref, rtol=2e-2, atol=3e-2)
+    assert float((out.double() - ref).abs().mean()) < 6e-3  # bf16 rounding of three intermediates, not a structural error
+    # slot layout of the intermediates: [T, topk, 2I] with gate rows first (demo_30B_A3B.py:376-420 packs [gate ; up])
+    ex = int(e[2, 1])
+    torch.testing.assert_close(mid[2, 1].float(), (h[2].float() @ gu[ex].float().t()).to(bf).float())
+    assert torch.equal(act[2, 1], silu_mul_k(mid[2, 1, :I], mid[2, 1, I:]))
+    # one expert, weight 1: the dense path's unfused operators
+    w1, e1 = torch.ones(T, 1), torch.zeros(T, 1, dtype=torch.int64)
+    out1 = moe_mlp_k(h, res, gu[:1], dn[:1], w1, e1)[0]
+    m1 = linear_k(h, gu[0])
+    dense = linear_k(silu_mul_k(m1[:, :I], m1[:, I:]), dn[0])  # bf16(W2 act)
+    assert torch.equal(out1, (res.float() + dense.float()).to(bf))
+    # the torch-order block (HF algorithm) agrees with the kernel-order one within bf16 tolerance
+    blk = res + moe_block_t(h, router, gu, dn, k)
+    torch.testing.assert_close(blk.float(), out.float(), rtol=3e-2, atol=6e-2)
