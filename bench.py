@@ -33,7 +33,8 @@ def cpu_baseline(shape, n_layers_sample=2, steps=3, context=80):
     cores = min(cores, int(os.environ.get("OMP_NUM_THREADS", cores)))
     torch.set_num_threads(cores)
     cfg = Qwen3Config(hidden_size=shape.hidden_size, num_q_heads=shape.num_q_heads, num_kv_heads=shape.num_kv_heads, head_dim=shape.head_dim,
-                      intermediate_size=shape.intermediate_size, num_layers=n_layers_sample, vocab_size=shape.vocab_size, rope_theta=shape.rope_theta)
+                      intermediate_size=shape.intermediate_size, num_layers=n_layers_sample, vocab_size=shape.vocab_size, rope_theta=shape.rope_theta,
+                      num_experts=shape.num_experts, num_experts_per_tok=shape.num_experts_per_tok, moe_intermediate_size=shape.moe_intermediate_size)
     g = torch.Generator().manual_seed(0)
     w = {"layers": [make_layer_weights(cfg, g) for _ in range(n_layers_sample)]}
     w["embed"] = torch.zeros(8, cfg.hidden_size, dtype=torch.bfloat16)
@@ -88,6 +89,8 @@ def main():
     ap.add_argument("--layers", type=int, default=36)
     ap.add_argument("--prompt-length", type=int, default=80)
     ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
+    ap.add_argument("--model", choices=["qwen3-8b", "qwen3-30b-a3b"], default="qwen3-8b",
+                    help="qwen3-8b: the headline dense shape; qwen3-30b-a3b: the mixture-of-experts shape (128 experts, top-8), reported alongside")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true", help="also run one 1 GiB device-to-device copy (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     args = ap.parse_args()
@@ -104,7 +107,8 @@ def main():
         print("bench.py: no GPU visible; the megakernel has no CPU path", file=sys.stderr)
         sys.exit(1)
     torch.cuda.set_device(0)
-    shape = Qwen3Shape(num_layers=args.layers)
+    moe = args.model == "qwen3-30b-a3b"
+    shape = Qwen3Shape.qwen3_30b_a3b(min(args.layers, 48) if args.layers != 36 else 48) if moe else Qwen3Shape(num_layers=args.layers)
     B, K, W, P = args.batch, args.steps, args.warmup, args.prompt_length
     max_seq = max(1200, P + W + K + 2)
     if args.calib_copy:
@@ -143,13 +147,18 @@ def main():
     ms_per_step = wall_ms / K
     # algorithmic bytes: weights once per step + K/V rows of every cached position (positions ctx0+1 .. ctx0+K incl. the new one)
     kv_positions = sum(ctx0 + 1 + i for i in range(K))
-    bytes_total = K * shape.weight_bytes_per_token() + B * kv_positions * shape.kv_bytes_per_position()
+    # mixture of experts: a step streams the experts its tokens select; B tokens choosing top-k of E uniformly touch
+    # E * (1 - (1 - k/E)^B) distinct experts per layer in expectation (exactly k for one token)
+    distinct = None
+    if moe and B > 1:
+        distinct = shape.num_experts * (1.0 - (1.0 - shape.num_experts_per_tok / shape.num_experts) ** B)
+    bytes_total = int(K * shape.weight_bytes_per_token(distinct) + B * kv_positions * shape.kv_bytes_per_position())
     achieved = bytes_total / (kernel_ms * 1e-3) / 1e9
     out = {
-        "metric": "decode TPOT ms/token Qwen3-8B-shape bf16", "value": round(ms_per_step, 4), "unit": "ms/token", "n_gpus": 1, "steps": K,
+        "metric": f"decode TPOT ms/token {'Qwen3-30B-A3B' if moe else 'Qwen3-8B'}-shape bf16", "value": round(ms_per_step, 4), "unit": "ms/token", "n_gpus": 1, "steps": K,
         "warmup": W, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
         "data": "synthetic (random-init weights ~N(0,0.02), seeded random prompts)",
-        "config": {"workload": f"Qwen3-8B shape, {shape.num_layers} layers, vocab {shape.vocab_size}, BS={B}, prompt {P}, "
+        "config": {"workload": f"{'Qwen3-30B-A3B (128 experts, top-8)' if moe else 'Qwen3-8B'} shape, {shape.num_layers} layers, vocab {shape.vocab_size}, BS={B}, prompt {P}, "
                                f"context {ctx0}..{ctx0 + K}, max_seq_len {max_seq}, page_size 4096, graph mode {args.mode}",
                    "batch": B, "tokens_per_s": round(B * 1e3 / ms_per_step, 1), "prefill_iterations": prefill_iters},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
