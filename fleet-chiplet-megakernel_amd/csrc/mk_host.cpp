@@ -895,7 +895,7 @@ int do_launch(mk_graph *g, hipStream_t stream, int max_iters, int run_scheduler)
   HIP_TRY(hipSetDevice(g->cfg.device));
   HIP_TRY(hipMemsetAsync(g->d_sync, 0, sizeof(MkSync), stream));
   const MkRuntime *rtp = g->d_rt;
-  void *args[] = {(void *)&rtp, (void *)&max_iters, (void *)&run_scheduler};
+  void *args[] = {(void *)&g->h_rt, (void *)&rtp, (void *)&max_iters, (void *)&run_scheduler};
   HIP_TRY(hipEventRecord(g->ev0, stream));
   HIP_TRY(hipLaunchCooperativeKernel((const void *)mk_persistent_kernel, dim3(g->G), dim3(MK_THREADS), args, MK_LDS_BYTES, stream));
   HIP_TRY(hipEventRecord(g->ev1, stream));

@@ -17,6 +17,12 @@ typedef __attribute__((__vector_size__(2 * sizeof(__bf16)))) __bf16 bf16x2_t;
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float f32x4 __attribute__((ext_vector_type(4)));
 
+// Stage descriptors are written once by the host before the first launch and never by the kernel: reading them
+// through the constant address space makes every field a scalar load, so shapes, pointers and everything derived
+// from them stay in scalar registers and branches on them are scalar branches.
+typedef const __attribute__((address_space(4))) MkStage CStage;
+typedef const __attribute__((address_space(4))) MkWeight CWeight;
+
 #define MK_SPIN_LIMIT (1u << 24)
 
 // prefetch depth of the single-token linear: LDS ring bytes per workgroup and register rows per worker wavefront
@@ -157,7 +163,7 @@ __device__ __forceinline__ void barrier_poll(Ctx &c) {
 // bookkeeping after the workgroup barrier that follows barrier_poll
 __device__ __forceinline__ void barrier_done(Ctx &c) {
   c.pending = false;
-  c.dead = c.dead || (*c.sh_dead != 0);
+  c.dead = c.dead || (__builtin_amdgcn_readfirstlane(*c.sh_dead) != 0);
   c.t_wait = (long long)wall_clock64();
 }
 
@@ -278,7 +284,7 @@ __device__ int mk_prepare_next_batch(const MkRuntime &rt, int *scratch_pages) {
 }
 
 // ----------------------------------------------------------------------------- weights
-__device__ __forceinline__ const u32x4 *weight_row(const MkWeight &w, int r, int k8) {
+__device__ __forceinline__ const u32x4 *weight_row(CWeight &w, int r, int k8) {
   if (w.nseg == 1) return (const u32x4 *)w.seg[0] + (size_t)r * k8;
   const int g = r / w.group_rows;
   int o = r - g * w.group_rows;
@@ -299,7 +305,7 @@ __device__ __forceinline__ const u32x4 *weight_row(const MkWeight &w, int r, int
 // stage (weight prefetch), and the main loop posts barrier_arrive(c) when the function returns.
 
 // Gather embedding rows.  Reference task: tasks/ampere/embedding.cuh:42-72.
-__device__ __forceinline__ void stage_embed(const MkStage &st, Ctx &c, const MkRuntime &rt, int M) {
+__device__ __forceinline__ void stage_embed(CStage &st, Ctx &c, const MkRuntime &rt, int M) {
   barrier_wait(c);
   const int k8 = st.k / 8;
   for (int t = c.vid; t < M; t += c.G) {
@@ -329,7 +335,7 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 // RMSNorm of full rows, one workgroup per token row (used when an iteration has several tokens;
 // single-token iterations fuse the norm into the consuming linear).  y = bf16((x * r) * w) with
 // r = rsqrt(mean(x^2) + eps) in fp32.  Reference task: tasks/mi300/rmsnorm_mi300.cuh:37-188.
-__device__ __forceinline__ void stage_norm(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_norm(CStage &st, Ctx &c, int M, char *smem) {
   barrier_wait(c);
   float *red = (float *)smem;
   uint32_t *xs = (uint32_t *)(smem + 1024);
@@ -358,7 +364,7 @@ __device__ __forceinline__ float silu_mul(float g, float u) { return g / (1.f + 
 
 // Stage the single input row of a one-token linear in LDS as packed bf16, applying the fused RMSNorm when the
 // stage asks for it (virtual workgroup 0 also stores the normalised row, which is the norm task's output tensor).
-__device__ __forceinline__ void stage_x_m1(const MkStage &st, const Ctx &c, uint32_t *xs, float *red) {
+__device__ __forceinline__ void stage_x_m1(CStage &st, const Ctx &c, uint32_t *xs, float *red) {
   const int tid = threadIdx.x, k4 = st.k / 4;
   const unsigned long long *xin = (const unsigned long long *)st.in;
   unsigned long long *xs2 = (unsigned long long *)xs;
@@ -389,7 +395,7 @@ __device__ __forceinline__ void stage_x_m1(const MkStage &st, const Ctx &c, uint
 // Same staging done by ONE wavefront (the control wavefront of a tuned single-token linear): lane l owns the
 // 16-byte segments l, l+64, ... of the row, the sum of squares is a wavefront reduction, no workgroup barrier inside.
 template <int KL>
-__device__ __forceinline__ void stage_x_m1_wave(const MkStage &st, const Ctx &c, uint32_t *xs, int lane) {
+__device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32_t *xs, int lane) {
   const u32x4 *xin = (const u32x4 *)st.in;
   u32x4 *xs4 = (u32x4 *)xs;
   u32x4 v[KL];
@@ -439,8 +445,8 @@ __device__ __forceinline__ void stage_x_m1_wave(const MkStage &st, const Ctx &c,
 // Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:359-576).
 template <int KL, int R, bool SILU>
-__device__ __forceinline__ void stage_linear_m1_t(const MkStage &st, Ctx &c, char *smem) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int K8 = KL * 64;
   constexpr int NW = MK_WAVES - 1;                         // worker wavefronts
   constexpr int PF_BYTES = (MK_TUNE_PF_BYTES / NW) & ~1023;  // LDS ring per worker (0 = ring disabled)
@@ -560,8 +566,8 @@ __device__ __forceinline__ void stage_linear_m1_t(const MkStage &st, Ctx &c, cha
 
 // Generic single-token linear for reduction lengths that are not a multiple of 512 or have no tuned
 // instantiation: same arithmetic, no cross-barrier prefetch.
-__device__ __forceinline__ void stage_linear_m1_generic(const MkStage &st, Ctx &c, char *smem) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__device__ __forceinline__ void stage_linear_m1_generic(CStage &st, Ctx &c, char *smem) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int K = st.k, k8 = K / 8;
   uint32_t *xs = (uint32_t *)smem;
   float *red = (float *)(smem + MK_RED_OFFSET);
@@ -603,7 +609,7 @@ __device__ __forceinline__ void stage_linear_m1_generic(const MkStage &st, Ctx &
   }
 }
 
-__device__ __forceinline__ void stage_linear_m1(const MkStage &st, Ctx &c, char *smem) {
+__device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
   if (st.k == 4096) {
     if (silu) stage_linear_m1_t<8, MK_TUNE_R8, true>(st, c, smem);
@@ -628,15 +634,22 @@ __device__ __forceinline__ void stage_linear_m1(const MkStage &st, Ctx &c, char 
 // weight row) against a 32(k) x 16(m) activation fragment that comes from the L2-resident activation rows.
 // Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
+#ifndef MK_TUNE_TG
+#define MK_TUNE_TG 6
+#endif
+#ifndef MK_TUNE_NB
+#define MK_TUNE_NB 2
+#endif
 template <int MT>
-__device__ __forceinline__ void stage_linear_mfma(const MkStage &st, Ctx &c, int M, char *smem) {
-  constexpr int TG = 6;  // weight tiles per K sweep
+__device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, char *smem) {
+  constexpr int TG = MK_TUNE_TG;  // weight tiles per K sweep
+  constexpr int NB = MK_TUNE_NB;  // 64-wide k steps in flight per wavefront
   barrier_wait(c);
   // activations were produced by other workgroups: invalidate this CU's L1 once, then use cached loads so the rows
   // are shared through the XCD's L2
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   __syncthreads();
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const bool silu = st.flags & MK_F_SILU;
   const int K = st.k, k8 = K / 8;
@@ -645,6 +658,8 @@ __device__ __forceinline__ void stage_linear_mfma(const MkStage &st, Ctx &c, int
   const int t_begin = (int)(((long long)c.vid * ntiles) / c.G), t_end = (int)(((long long)(c.vid + 1) * ntiles) / c.G);
   const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
   const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
+  const bool pipe = (K & 255) == 0;  // every wavefront's K slice is a whole number of 64-wide steps
+  const int lgw = pipe ? 16 : 8;     // k elements a lane group owns per step
   const int kq = ((K / 32 + MK_WAVES - 1) / MK_WAVES) * 32;  // K slice per wavefront, multiple of 32
   const int kbeg = min(K, wave * kq), kend = min(K, kbeg + kq);
   const int half = st.silu_half;
@@ -652,7 +667,7 @@ __device__ __forceinline__ void stage_linear_mfma(const MkStage &st, Ctx &c, int
   f32x4 *red = (f32x4 *)smem;           // [waves][TG][MT][64]
   const uint16_t *xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; mt++) xrow[mt] = x + (size_t)min(mt * 16 + lr, M - 1) * ldx + lg * 8;
+  for (int mt = 0; mt < MT; mt++) xrow[mt] = x + (size_t)min(mt * 16 + lr, M - 1) * ldx + lg * lgw;
 
   for (int ot0 = t_begin; ot0 < t_end; ot0 += otg) {
     const int not_ = min(otg, t_end - ot0);       // output tiles in this sweep
@@ -667,27 +682,67 @@ __device__ __forceinline__ void stage_linear_mfma(const MkStage &st, Ctx &c, int
         const int g = o / half;
         vr = g * 2 * half + (o - g * half) + ((t & 1) ? half : 0);
       }
-      wrow[t] = (const uint16_t *)weight_row(st.w, vr, k8) + lg * 8;
+      wrow[t] = (const uint16_t *)weight_row(st.w, vr, k8) + lg * lgw;
     }
     f32x4 acc[TG][MT];
 #pragma unroll
     for (int t = 0; t < TG; t++)
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-#pragma unroll 2
-    for (int k = kbeg; k < kend; k += 32) {
-      bf16x8 a[TG], b[MT];
+    if (pipe) {
+      // 64 k per step: a lane owns 32 contiguous bytes of its weight row and of its token row (two matrix-core
+      // operands), so the four lane groups of a row cover one whole 128-byte line; NB steps are kept in flight.
+      const int nsteps = (kend - kbeg) >> 6;
+      bf16x8 a[NB][TG][2], b[NB][MT][2];
+      auto load_step = [&](int s_, bf16x8 (&aa)[TG][2], bf16x8 (&bb)[MT][2]) {
+        const int k = kbeg + (s_ << 6);
 #pragma unroll
-      for (int t = 0; t < TG; t++)
-        if (t < nt) a[t] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k));
+        for (int t = 0; t < TG; t++)
+          if (t < nt) {
+            aa[t][0] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k));
+            aa[t][1] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k + 8));
+          }
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) b[mt] = *(const bf16x8 *)(xrow[mt] + k);
-#pragma unroll
-      for (int t = 0; t < TG; t++)
-        if (t < nt) {
-#pragma unroll
-          for (int mt = 0; mt < MT; mt++) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[mt], acc[t][mt], 0, 0, 0);
+        for (int mt = 0; mt < MT; mt++) {
+          bb[mt][0] = *(const bf16x8 *)(xrow[mt] + k);
+          bb[mt][1] = *(const bf16x8 *)(xrow[mt] + k + 8);
         }
+      };
+#pragma unroll
+      for (int j = 0; j < NB; j++)
+        if (j < nsteps) load_step(j, a[j], b[j]);
+      for (int s0 = 0; s0 < nsteps; s0 += NB) {
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+          if (s0 + j < nsteps) {
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+              for (int t = 0; t < TG; t++)
+                if (t < nt) {
+#pragma unroll
+                  for (int mt = 0; mt < MT; mt++) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][t][h], b[j][mt][h], acc[t][mt], 0, 0, 0);
+                }
+            if (s0 + j + NB < nsteps) load_step(s0 + j + NB, a[j], b[j]);
+          }
+        }
+      }
+    } else {
+#pragma unroll 2
+      for (int k = kbeg; k < kend; k += 32) {
+        bf16x8 a[TG], b[MT];
+#pragma unroll
+        for (int t = 0; t < TG; t++)
+          if (t < nt) a[t] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k));
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) b[mt] = *(const bf16x8 *)(xrow[mt] + k);
+#pragma unroll
+        for (int t = 0; t < TG; t++)
+          if (t < nt) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[t], b[mt], acc[t][mt], 0, 0, 0);
+          }
+      }
     }
     __syncthreads();  // previous sweep's epilogue has finished reading LDS
 #pragma unroll
@@ -734,7 +789,7 @@ __device__ __forceinline__ void stage_linear_mfma(const MkStage &st, Ctx &c, int
 
 // Standalone SwiGLU over interleaved [gate ; up] groups (used when the graph keeps the
 // gate/up linear and the activation apart).  Reference task: tasks/mi300/silu_mul_mi300.cuh:42-184.
-__device__ __forceinline__ void stage_silu_mul(const MkStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_silu_mul(CStage &st, Ctx &c, int M) {
   barrier_wait(c);
   const int n = st.n, half = st.silu_half;
   const uint16_t *in = (const uint16_t *)st.in;
@@ -828,9 +883,9 @@ __device__ __forceinline__ void moe_route_wave(const uint16_t *logits, int E, in
 
 // Router stage for multi-token iterations: one wavefront per token writes the routing weights and the token's
 // column of the routing table.  Columns of tokens that are not part of the iteration are left alone.
-__device__ __forceinline__ void stage_moe_topk(const MkStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_moe_topk(CStage &st, Ctx &c, int M) {
   barrier_wait(c);
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   const int E = st.num_experts;
   for (int t = c.vid * MK_WAVES + wave; t < M; t += c.G * MK_WAVES) {
     int sel[4];
@@ -847,8 +902,8 @@ __device__ __forceinline__ void stage_moe_topk(const MkStage &st, Ctx &c, int M)
 // Build the active-expert list and the (token, slot) pairs of every active expert from the routing table.
 // Single-token iterations keep slot order (active expert s is the expert of slot s); multi-token iterations list
 // experts in ascending id with their tokens in ascending order.
-__device__ __forceinline__ void moe_build_lists(const MkStage &st, MoeLds *L, int M, bool r_in_lds) {
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+__device__ __forceinline__ void moe_build_lists(CStage &st, MoeLds *L, int M, bool r_in_lds) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int E = st.num_experts;
   if (M == 1) {
     if (tid <= st.topk) {  // slot s is "active expert" s; a slot no expert claims (caller-written table) stays empty
@@ -917,9 +972,9 @@ __device__ __forceinline__ void moe_build_lists(const MkStage &st, MoeLds *L, in
 // Reference tasks: moe_linear_kernel_mi300 (tasks/mi300/moe_linear_mi300.cuh:53-295), silu_mul_task_impl,
 // mul_sum_add_mi300_task_impl (tasks/mi300/moe_mul_sum_add_mi300.cuh:31-55).
 template <int KL, int R, bool SILU>
-__device__ __forceinline__ void stage_moe_linear_t(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_moe_linear_t(CStage &st, Ctx &c, int M, char *smem) {
   constexpr int NROW = SILU ? 2 : 1;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   MoeLds *L = (MoeLds *)(smem + MK_PF_OFFSET);
   const int k8 = st.k / 8;
   const bool combine = !SILU && (st.flags & MK_F_MOE_COMBINE) && M == 1;
@@ -1056,7 +1111,7 @@ __device__ __forceinline__ void stage_moe_linear_t(const MkStage &st, Ctx &c, in
   }
 }
 
-__device__ __forceinline__ void stage_moe_linear(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
   if (st.k <= 1024) {
     if (silu) stage_moe_linear_t<2, 4, true>(st, c, M, smem);
@@ -1073,7 +1128,7 @@ __device__ __forceinline__ void stage_moe_linear(const MkStage &st, Ctx &c, int 
 // Weighted sum of the expert outputs plus residual for multi-token iterations:
 // out[t, :] = bf16(res[t, :] + sum_k w[t, k] * y[t, k, :]), fp32, slots in order.
 // Reference task: mul_sum_add_mi300_task_impl (tasks/mi300/moe_mul_sum_add_mi300.cuh:31-55).
-__device__ __forceinline__ void stage_moe_combine(const MkStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_moe_combine(CStage &st, Ctx &c, int M) {
   barrier_wait(c);
   const int n = st.n, total = M * n;
   const uint16_t *in = (const uint16_t *)st.in, *res = (const uint16_t *)st.res;
@@ -1120,10 +1175,10 @@ __device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst
 // paged_attention_minimal_decode (tasks/mi300/paged_attention_decode_minimal_mi300.cuh:100-371),
 // gang_attention_split_kv_kernel (tasks/mi300/gang_attention_mi300.cuh:49-153).
 template <int QPK>
-__device__ __forceinline__ void stage_attn(const MkStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
+__device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
   barrier_wait(c);
   constexpr int D = 128;
-  const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j16 = lane & 15, gg = wave * 4 + (lane >> 4);
   const int nkv = st.num_kv_heads;
   uint16_t *qs = (uint16_t *)smem;                          // [QPK][128]
@@ -1307,7 +1362,7 @@ __device__ __forceinline__ void stage_attn(const MkStage &st, Ctx &c, const MkRu
 
 // Greedy sampling, stage 1: every workgroup scans a contiguous slice of each token's logits and keeps
 // (max, lowest index attaining it).  Reference task: tasks/mi300/argmax_mi300.cuh:78-127.
-__device__ __forceinline__ void stage_argmax_partial(const MkStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_argmax_partial(CStage &st, Ctx &c, int M, char *smem) {
   barrier_wait(c);
   float *sv = (float *)smem;
   int *si = (int *)(smem + 1024);
@@ -1317,7 +1372,7 @@ __device__ __forceinline__ void stage_argmax_partial(const MkStage &st, Ctx &c, 
   const int c0 = c.vid * per, c1 = min(n, c0 + per);
   float *pv = (float *)st.aux0;
   int *pi = (int *)st.aux1;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   for (int t = 0; t < M; t++) {
     const uint16_t *row = (const uint16_t *)st.in + (size_t)t * st.ld_in;
     float best = -INFINITY;
@@ -1363,12 +1418,12 @@ __device__ __forceinline__ void stage_argmax_partial(const MkStage &st, Ctx &c, 
 
 // Greedy sampling, stage 2: one wavefront per token reduces the per-workgroup partials.
 // Reference task: tasks/mi300/argmax_mi300.cuh:129-158.
-__device__ __forceinline__ void stage_argmax_reduce(const MkStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_argmax_reduce(CStage &st, Ctx &c, int M) {
   barrier_wait(c);
   const float *pv = (const float *)st.aux0;
   const int *pi = (const int *)st.aux1;
   long long *out = (long long *)st.out;
-  const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+  const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   for (int t = c.vid * MK_WAVES + wave; t < M; t += c.G * MK_WAVES) {
     float best = -INFINITY;
     int bi = 0x7fffffff;
@@ -1394,12 +1449,13 @@ __device__ __forceinline__ void stage_argmax_reduce(const MkStage &st, Ctx &c, i
 }
 
 // ----------------------------------------------------------------------------- the kernel
-extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel(const MkRuntime *rtp, int max_iters,
+extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel(const MkRuntime rt, const MkRuntime *rtp, int max_iters,
                                                                                 int run_scheduler) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int sh_bcast[4];
   __shared__ int sh_quota[10];
-  const MkRuntime rt = *rtp;
+  // rt arrives by value in the kernel-argument segment (scalar loads); rtp is the same structure in device memory
+  // for the one non-inlined function that takes its address (the scheduler step)
   Ctx c;
   c.G = gridDim.x;
   c.sync = rt.sync;
@@ -1435,13 +1491,15 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     sh_bcast[3] = (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
   __syncthreads();
-  c.vid = sh_bcast[0];
-  c.nxcd = sh_bcast[1];
-  c.quota = sh_bcast[2];
-  c.dead = sh_bcast[3] != 0;
-  for (int i = 0; i < 8; i++) c.quotas[i] = (unsigned)sh_quota[i];
-  c.xi = sh_quota[8];
-  c.rank = sh_quota[9];
+  // values read back from LDS are the same in every lane: tell the compiler, so that everything derived from them
+  // (tile ranges, loop bounds, guards) lives in scalar registers and branches stay scalar
+  c.vid = __builtin_amdgcn_readfirstlane(sh_bcast[0]);
+  c.nxcd = __builtin_amdgcn_readfirstlane(sh_bcast[1]);
+  c.quota = __builtin_amdgcn_readfirstlane(sh_bcast[2]);
+  c.dead = __builtin_amdgcn_readfirstlane(sh_bcast[3]) != 0;
+  for (int i = 0; i < 8; i++) c.quotas[i] = (unsigned)__builtin_amdgcn_readfirstlane(sh_quota[i]);
+  c.xi = __builtin_amdgcn_readfirstlane(sh_quota[8]);
+  c.rank = __builtin_amdgcn_readfirstlane(sh_quota[9]);
   __syncthreads();
 
   for (int it = 0; it < max_iters && !c.dead; it++) {
@@ -1449,7 +1507,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     if (run_scheduler) {
       barrier_wait(c);  // the previous iteration's sampled tokens are complete
       if (c.vid == 0 && threadIdx.x == 0) {
-        const int ntok = mk_prepare_next_batch(rt, (int *)smem);
+        const int ntok = mk_prepare_next_batch(*rtp, (int *)smem);
         if (ntok == 0) rt.sched->finished = 1;
         else rt.sched->iterations++;
         if (rt.timing && rt.sched->iterations <= rt.timing_cap) rt.timing[rt.sched->iterations] = (long long)wall_clock64();
@@ -1459,12 +1517,12 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     barrier_wait(c);
     if (threadIdx.x == 0) sh_bcast[0] = ldc_i32(&rt.sched->num_tokens);
     __syncthreads();
-    const int M = sh_bcast[0];
+    const int M = __builtin_amdgcn_readfirstlane(sh_bcast[0]);
     __syncthreads();
     if (M == 0 || c.dead) break;
 
     for (int s = 0; s < rt.num_stages && !c.dead; s++) {
-      const MkStage &st = rt.stages[s];
+      CStage &st = ((CStage *)(unsigned long long)rt.stages)[s];
       const int op = st.op, flags = st.flags;
       if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
       const long long t_in = (long long)wall_clock64();
