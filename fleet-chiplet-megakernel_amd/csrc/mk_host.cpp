@@ -1192,7 +1192,7 @@ int mk_compile(mk_graph *g) {
   const size_t units = (size_t)std::max(g->G, rt.max_tokens * max_kv) + MK_ATTN_MAX_CHUNKS;
   if ((rc = dev_alloc(g, &p, units * 8 * (128 + 2) * sizeof(float)))) return rc;
   rt.attn_part = (float *)p;
-  g->attn_cnt_n = (size_t)rt.max_tokens * max_kv;
+  g->attn_cnt_n = (size_t)rt.max_tokens * max_kv * 32;  // one 128-byte line per (token, kv head) counter
   if ((rc = dev_alloc(g, &p, sizeof(unsigned) * g->attn_cnt_n))) return rc;
   rt.attn_cnt = (unsigned *)p;
   g->timing_cap = 8192;

@@ -29,6 +29,12 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_PF_BYTES
 #define MK_TUNE_PF_BYTES 0  // measured: the ring does not pay once the poll sits on the control wavefront
 #endif
+#ifndef MK_DEBUG_ATTN
+#define MK_DEBUG_ATTN 0
+#endif
+#ifndef MK_TUNE_XFENCE
+#define MK_TUNE_XFENCE 0
+#endif
 #ifndef MK_TUNE_R8
 #define MK_TUNE_R8 4
 #endif
@@ -72,15 +78,26 @@ __device__ __forceinline__ float dot8(u32x4 a, u32x4 b, float c) {
   c = dot2(a.w, b.w, c);
   return c;
 }
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-  return v;
+// Cross-lane reductions on the DPP path (one VALU instruction per step) instead of LDS-crossbar shuffles: a
+// 16-lane row is all-reduced with rotations by 8, 4, 2, 1 (every lane ends with the row total), the four rows of a
+// wavefront are then combined through scalar lane reads.  Callers run with whole rows / whole wavefronts active.
+template <int CTRL>
+__device__ __forceinline__ float dpp_f32(float v) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_update_dpp(0, __builtin_bit_cast(int, v), CTRL, 0xF, 0xF, true));
 }
 __device__ __forceinline__ float group16_sum(float v) {
-#pragma unroll
-  for (int o = 8; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+  v += dpp_f32<0x128>(v);  // row_ror:8
+  v += dpp_f32<0x124>(v);  // row_ror:4
+  v += dpp_f32<0x122>(v);  // row_ror:2
+  v += dpp_f32<0x121>(v);  // row_ror:1
   return v;
+}
+__device__ __forceinline__ float lane_f32(float v, int l) {
+  return __builtin_bit_cast(float, __builtin_amdgcn_readlane(__builtin_bit_cast(int, v), l));
+}
+__device__ __forceinline__ float wave_sum(float v) {
+  v = group16_sum(v);
+  return (lane_f32(v, 0) + lane_f32(v, 16)) + (lane_f32(v, 32) + lane_f32(v, 48));
 }
 __device__ __forceinline__ unsigned xcc_id() {
   // HW_REG_XCC_ID (id 20), bits [3:0]
@@ -399,8 +416,16 @@ __device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32
   const u32x4 *xin = (const u32x4 *)st.in;
   u32x4 *xs4 = (u32x4 *)xs;
   u32x4 v[KL];
+#if MK_TUNE_XFENCE
+  // every workgroup reads the same few KB: one cache invalidate, then ordinary loads that share the row through the
+  // die's L2, instead of 256 workgroups each pulling it from memory with device-scope loads
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+#pragma unroll
+  for (int kc = 0; kc < KL; kc++) v[kc] = xin[kc * 64 + lane];
+#else
 #pragma unroll
   for (int kc = 0; kc < KL; kc++) v[kc] = ldc_16B(xin + kc * 64 + lane);
+#endif
   if (st.flags & MK_F_NORM) {
     float ss = 0.f;
 #pragma unroll
@@ -816,9 +841,11 @@ struct MoeLds {
 };
 
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-  for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-  return v;
+  v = fmaxf(v, dpp_f32<0x128>(v));
+  v = fmaxf(v, dpp_f32<0x124>(v));
+  v = fmaxf(v, dpp_f32<0x122>(v));
+  v = fmaxf(v, dpp_f32<0x121>(v));
+  return fmaxf(fmaxf(lane_f32(v, 0), lane_f32(v, 16)), fmaxf(lane_f32(v, 32), lane_f32(v, 48)));
 }
 
 // Route one token with one wavefront: fp32 softmax over all experts, `topk` rounds of arg-max (equal probabilities
@@ -1144,10 +1171,14 @@ __device__ __forceinline__ void stage_moe_combine(CStage &st, Ctx &c, int M) {
 
 // Per-head RMSNorm + rotate-half RoPE of one 128-wide head row by one wavefront (lane l owns elements
 // l and l+64, the two halves of a rotation pair).  The normalised value is rounded to bf16 before the
-// rotation, as in the reference (tasks/mi300/kv_cache_update_mi300.cuh:129-182).
-__device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst, const uint16_t *nw, const uint16_t *cos_row,
-                                              const uint16_t *sin_row, int flags, float eps, int lane) {
-  float x0 = bf2f(ldc_u16(src + lane)), x1 = bf2f(ldc_u16(src + lane + 64));
+// rotation, as in the reference (tasks/mi300/kv_cache_update_mi300.cuh:129-182).  Split in a load half and a
+// compute half so that a wavefront can have the loads of several rows in flight.
+__device__ __forceinline__ void head_row_load(const uint16_t *src, int lane, float &x0, float &x1) {
+  x0 = bf2f(ldc_u16(src + lane));
+  x1 = bf2f(ldc_u16(src + lane + 64));
+}
+__device__ __forceinline__ void head_row_finish(float x0, float x1, uint16_t *dst, const uint16_t *nw, const uint16_t *cos_row, const uint16_t *sin_row,
+                                                int flags, float eps, int lane) {
   if (flags & MK_F_QK_NORM) {
     const float ss = wave_sum(x0 * x0 + x1 * x1);
     const float r = rsqrtf(ss * (1.f / 128.f) + eps);
@@ -1165,19 +1196,32 @@ __device__ __forceinline__ void prep_head_row(const uint16_t *src, uint16_t *dst
   dst[lane + 64] = (uint16_t)f2bf(x1);
 }
 
+struct AttnUnit {
+  int t, h, cidx, C, start, end, p, p0, t0, new_lo, n_new, cend;
+  const int *pages;
+};
+
 // GQA decode attention with the q/k-norm, RoPE and KV append fused in front.  Work unit =
 // (token, kv head, KV chunk); chunks of one (token, kv head) are adjacent virtual workgroups so a
 // kv head stays on one XCD.  Inside a workgroup, sixteen 16-lane groups each walk every 16th
 // position of the chunk with their own online-softmax state (fp32 running max / sum, exp2 with
 // log2e folded into the scale); each lane owns 8 of the 128 head dims.  Groups are merged through
 // LDS, chunks through an HBM workspace by the last workgroup to arrive.
+//
+// The cached K/V rows of a chunk do not depend on the running iteration (positions below the request's first new
+// token were appended by earlier iterations), so the first unit's rows are requested BEFORE the grid barrier of the
+// previous stage is awaited, like the weight rows of a linear.  They are read with ordinary loads: every iteration
+// starts with a cache invalidate, rows are line-aligned per (position, head), and a row is never read in the
+// iteration that writes it (the new positions come from LDS).
 // Reference tasks: kv_cache_update_impl (tasks/mi300/kv_cache_update_mi300.cuh:41-327),
 // paged_attention_minimal_decode (tasks/mi300/paged_attention_decode_minimal_mi300.cuh:100-371),
 // gang_attention_split_kv_kernel (tasks/mi300/gang_attention_mi300.cuh:49-153).
 template <int QPK>
 __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
-  barrier_wait(c);
   constexpr int D = 128;
+  constexpr int NPRE = 4;                     // positions per lane group requested ahead
+  constexpr int DPT = QPK * D / MK_THREADS;   // merged outputs per thread (all of one head)
+  constexpr int TPH = D / DPT;                // threads per head in the merges
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j16 = lane & 15, gg = wave * 4 + (lane >> 4);
   const int nkv = st.num_kv_heads;
@@ -1194,39 +1238,102 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   const u32x4 *kc = (const u32x4 *)st.k_cache;
   const u32x4 *vc = (const u32x4 *)st.v_cache;
 
-  for (int u = c.vid; u < n_units; u += c.G) {
-    const int item = u / cmax, cidx = u - item * cmax;
-    const int t = item / nkv, h = item - t * nkv;
-    const int p = ldc_i32(&rt.tok_pos[t]), L = p + 1;
+  auto decode = [&](int u, AttnUnit &a) -> bool {
+    const int item = u / cmax;
+    a.cidx = u - item * cmax;
+    a.t = item / nkv;
+    a.h = item - a.t * nkv;
+    a.p = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_pos[a.t]));
+    const int L = a.p + 1;
     int C = (L + 63) / 64;  // at least 64 positions (4 per lane group) per chunk
-    C = C > cmax ? cmax : C;
-    if (cidx >= C) continue;
-    const int start = (int)(((long long)L * cidx) / C), end = (int)(((long long)L * (cidx + 1)) / C);
-    const int slot = ldc_i32(&rt.tok_slot[t]), t0 = ldc_i32(&rt.tok_first[t]), p0 = ldc_i32(&rt.tok_pos[t0]);
-    const int *pages = rt.kv_indices + ldc_i32(&rt.kv_indptr[slot]);
-    const int new_lo = max(start, p0);                 // new positions handled here: [new_lo, end)
-    const int n_new = end > new_lo ? end - new_lo : 0;
+    a.C = C > cmax ? cmax : C;
+    if (a.cidx >= a.C) return false;
+    a.start = (int)(((long long)L * a.cidx) / a.C);
+    a.end = (int)(((long long)L * (a.cidx + 1)) / a.C);
+    const int slot = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_slot[a.t]));
+    a.t0 = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_first[a.t]));
+    a.p0 = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_pos[a.t0]));
+    a.pages = rt.kv_indices + __builtin_amdgcn_readfirstlane(ldc_i32(&rt.kv_indptr[slot]));
+    a.new_lo = max(a.start, a.p0);  // new positions handled here: [new_lo, end)
+    a.n_new = a.end > a.new_lo ? a.end - a.new_lo : 0;
+    a.cend = min(a.end, a.p0);      // cached positions handled here: [start, cend)
+    return true;
+  };
+  auto kvoff = [&](const AttnUnit &a, int pos) -> size_t {
+    const int pg = pos / ps;
+    const size_t row = (size_t)a.pages[pg] * ps + (pos - pg * ps);
+    return (row * nkv + a.h) * (D / 8) + j16;
+  };
+
+  // ---- before the barrier: the first unit's cached rows
+  AttnUnit a0;
+  const bool have0 = c.vid < n_units && decode(c.vid, a0);
+  u32x4 pk[NPRE], pv[NPRE];
+  if (have0) {
+#pragma unroll
+    for (int i = 0; i < NPRE; i++) {
+      const int pos = a0.start + gg + 16 * i;
+      if (pos < a0.cend) {
+        const size_t off = kvoff(a0, pos);
+        pk[i] = kc[off];
+        pv[i] = vc[off];
+      }
+    }
+  }
+  barrier_wait(c);
+
+  for (int u = c.vid; u < n_units; u += c.G) {
+    AttnUnit a;
+    const bool first = u == c.vid;
+    if (first) {
+      if (!have0) continue;
+      a = a0;
+    } else if (!decode(u, a)) {
+      continue;
+    }
+    const int t = a.t, h = a.h, p = a.p, C = a.C;
     __syncthreads();  // LDS reuse across units
-    // ---- phase A: prepare q heads and the new K/V rows of this chunk
-    for (int row = wave; row < QPK + n_new; row += MK_WAVES) {
-      if (row < QPK) {
-        const uint16_t *src = (const uint16_t *)st.in + (size_t)t * st.ld_in + (size_t)h * (QPK + 2) * D + row * D;
-        prep_head_row(src, qs + row * D, (const uint16_t *)st.q_norm_w, (const uint16_t *)st.cos_tab + (size_t)p * st.ld_cos,
-                      (const uint16_t *)st.sin_tab + (size_t)p * st.ld_cos, st.flags, st.eps, lane);
-      } else {
-        const int j = row - QPK, pos = new_lo + j, tt = t0 + (pos - p0);
-        const uint16_t *src = (const uint16_t *)st.in + (size_t)tt * st.ld_in + (size_t)h * (QPK + 2) * D + QPK * D;
-        prep_head_row(src, knew + j * D, (const uint16_t *)st.k_norm_w, (const uint16_t *)st.cos_tab + (size_t)pos * st.ld_cos,
-                      (const uint16_t *)st.sin_tab + (size_t)pos * st.ld_cos, st.flags, st.eps, lane);
-        vnew[j * D + lane] = ldc_u16(src + D + lane);
-        vnew[j * D + lane + 64] = ldc_u16(src + D + lane + 64);
+    // ---- phase A: prepare q heads and the new K/V rows of this chunk, two rows per wavefront in flight
+    const int n_rows = QPK + a.n_new;
+    for (int row0 = wave; row0 < n_rows; row0 += 2 * MK_WAVES) {
+      float x0[2], x1[2];
+      const uint16_t *src[2];
+#pragma unroll
+      for (int r = 0; r < 2; r++) {
+        const int row = row0 + r * MK_WAVES;
+        if (row < n_rows) {
+          if (row < QPK) {
+            src[r] = (const uint16_t *)st.in + (size_t)t * st.ld_in + (size_t)h * (QPK + 2) * D + row * D;
+          } else {
+            const int tt = a.t0 + (a.new_lo + (row - QPK) - a.p0);
+            src[r] = (const uint16_t *)st.in + (size_t)tt * st.ld_in + (size_t)h * (QPK + 2) * D + QPK * D;
+            vnew[(row - QPK) * D + lane] = ldc_u16(src[r] + D + lane);
+            vnew[(row - QPK) * D + lane + 64] = ldc_u16(src[r] + D + lane + 64);
+          }
+          head_row_load(src[r], lane, x0[r], x1[r]);
+        }
+      }
+#pragma unroll
+      for (int r = 0; r < 2; r++) {
+        const int row = row0 + r * MK_WAVES;
+        if (row < n_rows) {
+          const bool isq = row < QPK;
+          const int pos = isq ? p : a.new_lo + (row - QPK);
+          head_row_finish(x0[r], x1[r], isq ? qs + row * D : knew + (row - QPK) * D, (const uint16_t *)(isq ? st.q_norm_w : st.k_norm_w),
+                          (const uint16_t *)st.cos_tab + (size_t)pos * st.ld_cos, (const uint16_t *)st.sin_tab + (size_t)pos * st.ld_cos, st.flags, st.eps,
+                          lane);
+        }
       }
     }
     __syncthreads();
+#if MK_DEBUG_ATTN
+    long long *dbg2 = rt.stage_prof ? rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + 5) : nullptr;
+    if (dbg2 && tid == 0) dbg2[0] = (long long)wall_clock64();
+#endif
     // the chunk that owns the newest position appends this token's K/V and publishes q
-    if (cidx == C - 1) {
-      const int j = p - new_lo;
-      const size_t rowi = (size_t)ldc_i32(&pages[p / ps]) * ps + (p % ps);
+    if (a.cidx == C - 1) {
+      const int j = p - a.new_lo;
+      const size_t rowi = (size_t)a.pages[p / ps] * ps + (p % ps);
       uint32_t *kd = (uint32_t *)st.k_cache + (rowi * nkv + h) * (D / 2);
       uint32_t *vd = (uint32_t *)st.v_cache + (rowi * nkv + h) * (D / 2);
       if (tid < 64) kd[tid] = ((const uint32_t *)(knew + j * D))[tid];
@@ -1262,24 +1369,71 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         m[hh] = mn;
       }
     };
-    const int cend = min(end, p0);
-    int pos = start + gg;
-    // two positions per group in flight
-    for (; pos + 16 < cend; pos += 32) {
-      const size_t rowa = (size_t)ldc_i32(&pages[pos / ps]) * ps + (pos % ps);
-      const size_t rowb = (size_t)ldc_i32(&pages[(pos + 16) / ps]) * ps + ((pos + 16) % ps);
-      const size_t offa = (rowa * nkv + h) * (D / 8) + j16, offb = (rowb * nkv + h) * (D / 8) + j16;
-      const u32x4 ka = ldc_16B(kc + offa), va = ldc_16B(vc + offa), kb = ldc_16B(kc + offb), vb = ldc_16B(vc + offb);
-      process(ka, va);
-      process(kb, vb);
+    // NPRE positions at a time: all scores first (independent reductions), then ONE rescale of the running state.
+    // Entries at or beyond cend hold whatever the registers held; their scores are forced to -inf (weight 0).
+    auto process_block = [&](const u32x4 (&kk)[NPRE], const u32x4 (&vv)[NPRE], int pos0) {
+      float sc[NPRE][QPK];  // scores, then softmax weights
+#pragma unroll
+      for (int i = 0; i < NPRE; i++) {
+        const bool ok = pos0 + 16 * i < a.cend;
+#pragma unroll
+        for (int hh = 0; hh < QPK; hh++) {
+          const float d = group16_sum(dot8(kk[i], qv[hh], 0.f)) * st.sm_scale_log2;
+          sc[i][hh] = ok ? d : -INFINITY;
+        }
+      }
+#pragma unroll
+      for (int hh = 0; hh < QPK; hh++) {
+        float mn = m[hh];
+#pragma unroll
+        for (int i = 0; i < NPRE; i++) mn = fmaxf(mn, sc[i][hh]);
+        const float alpha = __builtin_amdgcn_exp2f(m[hh] - mn);
+        float ps_ = 0.f;
+#pragma unroll
+        for (int i = 0; i < NPRE; i++) {
+          sc[i][hh] = __builtin_amdgcn_exp2f(sc[i][hh] - mn);
+          ps_ += sc[i][hh];
+        }
+        l[hh] = l[hh] * alpha + ps_;
+        m[hh] = mn;
+#pragma unroll
+        for (int d = 0; d < 8; d++) acc[hh][d] *= alpha;
+      }
+#pragma unroll
+      for (int i = 0; i < NPRE; i++) {
+        const bool ok = pos0 + 16 * i < a.cend;
+        const u32x4 w = vv[i];
+        float v[8] = {bf_lo(w.x), bf_hi(w.x), bf_lo(w.y), bf_hi(w.y), bf_lo(w.z), bf_hi(w.z), bf_lo(w.w), bf_hi(w.w)};
+#pragma unroll
+        for (int d = 0; d < 8; d++) v[d] = ok ? v[d] : 0.f;  // 0 * NaN from an unloaded register would poison the sum
+#pragma unroll
+        for (int hh = 0; hh < QPK; hh++) {
+#pragma unroll
+          for (int d = 0; d < 8; d++) acc[hh][d] += sc[i][hh] * v[d];
+        }
+      }
+    };
+    int pos = a.start + gg;
+    if (first) {
+      if (pos < a.cend) process_block(pk, pv, pos);
+      pos += 16 * NPRE;
     }
-    for (; pos < cend; pos += 16) {
-      const size_t rowi = (size_t)ldc_i32(&pages[pos / ps]) * ps + (pos % ps);
-      const size_t off = (rowi * nkv + h) * (D / 8) + j16;
-      process(ldc_16B(kc + off), ldc_16B(vc + off));
+    for (; pos < a.cend; pos += 16 * NPRE) {
+      u32x4 kk[NPRE], vv[NPRE];
+#pragma unroll
+      for (int i = 0; i < NPRE; i++)
+        if (pos + 16 * i < a.cend) {
+          const size_t off = kvoff(a, pos + 16 * i);
+          kk[i] = kc[off];
+          vv[i] = vc[off];
+        }
+      process_block(kk, vv, pos);
     }
-    for (int j = gg; j < n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
+    for (int j = gg; j < a.n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
     // ---- phase C: merge the 16 groups through LDS
+#if MK_DEBUG_ATTN
+    if (dbg2 && tid == 0) dbg2[1] = (long long)wall_clock64();
+#endif
 #pragma unroll
     for (int hh = 0; hh < QPK; hh++) {
       float *pp = part + (gg * QPK + hh) * 132;
@@ -1291,70 +1445,94 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
     }
     __syncthreads();
+#if MK_DEBUG_ATTN
+    if (dbg2 && tid == 0) dbg2[2] = (long long)wall_clock64();
+#endif
     float *gpart = rt.attn_part + (size_t)u * QPK * (D + 2);
     uint16_t *orow = (uint16_t *)st.out + (size_t)t * st.ld_out + (size_t)h * QPK * D;
-    for (int o = tid; o < QPK * D; o += MK_THREADS) {
-      const int hh = o >> 7, d = o & 127;
+    const int mh = tid / TPH, md = (tid - mh * TPH) * DPT;  // this thread merges dims [md, md+DPT) of head mh
+    {
       float mx = -INFINITY;
 #pragma unroll
-      for (int g = 0; g < 16; g++) mx = fmaxf(mx, part[(g * QPK + hh) * 132 + 128]);
-      float ls = 0.f, os = 0.f;
+      for (int g = 0; g < 16; g++) mx = fmaxf(mx, part[(g * QPK + mh) * 132 + 128]);
+      float ls = 0.f, os[DPT];
+#pragma unroll
+      for (int d = 0; d < DPT; d++) os[d] = 0.f;
 #pragma unroll
       for (int g = 0; g < 16; g++) {
-        const float *pp = part + (g * QPK + hh) * 132;
+        const float *pp = part + (g * QPK + mh) * 132;
         const float wgt = __builtin_amdgcn_exp2f(pp[128] - mx);
         ls += pp[129] * wgt;
-        os += pp[d] * wgt;
+#pragma unroll
+        for (int d = 0; d < DPT; d++) os[d] += pp[md + d] * wgt;
       }
       if (C == 1) {
-        orow[o] = (uint16_t)f2bf(os / ls);
+#pragma unroll
+        for (int d = 0; d < DPT; d++) orow[mh * D + md + d] = (uint16_t)f2bf(os[d] / ls);
       } else {
-        gpart[hh * (D + 2) + d] = os;
-        if (d == 0) {
-          gpart[hh * (D + 2) + D] = mx;
-          gpart[hh * (D + 2) + D + 1] = ls;
+#pragma unroll
+        for (int d = 0; d < DPT; d++) gpart[mh * (D + 2) + md + d] = os[d];
+        if (md == 0) {
+          gpart[mh * (D + 2) + D] = mx;
+          gpart[mh * (D + 2) + D + 1] = ls;
         }
       }
     }
     if (C > 1) {
       // ---- phase D: the last chunk to finish merges all chunks of this (token, kv head)
+#if MK_DEBUG_ATTN
+      long long *dbg = rt.stage_prof ? rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + 1) : nullptr;
+      if (dbg && tid == 0) dbg[0] = (long long)wall_clock64();
+#endif
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(&rt.attn_cnt[item], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+        const unsigned old = __hip_atomic_fetch_add(&rt.attn_cnt[(size_t)(u / cmax) * 32], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
         const int last = (old == (unsigned)(C - 1));
-        if (last) __hip_atomic_store(&rt.attn_cnt[item], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        if (last) __hip_atomic_store(&rt.attn_cnt[(size_t)(u / cmax) * 32], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         *sflag = last;
+#if MK_DEBUG_ATTN
+        if (dbg) dbg[1] = (long long)wall_clock64();
+#endif
       }
       __syncthreads();
       if (*sflag) {
-        // all chunk partials are read with independent device-scope loads, eight chunks in flight per thread
-        const float *ip = rt.attn_part + (size_t)item * cmax * QPK * (D + 2);
-        for (int o = tid; o < QPK * D; o += MK_THREADS) {
-          const int hh = o >> 7, d = o & 127;
-          float mx = -INFINITY, ls = 0.f, os = 0.f;
-          for (int c0 = 0; c0 < C; c0 += 8) {
-            float mv[8], lv[8], ov[8];
+        // every chunk partial is read with independent device-scope loads, sixteen chunks in flight per thread
+        const float *ip = rt.attn_part + (size_t)(u / cmax) * cmax * QPK * (D + 2);
+        float mx = -INFINITY, ls = 0.f, os[DPT];
 #pragma unroll
-            for (int j = 0; j < 8; j++) {
-              const int cc = min(c0 + j, C - 1);
-              const float *pp = ip + ((size_t)cc * QPK + hh) * (D + 2);
-              mv[j] = ldc_f32(pp + D);
-              lv[j] = ldc_f32(pp + D + 1);
-              ov[j] = ldc_f32(pp + d);
-            }
+        for (int d = 0; d < DPT; d++) os[d] = 0.f;
+        for (int c0 = 0; c0 < C; c0 += 16) {
+          float mv[16], lv[16], ov[16][DPT];
 #pragma unroll
-            for (int j = 0; j < 8; j++)
-              if (c0 + j < C) {
-                const float mn = fmaxf(mx, mv[j]);
-                const float a = __builtin_amdgcn_exp2f(mx - mn), b = __builtin_amdgcn_exp2f(mv[j] - mn);
-                ls = ls * a + lv[j] * b;
-                os = os * a + ov[j] * b;
-                mx = mn;
-              }
+          for (int j = 0; j < 16; j++) {
+            const int cc = min(c0 + j, C - 1);
+            const float *pp = ip + ((size_t)cc * QPK + mh) * (D + 2);
+            mv[j] = ldc_f32(pp + D);
+            lv[j] = ldc_f32(pp + D + 1);
+#pragma unroll
+            for (int d = 0; d < DPT; d++) ov[j][d] = ldc_f32(pp + md + d);
           }
-          orow[o] = (uint16_t)f2bf(os / ls);
+#pragma unroll
+          for (int j = 0; j < 16; j++)
+            if (c0 + j < C) {
+              const float mn = fmaxf(mx, mv[j]);
+              const float sa = __builtin_amdgcn_exp2f(mx - mn), sb = __builtin_amdgcn_exp2f(mv[j] - mn);
+              ls = ls * sa + lv[j] * sb;
+#pragma unroll
+              for (int d = 0; d < DPT; d++) os[d] = os[d] * sa + ov[j][d] * sb;
+              mx = mn;
+            }
         }
+#if MK_DEBUG_ATTN
+        if (dbg && tid == 0) dbg[2] = (long long)wall_clock64();
+#endif
+#pragma unroll
+        for (int d = 0; d < DPT; d++) orow[mh * D + md + d] = (uint16_t)f2bf(os[d] / ls);
+#if MK_DEBUG_ATTN
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        if (dbg && tid == 0) dbg[3] = (long long)wall_clock64();
+#endif
       }
     }
   }
@@ -1515,7 +1693,12 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       barrier_arrive(c);
     }
     barrier_wait(c);
-    if (threadIdx.x == 0) sh_bcast[0] = ldc_i32(&rt.sched->num_tokens);
+    // one cache invalidate per iteration: whatever this CU's L1 or this die's L2 kept from earlier iterations
+    // (KV rows, page tables) is dropped, so this iteration's ordinary loads of such data see what was written back
+    if (threadIdx.x == 0) {
+      __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      sh_bcast[0] = ldc_i32(&rt.sched->num_tokens);
+    }
     __syncthreads();
     const int M = __builtin_amdgcn_readfirstlane(sh_bcast[0]);
     __syncthreads();

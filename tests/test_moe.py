@@ -199,20 +199,24 @@ def test_moe_bs1_greedy_matches_oracle_teacher_forced(mode):
     orc = Qwen3Oracle(cfg, w, "kernel")
     cache = KVCache(cfg, max_seq)
     toks = prompt.tolist()
-    n_margin = 0
+    n_margin = n_compared = 0
     for it in range(P + NEW - 1):
         dec.mpk.run_steps(1)
         gpu_logits = dec.logits()[0].float().cpu()
         gpu_tok = int(dec.meta["output_tokens"][0, 0].item())
         ref_logits = orc.forward(torch.tensor([toks[it]]), cache, it)[0].float()
-        torch.testing.assert_close(gpu_logits, ref_logits, atol=2e-2, rtol=1e-2)
-        top2 = ref_logits.topk(2).values
-        if float(top2[0] - top2[1]) > 0.05:
-            assert gpu_tok == int(argmax_k(ref_logits[None].to(torch.bfloat16))[0]), f"argmax mismatch at iteration {it}"
-            n_margin += 1
+        # top-k routing is discontinuous: a step where some layer's k-th and (k+1)-th router probabilities are within 1% of each
+        # other (a bf16 rounding of the logits) may legitimately pick another expert; such steps are not compared
+        if min(orc.route_margins) > 0.01:
+            torch.testing.assert_close(gpu_logits, ref_logits, atol=2e-2, rtol=1e-2)
+            n_compared += 1
+            top2 = ref_logits.topk(2).values
+            if float(top2[0] - top2[1]) > 0.05:
+                assert gpu_tok == int(argmax_k(ref_logits[None].to(torch.bfloat16))[0]), f"argmax mismatch at iteration {it}"
+                n_margin += 1
         if it + 1 >= P:
             toks.append(gpu_tok)
-    assert n_margin > 0
+    assert n_margin > 0 and n_compared >= (P + NEW - 1) // 2
     assert dec.mpk.run_steps(4)
     assert dec.meta["tokens"][0].cpu().tolist()[:P + NEW] == toks[:P + NEW]
     dec.mpk.finalize()
@@ -239,7 +243,7 @@ def test_moe_batched_decode_continuous_batching():
         lg = orc.forward(torch.tensor(tk[:P]), cache, 0)[-1:]
         for p in range(P, max_seq):
             top2 = lg[0].float().topk(2).values
-            if float(top2[0] - top2[1]) > 0.05:
+            if float(top2[0] - top2[1]) > 0.05 and min(orc.route_margins) > 0.01:
                 assert tk[p] == int(argmax_k(lg)[0]), f"request {r}: token at position {p} differs from the oracle"
                 hits += 1
             if p + 1 < max_seq:
