@@ -1181,20 +1181,28 @@ int mk_compile(mk_graph *g) {
   rt.sched = g->d_sched = (MkSched *)p;
   if ((rc = dev_alloc(g, &p, sizeof(MkSync)))) return rc;
   rt.sync = g->d_sync = (MkSync *)p;
+  // attention split-KV workspace: one partial (max, sum, 128 values) per q head of every work unit, a buffer of its
+  // own for every attention stage (a partial address is then written once per iteration), and two sets of arrival
+  // counters (device scope / die-local), one 128-byte line per (token, kv head)
+  int max_kv = 1;
+  for (auto &s : g->stages)
+    if (s.op == MK_OP_ATTN && s.num_kv_heads > max_kv) max_kv = s.num_kv_heads;
+  g->attn_cnt_n = (size_t)rt.max_tokens * max_kv * 32 * 2;
+  if ((rc = dev_alloc(g, &p, sizeof(unsigned) * g->attn_cnt_n))) return rc;
+  rt.attn_cnt = (unsigned *)p;
+  rt.attn_part = nullptr;
+  for (auto &s : g->stages)
+    if (s.op == MK_OP_ATTN) {
+      const size_t units = (size_t)std::max(g->G, rt.max_tokens * s.num_kv_heads) + MK_ATTN_MAX_CHUNKS;
+      const int qpk = s.num_q_heads / s.num_kv_heads;
+      if ((rc = dev_alloc(g, &p, units * qpk * (128 + 2) * sizeof(float), false))) return rc;
+      s.aux0 = p;
+      s.aux1 = rt.attn_cnt + g->attn_cnt_n / 2;
+    }
   if ((rc = dev_alloc(g, &p, sizeof(MkStage) * (g->stages.size() + 1)))) return rc;
   g->d_stages = (MkStage *)p;
   rt.stages = g->d_stages;
   if (!g->stages.empty()) HIP_TRY(hipMemcpy(g->d_stages, g->stages.data(), sizeof(MkStage) * g->stages.size(), hipMemcpyHostToDevice));
-  // attention split-KV workspace: one partial (max, sum, 128 values) per q head of every work unit
-  int max_kv = 1;
-  for (auto &s : g->stages)
-    if (s.op == MK_OP_ATTN && s.num_kv_heads > max_kv) max_kv = s.num_kv_heads;
-  const size_t units = (size_t)std::max(g->G, rt.max_tokens * max_kv) + MK_ATTN_MAX_CHUNKS;
-  if ((rc = dev_alloc(g, &p, units * 8 * (128 + 2) * sizeof(float)))) return rc;
-  rt.attn_part = (float *)p;
-  g->attn_cnt_n = (size_t)rt.max_tokens * max_kv * 32;  // one 128-byte line per (token, kv head) counter
-  if ((rc = dev_alloc(g, &p, sizeof(unsigned) * g->attn_cnt_n))) return rc;
-  rt.attn_cnt = (unsigned *)p;
   g->timing_cap = 8192;
   if ((rc = dev_alloc(g, &p, sizeof(long long) * (g->timing_cap + 2)))) return rc;
   rt.timing = g->d_timing = (long long *)p;

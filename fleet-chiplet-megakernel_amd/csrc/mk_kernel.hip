@@ -32,6 +32,15 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_DEBUG_ATTN
 #define MK_DEBUG_ATTN 0
 #endif
+#ifndef MK_DEBUG_LIN
+#define MK_DEBUG_LIN 0
+#endif
+#ifndef MK_TUNE_EVEN
+#define MK_TUNE_EVEN 1
+#endif
+#ifndef MK_TUNE_LOCALMERGE
+#define MK_TUNE_LOCALMERGE 1
+#endif
 #ifndef MK_TUNE_XFENCE
 #define MK_TUNE_XFENCE 0
 #endif
@@ -57,6 +66,13 @@ struct Ctx {
   long long t_wait;  // (profiling) tick at which the last barrier_wait completed
   int *sh_dead;
   MkSync *sync;
+  const int *sh_tok;  // LDS copy of this iteration's token metadata: [0] position, [1] batch slot, [2] first token of the request, [3] first page-table entry
+  bool even_xcds;     // every die in use runs the same number of workgroups, so die index = vid / quota
+  int *sh_ticket;     // two LDS work counters, used alternately by consecutive executed stages
+  int seq;            // stages executed so far by this workgroup
+#if MK_DEBUG_LIN
+  long long *dbg;     // four debug timestamps of the instrumented stage
+#endif
 };
 
 // ----------------------------------------------------------------------------- small helpers
@@ -151,6 +167,8 @@ __device__ __forceinline__ bool spin_ok(MkSync *s, unsigned &spins, unsigned whe
 __device__ __forceinline__ void barrier_arrive(Ctx &c) {
   MkSync *s = c.sync;
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+  c.seq++;
+  if (threadIdx.x == 0) c.sh_ticket[c.seq & 1] = 0;  // the counter of the stage that starts now (last used two stages ago)
   __syncthreads();
   c.epoch++;
   if (threadIdx.x == 0) __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
@@ -412,7 +430,7 @@ __device__ __forceinline__ void stage_x_m1(CStage &st, const Ctx &c, uint32_t *x
 // Same staging done by ONE wavefront (the control wavefront of a tuned single-token linear): lane l owns the
 // 16-byte segments l, l+64, ... of the row, the sum of squares is a wavefront reduction, no workgroup barrier inside.
 template <int KL>
-__device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32_t *xs, int lane) {
+__device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32_t *xs, int lane, const u32x4 (&nwv)[KL]) {
   const u32x4 *xin = (const u32x4 *)st.in;
   u32x4 *xs4 = (u32x4 *)xs;
   u32x4 v[KL];
@@ -438,11 +456,10 @@ __device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32
     }
     ss = wave_sum(ss);
     const float r = rsqrtf(ss / (float)(KL * 512) + st.eps);
-    const u32x4 *nw = (const u32x4 *)st.norm_w;
     u32x4 *no = (c.vid == 0) ? (u32x4 *)st.norm_out : nullptr;
 #pragma unroll
     for (int kc = 0; kc < KL; kc++) {
-      const u32x4 g = nw[kc * 64 + lane];
+      const u32x4 g = nwv[kc];  // norm weights were requested before the barrier was awaited
       u32x4 y;
 #pragma unroll
       for (int e = 0; e < 4; e++) y[e] = pack2((bf_lo(v[kc][e]) * r) * bf_lo(g[e]), (bf_hi(v[kc][e]) * r) * bf_hi(g[e]));
@@ -473,58 +490,72 @@ template <int KL, int R, bool SILU>
 __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int K8 = KL * 64;
-  constexpr int NW = MK_WAVES - 1;                         // worker wavefronts
-  constexpr int PF_BYTES = (MK_TUNE_PF_BYTES / NW) & ~1023;  // LDS ring per worker (0 = ring disabled)
-  constexpr int NPF = PF_BYTES / (KL * 1024);              // rows per worker prefetched straight into LDS
+  constexpr int NROW = SILU ? 2 : 1;  // weight rows per output ([gate ; up] pair)
+  constexpr int U = R / NROW;         // outputs in flight per worker wavefront
   uint32_t *xs = (uint32_t *)smem;
   const bool ctrl = wave == 0;
-  const int ww = ctrl ? 0 : wave - 1;
-  char *pf_base = smem + MK_PF_OFFSET + ww * PF_BYTES;
-  const u32x4 *pf = (const u32x4 *)pf_base;
   const int n_out = SILU ? st.n / 2 : st.n;
-  const int nwaves = c.G * NW;
-  const int rpw = (n_out + nwaves - 1) / nwaves;
-  const int r0 = __builtin_amdgcn_readfirstlane((c.vid * NW + ww) * rpw);
-  const int r1 = min(n_out, r0 + rpw);
-  const int nw = ctrl ? 0 : max(0, r1 - r0) * (SILU ? 2 : 1);  // weight rows this wavefront streams
+  // The workgroup owns a contiguous range of outputs; its three worker wavefronts draw them one at a time from an LDS
+  // ticket counter, so all three stream until the range is exhausted however the CU's memory pipeline favours them.
+  const int oq = n_out / c.G, orem = n_out - oq * c.G;
+  const int o_begin = c.vid * oq + min(c.vid, orem), o_end = o_begin + oq + (c.vid < orem ? 1 : 0);
+  int *ticket = c.sh_ticket + (c.seq & 1);
   const int half = st.silu_half;
-  auto rowptr = [&](int i) -> const u32x4 * {
-    int vr;
-    if (SILU) {
-      const int o = r0 + (i >> 1);
-      const int g = o / half;
-      vr = g * 2 * half + (o - g * half) + ((i & 1) ? half : 0);
-    } else {
-      vr = r0 + i;
-    }
-    return weight_row(st.w, vr, K8) + lane;
+  auto take = [&]() -> int {  // next output index of this workgroup, or -1
+    int t = 0;
+    if (lane == 0) t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    t = __builtin_amdgcn_readfirstlane(t) + o_begin;
+    return t < o_end ? t : -1;
   };
-  const int npf = min(NPF, nw);
-  u32x4 buf[R][KL];
-  if (!ctrl) {
-    for (int j = 0; j < npf; j++) {
-      const u32x4 *p = rowptr(j);
-#pragma unroll
-      for (int kc = 0; kc < KL; kc++)
-        __builtin_amdgcn_global_load_lds((const void *)(p + kc * 64), (__attribute__((address_space(3))) void *)(pf_base + (j * KL + kc) * 1024), 16, 0, 0);
+  auto load_unit = [&](int o, u32x4 (&b)[NROW][KL]) {
+    int vr = o;
+    if (SILU) {
+      const int g = o / half;
+      vr = g * 2 * half + (o - g * half);
     }
 #pragma unroll
-    for (int j = 0; j < R; j++)
-      if (npf + j < nw) {
-        const u32x4 *p = rowptr(npf + j);
+    for (int h = 0; h < NROW; h++) {
+      const u32x4 *p = weight_row(st.w, vr + h * half, K8) + lane;
 #pragma unroll
-        for (int kc = 0; kc < KL; kc++) buf[j][kc] = ldg_stream(p + kc * 64);
-      }
+      for (int kc = 0; kc < KL; kc++) b[h][kc] = ldg_stream(p + kc * 64);
+    }
+  };
+  u32x4 buf[U][NROW][KL];
+  int uo[U];
+  if (!ctrl) {
+    // weights do not depend on the previous stage: the first U outputs' rows are requested before its barrier completes
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      uo[j] = take();
+      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+    }
   } else {
+    u32x4 nwv[KL];
+    if (st.flags & MK_F_NORM) {
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) nwv[kc] = ((const u32x4 *)st.norm_w)[kc * 64 + lane];
+    }
     if (c.pending && tid == 0) barrier_poll(c);
-    stage_x_m1_wave<KL>(st, c, xs, lane);
+#if MK_DEBUG_LIN
+    if (tid == 0 && c.dbg) c.dbg[0] = (long long)wall_clock64();
+#endif
+    stage_x_m1_wave<KL>(st, c, xs, lane, nwv);
+#if MK_DEBUG_LIN
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (tid == 0 && c.dbg) c.dbg[1] = (long long)wall_clock64();
+#endif
   }
   __syncthreads();
   barrier_done(c);
   if (ctrl) return;
-  // residual values of this wavefront's rows, one per lane, fetched once up front
-  float resv = 0.f;
-  if ((st.flags & MK_F_RES) && r0 + lane < r1) resv = bf2f(ldc_u16((const uint16_t *)st.res + r0 + lane));
+#if MK_DEBUG_LIN
+  if (tid == 64 && c.dbg) c.dbg[2] = (long long)wall_clock64();
+#endif
+  const bool has_res = st.flags & MK_F_RES;
+  const uint16_t *res = (const uint16_t *)st.res;
+  float ures[U];
+#pragma unroll
+  for (int j = 0; j < U; j++) ures[j] = (has_res && uo[j] >= 0) ? bf2f(ldc_u16(res + uo[j])) : 0.f;
   const u32x4 *xs4 = (const u32x4 *)xs;
   u32x4 xr[KL <= 8 ? KL : 1];
   if (KL <= 8) {
@@ -532,61 +563,37 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
     for (int kc = 0; kc < (KL <= 8 ? KL : 1); kc++) xr[kc] = xs4[kc * 64 + lane];
   }
   uint16_t *out = (uint16_t *)st.out;
-  float gate = 0.f, outv = 0.f;
-  int obase = 0;  // outputs [obase, obase+64) of this wavefront are collected in lanes before being stored
-  auto finish_row = [&](int idx, float a) {
-    a = wave_sum(a);
-    int o;
-    float v;
-    bool have = true;
-    if (SILU) {
-      o = idx >> 1;
-      if ((idx & 1) == 0) {
-        gate = a;
-        have = false;
-      }
-      v = silu_mul(gate, a);
-    } else {
-      o = idx;
-      v = a + __shfl(resv, o & 63, 64);
-    }
-    if (have) {
-      if (o - obase >= 64) {
-        out[r0 + obase + lane] = (uint16_t)f2bf(outv);
-        obase += 64;
-      }
-      if (lane == o - obase) outv = v;
-    }
-  };
-  // LDS ring rows: wait for the direct-to-LDS loads (issued first, so they are the oldest in the queue)
-  if (npf > 0) {
-    if ((st.flags & MK_F_RES) || nw - npf < R) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    else asm volatile("s_waitcnt vmcnt(%0)" ::"n"(R * KL) : "memory");  // all but the R*KL youngest (register) loads
-  }
-  for (int i = 0; i < npf; i++) {
-    float a = 0.f;
+  while (true) {
+    bool any = false;
 #pragma unroll
-    for (int kc = 0; kc < KL; kc++) a = dot8(pf[(i * KL + kc) * 64 + lane], KL <= 8 ? xr[KL <= 8 ? kc : 0] : xs4[kc * 64 + lane], a);
-    finish_row(i, a);
-  }
-  for (int i = npf; i < nw; i += R) {
+    for (int j = 0; j < U; j++) {
+      if (uo[j] >= 0) {
+        any = true;
+        float a[NROW];
 #pragma unroll
-    for (int j = 0; j < R; j++) {
-      if (i + j < nw) {
-        float a = 0.f;
+        for (int h = 0; h < NROW; h++) {
+          a[h] = 0.f;
 #pragma unroll
-        for (int kc = 0; kc < KL; kc++) a = dot8(buf[j][kc], KL <= 8 ? xr[KL <= 8 ? kc : 0] : xs4[kc * 64 + lane], a);
-        if (i + j + R < nw) {
-          const u32x4 *p = rowptr(i + j + R);
-#pragma unroll
-          for (int kc = 0; kc < KL; kc++) buf[j][kc] = ldg_stream(p + kc * 64);
+          for (int kc = 0; kc < KL; kc++) a[h] = dot8(buf[j][h][kc], KL <= 8 ? xr[KL <= 8 ? kc : 0] : xs4[kc * 64 + lane], a[h]);
         }
-        finish_row(i + j, a);
+        const int o = uo[j];
+        const float r = ures[j];
+        uo[j] = take();
+        if (uo[j] >= 0) {
+          load_unit(uo[j], buf[j]);
+          if (has_res) ures[j] = bf2f(ldc_u16(res + uo[j]));
+        }
+#pragma unroll
+        for (int h = 0; h < NROW; h++) a[h] = wave_sum(a[h]);
+        const float v = SILU ? silu_mul(a[0], a[NROW - 1]) : a[0] + r;
+        if (lane == 0) out[o] = (uint16_t)f2bf(v);
       }
     }
+    if (!any) break;
   }
-  const int n_o = max(0, r1 - r0);
-  if (obase + lane < n_o) out[r0 + obase + lane] = (uint16_t)f2bf(outv);
+#if MK_DEBUG_LIN
+  if (tid == 64 && c.dbg) c.dbg[3] = (long long)wall_clock64();
+#endif
 }
 
 // Generic single-token linear for reduction lengths that are not a multiple of 512 or have no tuned
@@ -1243,17 +1250,16 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     a.cidx = u - item * cmax;
     a.t = item / nkv;
     a.h = item - a.t * nkv;
-    a.p = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_pos[a.t]));
+    a.p = __builtin_amdgcn_readfirstlane(c.sh_tok[a.t]);
     const int L = a.p + 1;
     int C = (L + 63) / 64;  // at least 64 positions (4 per lane group) per chunk
     a.C = C > cmax ? cmax : C;
     if (a.cidx >= a.C) return false;
     a.start = (int)(((long long)L * a.cidx) / a.C);
     a.end = (int)(((long long)L * (a.cidx + 1)) / a.C);
-    const int slot = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_slot[a.t]));
-    a.t0 = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_first[a.t]));
-    a.p0 = __builtin_amdgcn_readfirstlane(ldc_i32(&rt.tok_pos[a.t0]));
-    a.pages = rt.kv_indices + __builtin_amdgcn_readfirstlane(ldc_i32(&rt.kv_indptr[slot]));
+    a.t0 = __builtin_amdgcn_readfirstlane(c.sh_tok[2 * MK_MAX_TOKENS + a.t]);
+    a.p0 = __builtin_amdgcn_readfirstlane(c.sh_tok[a.t0]);
+    a.pages = rt.kv_indices + __builtin_amdgcn_readfirstlane(c.sh_tok[3 * MK_MAX_TOKENS + a.t]);
     a.new_lo = max(a.start, a.p0);  // new positions handled here: [new_lo, end)
     a.n_new = a.end > a.new_lo ? a.end - a.new_lo : 0;
     a.cend = min(a.end, a.p0);      // cached positions handled here: [start, cend)
@@ -1448,7 +1454,12 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
 #if MK_DEBUG_ATTN
     if (dbg2 && tid == 0) dbg2[2] = (long long)wall_clock64();
 #endif
-    float *gpart = rt.attn_part + (size_t)u * QPK * (D + 2);
+    // When every chunk of this (token, kv head) runs on one die, the partials and the arrival counter never leave that
+    // die's L2: workgroup-scope atomic, ordinary stores and loads (each stage has its own partial buffer and the L1 is
+    // invalidated once per iteration, so a partial is never read from a stale line).  Otherwise device scope.
+    const int item = u / cmax;
+    const bool local = MK_TUNE_LOCALMERGE && c.even_xcds && (item * cmax) / c.quota == (item * cmax + C - 1) / c.quota;
+    float *gpart = (float *)st.aux0 + (size_t)u * QPK * (D + 2);
     uint16_t *orow = (uint16_t *)st.out + (size_t)t * st.ld_out + (size_t)h * QPK * D;
     const int mh = tid / TPH, md = (tid - mh * TPH) * DPT;  // this thread merges dims [md, md+DPT) of head mh
     {
@@ -1487,9 +1498,16 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) {
-        const unsigned old = __hip_atomic_fetch_add(&rt.attn_cnt[(size_t)(u / cmax) * 32], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
-        const int last = (old == (unsigned)(C - 1));
-        if (last) __hip_atomic_store(&rt.attn_cnt[(size_t)(u / cmax) * 32], 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        int last;
+        if (local) {
+          unsigned *cnt = (unsigned *)st.aux1 + (size_t)item * 32;
+          last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_WORKGROUP) == (unsigned)(C - 1);
+          if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+        } else {
+          unsigned *cnt = &rt.attn_cnt[(size_t)item * 32];
+          last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(C - 1);
+          if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
         *sflag = last;
 #if MK_DEBUG_ATTN
         if (dbg) dbg[1] = (long long)wall_clock64();
@@ -1498,7 +1516,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       __syncthreads();
       if (*sflag) {
         // every chunk partial is read with independent device-scope loads, sixteen chunks in flight per thread
-        const float *ip = rt.attn_part + (size_t)(u / cmax) * cmax * QPK * (D + 2);
+        const float *ip = (const float *)st.aux0 + (size_t)item * cmax * QPK * (D + 2);
         float mx = -INFINITY, ls = 0.f, os[DPT];
 #pragma unroll
         for (int d = 0; d < DPT; d++) os[d] = 0.f;
@@ -1508,10 +1526,17 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
           for (int j = 0; j < 16; j++) {
             const int cc = min(c0 + j, C - 1);
             const float *pp = ip + ((size_t)cc * QPK + mh) * (D + 2);
-            mv[j] = ldc_f32(pp + D);
-            lv[j] = ldc_f32(pp + D + 1);
+            if (local) {
+              mv[j] = pp[D];
+              lv[j] = pp[D + 1];
 #pragma unroll
-            for (int d = 0; d < DPT; d++) ov[j][d] = ldc_f32(pp + md + d);
+              for (int d = 0; d < DPT; d++) ov[j][d] = pp[md + d];
+            } else {
+              mv[j] = ldc_f32(pp + D);
+              lv[j] = ldc_f32(pp + D + 1);
+#pragma unroll
+              for (int d = 0; d < DPT; d++) ov[j][d] = ldc_f32(pp + md + d);
+            }
           }
 #pragma unroll
           for (int j = 0; j < 16; j++)
@@ -1632,6 +1657,8 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int sh_bcast[4];
   __shared__ int sh_quota[10];
+  __shared__ int sh_tok[4][MK_MAX_TOKENS];
+  __shared__ int sh_ticket[2];
   // rt arrives by value in the kernel-argument segment (scalar loads); rtp is the same structure in device memory
   // for the one non-inlined function that takes its address (the scheduler step)
   Ctx c;
@@ -1643,6 +1670,10 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.dead = false;
   c.t_wait = 0;
   c.sh_dead = &sh_bcast[3];
+  c.sh_tok = &sh_tok[0][0];
+  c.sh_ticket = sh_ticket;
+  c.seq = 0;
+  if (threadIdx.x == 0) sh_ticket[0] = sh_ticket[1] = 0;
   // ---- XCD discovery: rank of this workgroup inside its die, dies in use, workgroups per die
   if (threadIdx.x == 0) {
     MkSync *s = rt.sync;
@@ -1678,6 +1709,8 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   for (int i = 0; i < 8; i++) c.quotas[i] = (unsigned)__builtin_amdgcn_readfirstlane(sh_quota[i]);
   c.xi = __builtin_amdgcn_readfirstlane(sh_quota[8]);
   c.rank = __builtin_amdgcn_readfirstlane(sh_quota[9]);
+  c.even_xcds = true;
+  for (int i = 0; i < 8; i++) c.even_xcds = c.even_xcds && (c.quotas[i] == 0 || c.quotas[i] == (unsigned)c.quota);
   __syncthreads();
 
   for (int it = 0; it < max_iters && !c.dead; it++) {
@@ -1701,6 +1734,14 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     }
     __syncthreads();
     const int M = __builtin_amdgcn_readfirstlane(sh_bcast[0]);
+    // token metadata of this iteration, read once (it is on the critical path of every attention stage otherwise)
+    if ((int)threadIdx.x < M) {
+      const int t = threadIdx.x, slot = ldc_i32(&rt.tok_slot[t]);
+      sh_tok[0][t] = ldc_i32(&rt.tok_pos[t]);
+      sh_tok[1][t] = slot;
+      sh_tok[2][t] = ldc_i32(&rt.tok_first[t]);
+      sh_tok[3][t] = ldc_i32(&rt.kv_indptr[slot]);
+    }
     __syncthreads();
     if (M == 0 || c.dead) break;
 
@@ -1709,6 +1750,9 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       const int op = st.op, flags = st.flags;
       if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
       const long long t_in = (long long)wall_clock64();
+#if MK_DEBUG_LIN
+      c.dbg = (rt.stage_prof && s == MK_DEBUG_LIN) ? rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + 1) : nullptr;
+#endif
       switch (op) {
         case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
