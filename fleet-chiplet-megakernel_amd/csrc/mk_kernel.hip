@@ -35,6 +35,9 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_DEBUG_LIN
 #define MK_DEBUG_LIN 0
 #endif
+#ifndef MK_TUNE_WT
+#define MK_TUNE_WT 1
+#endif
 #ifndef MK_TUNE_EVEN
 #define MK_TUNE_EVEN 1
 #endif
@@ -70,6 +73,7 @@ struct Ctx {
   bool even_xcds;     // every die in use runs the same number of workgroups, so die index = vid / quota
   int *sh_ticket;     // two LDS work counters, used alternately by consecutive executed stages
   int seq;            // stages executed so far by this workgroup
+  bool wrote_through; // the stage that just ran wrote all its outputs with write-through stores: no L2 write-back at its barrier
 #if MK_DEBUG_LIN
   long long *dbg;     // four debug timestamps of the instrumented stage
 #endif
@@ -138,6 +142,14 @@ __device__ __forceinline__ u32x4 ldc_16B(const u32x4 *p) {
   u32x4 r = {(uint32_t)a, (uint32_t)(a >> 32), (uint32_t)b, (uint32_t)(b >> 32)};
   return r;
 }
+// Stores that are written through to memory (device scope), for outputs of stages that skip the L2 write-back at
+// their barrier.
+__device__ __forceinline__ void stc_u16(uint16_t *p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void stc_16B(u32x4 *p, u32x4 v) {
+  unsigned long long *q = (unsigned long long *)p;
+  __hip_atomic_store(q, (unsigned long long)v.x | ((unsigned long long)v.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  __hip_atomic_store(q + 1, (unsigned long long)v.z | ((unsigned long long)v.w << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ uint16_t ldc_u16(const uint16_t *p) {
   const uintptr_t a = (uintptr_t)p;
   const uint32_t w = ldc_u32((const void *)(a & ~(uintptr_t)3));
@@ -171,7 +183,14 @@ __device__ __forceinline__ void barrier_arrive(Ctx &c) {
   if (threadIdx.x == 0) c.sh_ticket[c.seq & 1] = 0;  // the counter of the stage that starts now (last used two stages ago)
   __syncthreads();
   c.epoch++;
-  if (threadIdx.x == 0) __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  if (threadIdx.x == 0) {
+#if MK_TUNE_WT
+    if (c.wrote_through) __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    else
+#endif
+      __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
+  }
+  c.wrote_through = false;
   c.pending = true;
 }
 
@@ -464,7 +483,7 @@ __device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32
 #pragma unroll
       for (int e = 0; e < 4; e++) y[e] = pack2((bf_lo(v[kc][e]) * r) * bf_lo(g[e]), (bf_hi(v[kc][e]) * r) * bf_hi(g[e]));
       xs4[kc * 64 + lane] = y;
-      if (no) no[kc * 64 + lane] = y;
+      if (no) stc_16B(no + kc * 64 + lane, y);
     }
   } else {
 #pragma unroll
@@ -540,17 +559,14 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
     if (tid == 0 && c.dbg) c.dbg[0] = (long long)wall_clock64();
 #endif
     stage_x_m1_wave<KL>(st, c, xs, lane, nwv);
-#if MK_DEBUG_LIN
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (tid == 0 && c.dbg) c.dbg[1] = (long long)wall_clock64();
-#endif
+
   }
   __syncthreads();
   barrier_done(c);
-  if (ctrl) return;
-#if MK_DEBUG_LIN
-  if (tid == 64 && c.dbg) c.dbg[2] = (long long)wall_clock64();
-#endif
+  if (ctrl) {
+    c.wrote_through = true;
+    return;
+  }
   const bool has_res = st.flags & MK_F_RES;
   const uint16_t *res = (const uint16_t *)st.res;
   float ures[U];
@@ -586,13 +602,14 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
 #pragma unroll
         for (int h = 0; h < NROW; h++) a[h] = wave_sum(a[h]);
         const float v = SILU ? silu_mul(a[0], a[NROW - 1]) : a[0] + r;
-        if (lane == 0) out[o] = (uint16_t)f2bf(v);
+        if (lane == 0) stc_u16(out + o, (uint16_t)f2bf(v));
       }
     }
     if (!any) break;
   }
+  c.wrote_through = true;
 #if MK_DEBUG_LIN
-  if (tid == 64 && c.dbg) c.dbg[3] = (long long)wall_clock64();
+  if (lane == 0 && c.dbg) c.dbg[wave] = (long long)wall_clock64();
 #endif
 }
 
@@ -1673,6 +1690,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.sh_tok = &sh_tok[0][0];
   c.sh_ticket = sh_ticket;
   c.seq = 0;
+  c.wrote_through = false;
   if (threadIdx.x == 0) sh_ticket[0] = sh_ticket[1] = 0;
   // ---- XCD discovery: rank of this workgroup inside its die, dies in use, workgroups per die
   if (threadIdx.x == 0) {
