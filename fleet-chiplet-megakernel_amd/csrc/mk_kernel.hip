@@ -1292,7 +1292,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   AttnUnit a0;
   const bool have0 = c.vid < n_units && decode(c.vid, a0);
   u32x4 pk[NPRE], pv[NPRE];
-  if (have0) {
+  auto prefetch0 = [&]() {
 #pragma unroll
     for (int i = 0; i < NPRE; i++) {
       const int pos = a0.start + gg + 16 * i;
@@ -1302,8 +1302,12 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         pv[i] = vc[off];
       }
     }
-  }
+  };
+  // the polling wavefront keeps its memory queue empty until the barrier is through (its loads would delay the poll
+  // results behind them); its rows are requested right after and land while the q rows are being fetched
+  if (have0 && wave != 0) prefetch0();
   barrier_wait(c);
+  if (have0 && wave == 0) prefetch0();
 
   for (int u = c.vid; u < n_units; u += c.G) {
     AttnUnit a;
@@ -1496,7 +1500,8 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
       if (C == 1) {
 #pragma unroll
-        for (int d = 0; d < DPT; d++) orow[mh * D + md + d] = (uint16_t)f2bf(os[d] / ls);
+        for (int d = 0; d < DPT; d += 2)  // written through: the stage's barrier skips the L2 write-back
+          __hip_atomic_store((uint32_t *)(orow + mh * D + md + d), pack2(os[d] / ls, os[d + 1] / ls), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
 #pragma unroll
         for (int d = 0; d < DPT; d++) gpart[mh * (D + 2) + md + d] = os[d];
@@ -1532,45 +1537,51 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
       __syncthreads();
       if (*sflag) {
-        // every chunk partial is read with independent device-scope loads, sixteen chunks in flight per thread
+        // every chunk partial is read with independent loads (8 bytes each), sixteen chunks in flight per thread
         const float *ip = (const float *)st.aux0 + (size_t)item * cmax * QPK * (D + 2);
         float mx = -INFINITY, ls = 0.f, os[DPT];
 #pragma unroll
         for (int d = 0; d < DPT; d++) os[d] = 0.f;
-        for (int c0 = 0; c0 < C; c0 += 16) {
-          float mv[16], lv[16], ov[16][DPT];
+        auto merge16 = [&](int c0, auto load8) {
+          float2 ml[16], ov[16][DPT / 2];
 #pragma unroll
           for (int j = 0; j < 16; j++) {
-            const int cc = min(c0 + j, C - 1);
-            const float *pp = ip + ((size_t)cc * QPK + mh) * (D + 2);
-            if (local) {
-              mv[j] = pp[D];
-              lv[j] = pp[D + 1];
+            if (c0 + j < C) {
+              const float *pp = ip + ((size_t)(c0 + j) * QPK + mh) * (D + 2);
+              ml[j] = load8(pp + D);
 #pragma unroll
-              for (int d = 0; d < DPT; d++) ov[j][d] = pp[md + d];
-            } else {
-              mv[j] = ldc_f32(pp + D);
-              lv[j] = ldc_f32(pp + D + 1);
-#pragma unroll
-              for (int d = 0; d < DPT; d++) ov[j][d] = ldc_f32(pp + md + d);
+              for (int d = 0; d < DPT / 2; d++) ov[j][d] = load8(pp + md + 2 * d);
             }
           }
 #pragma unroll
           for (int j = 0; j < 16; j++)
             if (c0 + j < C) {
-              const float mn = fmaxf(mx, mv[j]);
-              const float sa = __builtin_amdgcn_exp2f(mx - mn), sb = __builtin_amdgcn_exp2f(mv[j] - mn);
-              ls = ls * sa + lv[j] * sb;
+              const float mn = fmaxf(mx, ml[j].x);
+              const float sa = __builtin_amdgcn_exp2f(mx - mn), sb = __builtin_amdgcn_exp2f(ml[j].x - mn);
+              ls = ls * sa + ml[j].y * sb;
 #pragma unroll
-              for (int d = 0; d < DPT; d++) os[d] = os[d] * sa + ov[j][d] * sb;
+              for (int d = 0; d < DPT / 2; d++) {
+                os[2 * d] = os[2 * d] * sa + ov[j][d].x * sb;
+                os[2 * d + 1] = os[2 * d + 1] * sa + ov[j][d].y * sb;
+              }
               mx = mn;
             }
+        };
+        if (local) {
+          for (int c0 = 0; c0 < C; c0 += 16) merge16(c0, [](const float *q) { return *(const float2 *)q; });
+        } else {
+          for (int c0 = 0; c0 < C; c0 += 16)
+            merge16(c0, [](const float *q) {
+              const unsigned long long u = ldc_u64(q);
+              return make_float2(__uint_as_float((uint32_t)u), __uint_as_float((uint32_t)(u >> 32)));
+            });
         }
 #if MK_DEBUG_ATTN
         if (dbg && tid == 0) dbg[2] = (long long)wall_clock64();
 #endif
 #pragma unroll
-        for (int d = 0; d < DPT; d++) orow[mh * D + md + d] = (uint16_t)f2bf(os[d] / ls);
+        for (int d = 0; d < DPT; d += 2)  // written through: the stage's barrier skips the L2 write-back
+          __hip_atomic_store((uint32_t *)(orow + mh * D + md + d), pack2(os[d] / ls, os[d + 1] / ls), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #if MK_DEBUG_ATTN
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         if (dbg && tid == 0) dbg[3] = (long long)wall_clock64();
@@ -1578,6 +1589,10 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
     }
   }
+  // The attention outputs went through to memory.  The appended K/V rows and the published q rows stay in this die's
+  // L2 until a later barrier of this iteration writes it back (the sampling stages and the scheduler step always do);
+  // nothing reads them before the next iteration.
+  c.wrote_through = true;
 }
 
 // Greedy sampling, stage 1: every workgroup scans a contiguous slice of each token's logits and keeps
