@@ -1195,7 +1195,7 @@ int mk_compile(mk_graph *g) {
     if (s.op == MK_OP_ATTN) {
       const size_t units = (size_t)std::max(g->G, rt.max_tokens * s.num_kv_heads) + MK_ATTN_MAX_CHUNKS;
       const int qpk = s.num_q_heads / s.num_kv_heads;
-      if ((rc = dev_alloc(g, &p, units * qpk * (128 + 2) * sizeof(float), false))) return rc;
+      if ((rc = dev_alloc(g, &p, units * qpk * MK_ATTN_PSTRIDE * sizeof(float), false))) return rc;
       s.aux0 = p;
       s.aux1 = rt.attn_cnt + g->attn_cnt_n / 2;
     }

@@ -50,6 +50,9 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_R8
 #define MK_TUNE_R8 4
 #endif
+#ifndef MK_TUNE_R8N
+#define MK_TUNE_R8N 4
+#endif
 #ifndef MK_TUNE_R24
 #define MK_TUNE_R24 2
 #endif
@@ -662,7 +665,7 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
   const bool silu = st.flags & MK_F_SILU;
   if (st.k == 4096) {
     if (silu) stage_linear_m1_t<8, MK_TUNE_R8, true>(st, c, smem);
-    else stage_linear_m1_t<8, MK_TUNE_R8, false>(st, c, smem);
+    else stage_linear_m1_t<8, MK_TUNE_R8N, false>(st, c, smem);
   } else if (st.k == 12288 && !silu) {
     stage_linear_m1_t<24, MK_TUNE_R24, false>(st, c, smem);
   } else if (st.k == 2048) {
@@ -1480,7 +1483,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     // invalidated once per iteration, so a partial is never read from a stale line).  Otherwise device scope.
     const int item = u / cmax;
     const bool local = MK_TUNE_LOCALMERGE && c.even_xcds && (item * cmax) / c.quota == (item * cmax + C - 1) / c.quota;
-    float *gpart = (float *)st.aux0 + (size_t)u * QPK * (D + 2);
+    float *gpart = (float *)st.aux0 + (size_t)u * QPK * MK_ATTN_PSTRIDE;
     uint16_t *orow = (uint16_t *)st.out + (size_t)t * st.ld_out + (size_t)h * QPK * D;
     const int mh = tid / TPH, md = (tid - mh * TPH) * DPT;  // this thread merges dims [md, md+DPT) of head mh
     {
@@ -1503,12 +1506,11 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         for (int d = 0; d < DPT; d += 2)  // written through: the stage's barrier skips the L2 write-back
           __hip_atomic_store((uint32_t *)(orow + mh * D + md + d), pack2(os[d] / ls, os[d + 1] / ls), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       } else {
+        // 8-byte stores that together cover whole 128-byte lines (the running max and sum fill a line of their own, 16
+        // copies), so that the merging workgroup never reads a line that is only partly valid in the L2
 #pragma unroll
-        for (int d = 0; d < DPT; d++) gpart[mh * (D + 2) + md + d] = os[d];
-        if (md == 0) {
-          gpart[mh * (D + 2) + D] = mx;
-          gpart[mh * (D + 2) + D + 1] = ls;
-        }
+        for (int d = 0; d < DPT; d += 2) *(float2 *)(gpart + mh * MK_ATTN_PSTRIDE + md + d) = make_float2(os[d], os[d + 1]);
+        if (md < 16 * DPT) *(float2 *)(gpart + mh * MK_ATTN_PSTRIDE + D + 2 * (md / DPT)) = make_float2(mx, ls);
       }
     }
     if (C > 1) {
@@ -1538,7 +1540,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       __syncthreads();
       if (*sflag) {
         // every chunk partial is read with independent loads (8 bytes each), sixteen chunks in flight per thread
-        const float *ip = (const float *)st.aux0 + (size_t)item * cmax * QPK * (D + 2);
+        const float *ip = (const float *)st.aux0 + (size_t)item * cmax * QPK * MK_ATTN_PSTRIDE;
         float mx = -INFINITY, ls = 0.f, os[DPT];
 #pragma unroll
         for (int d = 0; d < DPT; d++) os[d] = 0.f;
@@ -1547,7 +1549,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
 #pragma unroll
           for (int j = 0; j < 16; j++) {
             if (c0 + j < C) {
-              const float *pp = ip + ((size_t)(c0 + j) * QPK + mh) * (D + 2);
+              const float *pp = ip + ((size_t)(c0 + j) * QPK + mh) * MK_ATTN_PSTRIDE;
               ml[j] = load8(pp + D);
 #pragma unroll
               for (int d = 0; d < DPT / 2; d++) ov[j][d] = load8(pp + md + 2 * d);

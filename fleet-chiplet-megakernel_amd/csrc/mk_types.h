@@ -16,6 +16,7 @@
 #define MK_MAX_SEGS 3         // a shuffled weight has at most 3 sources (q,k,v)
 #define MK_MAX_TOKENS 64      // max tokens per iteration supported by the kernels
 #define MK_ATTN_MAX_CHUNKS 32 // split-KV fan-out limit per (token, kv head)
+#define MK_ATTN_PSTRIDE 160   // floats per (work unit, q head) split-KV partial: 128 values + one 128-byte line of (max, sum)
 #define MK_MAX_NEW_PER_REQ 8  // prefill tokens per request per iteration (reference: MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
 // LDS map of one workgroup (dynamic, > 80 KB pins one workgroup per CU):
 //   [0, 24 KB)      input row(s) of the running stage / attention scratch (attention may run on into the ring)
