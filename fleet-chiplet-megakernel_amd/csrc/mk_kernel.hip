@@ -74,7 +74,8 @@ struct Ctx {
   MkSync *sync;
   const int *sh_tok;  // LDS copy of this iteration's token metadata: [0] position, [1] batch slot, [2] first token of the request, [3] first page-table entry
   bool even_xcds;     // every die in use runs the same number of workgroups, so die index = vid / quota
-  int *sh_ticket;     // two LDS work counters, used alternately by consecutive executed stages
+  int *sh_ticket;     // two LDS work counters, used alternately by consecutive executed stages; [2] = seq of the single-token
+                      // MoE stage that last filled the workgroup's expert list (kept outside the stages' scratch LDS)
   int seq;            // stages executed so far by this workgroup
   bool wrote_through; // the stage that just ran wrote all its outputs with write-through stores: no L2 write-back at its barrier
 #if MK_DEBUG_LIN
@@ -1165,8 +1166,194 @@ __device__ __forceinline__ void stage_moe_linear_t(CStage &st, Ctx &c, int M, ch
   }
 }
 
+// Single-token per-expert linear, tuned like the dense single-token linear: wavefront 0 polls the barrier, routes
+// (or reads the routing of the stage before), stages the input row(s) and publishes the routing outputs; wavefronts
+// 1..3 draw work from the workgroup's LDS ticket counter with R tickets of weight rows in flight each.  A ticket is
+// one [gate ; up] row pair of one slot's expert (SILU) or, for the W2 + weighted-sum form, output row j of ALL TK
+// slots' experts, so the combine stays inside one wavefront.  When the stage directly before was the W13 stage of the
+// same token its expert list is still in LDS: the first tickets' rows are then requested before the barrier.  All
+// outputs are written through.
+template <int KL, int R, bool SILU>
+__device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *smem) {
+  constexpr int TK = 8;
+  constexpr int NSUB = SILU ? 2 : TK;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  MoeLds *L = (MoeLds *)(smem + MK_PF_OFFSET);
+  const int k8 = st.k / 8, topk = st.topk, E = st.num_experts;
+  const bool ctrl = wave == 0;
+  const bool inline_topk = st.flags & MK_F_MOE_INLINE_TOPK;
+  const int NR = SILU ? st.n / 2 : st.n;
+  const int n_tk = SILU ? topk * NR : NR;
+  const int tq = n_tk / c.G, trem = n_tk - tq * c.G;
+  const int t_begin = c.vid * tq + min(c.vid, trem), t_end = t_begin + tq + (c.vid < trem ? 1 : 0);
+  int *ticket = c.sh_ticket + (c.seq & 1);
+  const bool reuse = !inline_topk && __builtin_amdgcn_readfirstlane(c.sh_ticket[2]) == c.seq - 1;
+  const u32x4 *W = (const u32x4 *)st.w.seg[0];
+  u32x4 *xs4 = (u32x4 *)smem;
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  auto take = [&]() -> int {
+    int t = 0;
+    if (lane == 0) t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    t = __builtin_amdgcn_readfirstlane(t) + t_begin;
+    return t < t_end ? t : -1;
+  };
+  auto load_ticket = [&](int tk, u32x4 (&b)[NSUB][KL]) {
+    int a = 0, j = tk;
+    if (SILU) {
+      a = tk / NR;
+      j = tk - a * NR;
+    }
+#pragma unroll
+    for (int h = 0; h < NSUB; h++) {
+      const int ei = __builtin_amdgcn_readfirstlane(L->act_e[SILU ? a : h]);
+      const u32x4 *p = W + ((size_t)max(ei, 0) * st.n + (size_t)(j + (SILU ? h * NR : 0))) * k8;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) b[h][kc] = (ei >= 0 && kc * 64 + lane < k8) ? ldg_stream(p + kc * 64 + lane) : zero;
+    }
+  };
+  u32x4 buf[R][NSUB][KL];
+  int ut[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) ut[j] = -1;
+  if (!ctrl) {
+    if (reuse) {
+#pragma unroll
+      for (int j = 0; j < R; j++) {
+        ut[j] = take();
+        if (ut[j] >= 0) load_ticket(ut[j], buf[j]);
+      }
+    }
+  } else {
+    if (c.pending && tid == 0) barrier_poll(c);
+    // input row(s): one row, or one row per slot (at most 12 16-byte segments per lane)
+    const int nx = (st.ld_in_slot ? topk : 1) * k8;
+    u32x4 xv[12];
+#pragma unroll
+    for (int i = 0; i < 12; i++) {
+      const int ci = i * 64 + lane;
+      if (ci < nx) {
+        const int sl = ci / k8, o = ci - sl * k8;
+        xv[i] = ldc_16B((const u32x4 *)((const uint16_t *)st.in + (size_t)sl * st.ld_in_slot) + o);
+      }
+    }
+    if (inline_topk) {
+      int sel[4];
+      float w;
+      int e;
+      moe_route_wave((const uint16_t *)st.moe_logits, E, topk, lane, sel, w, e);
+      if (lane < topk) {
+        L->act_e[lane] = e;
+        L->w[lane] = w;
+        if (c.vid == 0) __hip_atomic_store(st.moe_topk_w + lane, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+      if (c.vid == 0) {
+#pragma unroll
+        for (int j = 0; j < 4; j++)
+          if (j * 64 + lane < E) __hip_atomic_store(st.moe_routing + (size_t)(j * 64 + lane) * st.ld_routing, sel[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      }
+    } else if (!reuse) {
+      if (lane < topk) L->act_e[lane] = -1;
+#pragma unroll
+      for (int j = 0; j < 4; j++)
+        if (j * 64 + lane < E) {
+          const int r = ldc_i32(st.moe_routing + (size_t)(j * 64 + lane) * st.ld_routing);
+          if (r > 0 && r <= topk) L->act_e[r - 1] = j * 64 + lane;
+        }
+      if (!SILU && lane < topk) L->w[lane] = ldc_f32(st.moe_topk_w + lane);
+    }
+#pragma unroll
+    for (int i = 0; i < 12; i++)
+      if (i * 64 + lane < nx) xs4[i * 64 + lane] = xv[i];
+    if (lane == 0) c.sh_ticket[2] = c.seq;
+  }
+  __syncthreads();
+  barrier_done(c);
+  if (ctrl) {
+    if (c.vid == 0 && st.moe_mask) {  // active-expert list (its order is unspecified in the reference) and count
+      for (int i = lane; i < E; i += 64) __hip_atomic_store(st.moe_mask + i, i < topk ? L->act_e[i] : -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (lane == 0) __hip_atomic_store(st.moe_mask + E, topk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    }
+    c.wrote_through = true;
+    return;
+  }
+  float ures[R];
+#pragma unroll
+  for (int j = 0; j < R; j++) {
+    if (!reuse) {
+      ut[j] = take();
+      if (ut[j] >= 0) load_ticket(ut[j], buf[j]);
+    }
+    ures[j] = (!SILU && ut[j] >= 0) ? bf2f(ldc_u16((const uint16_t *)st.res + ut[j])) : 0.f;
+  }
+  uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
+  while (true) {
+    bool any = false;
+#pragma unroll
+    for (int j = 0; j < R; j++) {
+      if (ut[j] >= 0) {
+        any = true;
+        const int tk = ut[j];
+        int a = 0, row = tk;
+        if (SILU) {
+          a = tk / NR;
+          row = tk - a * NR;
+        }
+        float acc[NSUB];
+#pragma unroll
+        for (int h = 0; h < NSUB; h++) {
+          acc[h] = 0.f;
+          const u32x4 *x = xs4 + ((!SILU && st.ld_in_slot) ? h * k8 : 0);
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) {
+            const u32x4 xk = (kc * 64 + lane < k8) ? x[kc * 64 + lane] : zero;
+            acc[h] = dot8(buf[j][h][kc], xk, acc[h]);
+          }
+        }
+        const float r0 = ures[j];
+        ut[j] = take();
+        if (ut[j] >= 0) {
+          load_ticket(ut[j], buf[j]);
+          if (!SILU) ures[j] = bf2f(ldc_u16((const uint16_t *)st.res + ut[j]));
+        }
+#pragma unroll
+        for (int h = 0; h < NSUB; h++) acc[h] = wave_sum(acc[h]);
+        if (SILU) {
+          const uint32_t g = f2bf(acc[0]), up = f2bf(acc[1]);
+          if (lane == 0) {
+            uint16_t *y = out + (size_t)a * st.ld_out_slot;
+            stc_u16(y + row, (uint16_t)g);
+            stc_u16(y + row + NR, (uint16_t)up);
+            stc_u16(out2 + (size_t)a * st.ld_out2_slot + row, (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up))));
+          }
+        } else {
+          float comb = r0;
+#pragma unroll
+          for (int h = 0; h < NSUB; h++) {
+            const uint32_t v = f2bf(acc[h]);
+            if (lane == 0 && L->act_e[h] >= 0) stc_u16(out + (size_t)h * st.ld_out_slot + row, (uint16_t)v);
+            comb = fmaf(bf2f((uint16_t)v), L->w[h], comb);
+          }
+          if (lane == 0) stc_u16(out2 + row, (uint16_t)f2bf(comb));
+        }
+      }
+    }
+    if (!any) break;
+  }
+  c.wrote_through = true;
+}
+
 __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
+  if (M == 1) {
+    // tuned single-token forms: W13 + SwiGLU (one input row), W2 + weighted sum over exactly 8 slots
+    const int nx = (st.ld_in_slot ? st.topk : 1) * (st.k / 8);
+    if (silu && !st.ld_in_slot && nx <= 768) {
+      if (st.k <= 1024) return stage_moe_linear_m1<2, 4, true>(st, c, smem);
+      if (st.k <= 2048) return stage_moe_linear_m1<4, 3, true>(st, c, smem);
+    } else if (!silu && (st.flags & MK_F_MOE_COMBINE) && st.ld_in_slot && st.topk == 8 && nx <= 768) {
+      if (st.k <= 1024) return stage_moe_linear_m1<2, 2, false>(st, c, smem);
+    }
+  }
   if (st.k <= 1024) {
     if (silu) stage_moe_linear_t<2, 4, true>(st, c, M, smem);
     else stage_moe_linear_t<2, 6, false>(st, c, M, smem);
@@ -1692,7 +1879,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   __shared__ int sh_bcast[4];
   __shared__ int sh_quota[10];
   __shared__ int sh_tok[4][MK_MAX_TOKENS];
-  __shared__ int sh_ticket[2];
+  __shared__ int sh_ticket[3];
   // rt arrives by value in the kernel-argument segment (scalar loads); rtp is the same structure in device memory
   // for the one non-inlined function that takes its address (the scheduler step)
   Ctx c;
@@ -1708,7 +1895,10 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.sh_ticket = sh_ticket;
   c.seq = 0;
   c.wrote_through = false;
-  if (threadIdx.x == 0) sh_ticket[0] = sh_ticket[1] = 0;
+  if (threadIdx.x == 0) {
+    sh_ticket[0] = sh_ticket[1] = 0;
+    sh_ticket[2] = -2;
+  }
   // ---- XCD discovery: rank of this workgroup inside its die, dies in use, workgroups per die
   if (threadIdx.x == 0) {
     MkSync *s = rt.sync;
