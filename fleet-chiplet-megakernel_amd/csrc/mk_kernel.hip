@@ -567,8 +567,17 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   }
   __syncthreads();
   barrier_done(c);
-  if (ctrl) {
+  // Outputs are collected in LDS and written out together once every worker is done: one write-through request per
+  // 128-byte line instead of one 2-byte write per output.
+  uint16_t *so = (uint16_t *)(smem + MK_OUT_OFFSET);
+  auto flush = [&]() {
+    __syncthreads();
+    uint16_t *dst = (uint16_t *)st.out + o_begin;
+    for (int i = tid; i < o_end - o_begin; i += MK_THREADS) stc_u16(dst + i, so[i]);
     c.wrote_through = true;
+  };
+  if (ctrl) {
+    flush();
     return;
   }
   const bool has_res = st.flags & MK_F_RES;
@@ -582,7 +591,6 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
 #pragma unroll
     for (int kc = 0; kc < (KL <= 8 ? KL : 1); kc++) xr[kc] = xs4[kc * 64 + lane];
   }
-  uint16_t *out = (uint16_t *)st.out;
   while (true) {
     bool any = false;
 #pragma unroll
@@ -606,12 +614,12 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
 #pragma unroll
         for (int h = 0; h < NROW; h++) a[h] = wave_sum(a[h]);
         const float v = SILU ? silu_mul(a[0], a[NROW - 1]) : a[0] + r;
-        if (lane == 0) stc_u16(out + o, (uint16_t)f2bf(v));
+        if (lane == 0) so[o - o_begin] = (uint16_t)f2bf(v);
       }
     }
     if (!any) break;
   }
-  c.wrote_through = true;
+  flush();
 #if MK_DEBUG_LIN
   if (lane == 0 && c.dbg) c.dbg[wave] = (long long)wall_clock64();
 #endif
@@ -664,7 +672,11 @@ __device__ __forceinline__ void stage_linear_m1_generic(CStage &st, Ctx &c, char
 
 __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
-  if (st.k == 4096) {
+  // the tuned forms collect a workgroup's outputs in the LDS window [MK_OUT_OFFSET, MK_PF_OFFSET)
+  const bool fits = ((silu ? st.n / 2 : st.n) / c.G + 1) * 2 <= MK_PF_OFFSET - MK_OUT_OFFSET;
+  if (!fits) {
+    stage_linear_m1_generic(st, c, smem);
+  } else if (st.k == 4096) {
     if (silu) stage_linear_m1_t<8, MK_TUNE_R8, true>(st, c, smem);
     else stage_linear_m1_t<8, MK_TUNE_R8N, false>(st, c, smem);
   } else if (st.k == 12288 && !silu) {
@@ -1225,6 +1237,9 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
     }
   } else {
     if (c.pending && tid == 0) barrier_poll(c);
+#if MK_DEBUG_LIN
+    if (tid == 0 && c.dbg) c.dbg[0] = (long long)wall_clock64();
+#endif
     // input row(s): one row, or one row per slot (at most 12 16-byte segments per lane)
     const int nx = (st.ld_in_slot ? topk : 1) * k8;
     u32x4 xv[12];
@@ -1261,19 +1276,47 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
         }
       if (!SILU && lane < topk) L->w[lane] = ldc_f32(st.moe_topk_w + lane);
     }
+#if MK_DEBUG_LIN
+    if (tid == 0 && c.dbg) c.dbg[1] = (long long)wall_clock64();
+#endif
 #pragma unroll
     for (int i = 0; i < 12; i++)
       if (i * 64 + lane < nx) xs4[i * 64 + lane] = xv[i];
     if (lane == 0) c.sh_ticket[2] = c.seq;
+#if MK_DEBUG_LIN
+    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
+    if (tid == 0 && c.dbg) c.dbg[2] = (long long)wall_clock64();
+#endif
   }
   __syncthreads();
   barrier_done(c);
+  // outputs are collected in LDS ([array][ticket - t_begin]) and written out together once every worker is done
+  uint16_t *so = (uint16_t *)(smem + MK_OUT_OFFSET);
+  const int n_loc = t_end - t_begin;
+  constexpr int NARR = SILU ? 3 : TK + 1;
+  auto flush = [&]() {
+    __syncthreads();
+    uint16_t *o1 = (uint16_t *)st.out, *o2 = (uint16_t *)st.out2;
+    for (int i = tid; i < NARR * n_loc; i += MK_THREADS) {
+      const int arr = i / n_loc, tk = t_begin + (i - arr * n_loc);
+      uint16_t *dst;
+      if (SILU) {
+        const int a = tk / NR, row = tk - a * NR;
+        dst = arr == 2 ? o2 + (size_t)a * st.ld_out2_slot + row : o1 + (size_t)a * st.ld_out_slot + row + arr * NR;
+      } else {
+        if (arr < TK && L->act_e[arr] < 0) continue;
+        dst = arr == TK ? o2 + tk : o1 + (size_t)arr * st.ld_out_slot + tk;
+      }
+      stc_u16(dst, so[i]);
+    }
+    c.wrote_through = true;
+  };
   if (ctrl) {
     if (c.vid == 0 && st.moe_mask) {  // active-expert list (its order is unspecified in the reference) and count
       for (int i = lane; i < E; i += 64) __hip_atomic_store(st.moe_mask + i, i < topk ? L->act_e[i] : -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (lane == 0) __hip_atomic_store(st.moe_mask + E, topk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    c.wrote_through = true;
+    flush();
     return;
   }
   float ures[R];
@@ -1285,7 +1328,6 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
     }
     ures[j] = (!SILU && ut[j] >= 0) ? bf2f(ldc_u16((const uint16_t *)st.res + ut[j])) : 0.f;
   }
-  uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
   while (true) {
     bool any = false;
 #pragma unroll
@@ -1320,26 +1362,25 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
         if (SILU) {
           const uint32_t g = f2bf(acc[0]), up = f2bf(acc[1]);
           if (lane == 0) {
-            uint16_t *y = out + (size_t)a * st.ld_out_slot;
-            stc_u16(y + row, (uint16_t)g);
-            stc_u16(y + row + NR, (uint16_t)up);
-            stc_u16(out2 + (size_t)a * st.ld_out2_slot + row, (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up))));
+            so[tk - t_begin] = (uint16_t)g;
+            so[n_loc + tk - t_begin] = (uint16_t)up;
+            so[2 * n_loc + tk - t_begin] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
           }
         } else {
           float comb = r0;
 #pragma unroll
           for (int h = 0; h < NSUB; h++) {
             const uint32_t v = f2bf(acc[h]);
-            if (lane == 0 && L->act_e[h] >= 0) stc_u16(out + (size_t)h * st.ld_out_slot + row, (uint16_t)v);
+            if (lane == 0) so[h * n_loc + tk - t_begin] = (uint16_t)v;
             comb = fmaf(bf2f((uint16_t)v), L->w[h], comb);
           }
-          if (lane == 0) stc_u16(out2 + row, (uint16_t)f2bf(comb));
+          if (lane == 0) so[TK * n_loc + tk - t_begin] = (uint16_t)f2bf(comb);
         }
       }
     }
     if (!any) break;
   }
-  c.wrote_through = true;
+  flush();
 }
 
 __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char *smem) {
@@ -1347,7 +1388,10 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
   if (M == 1) {
     // tuned single-token forms: W13 + SwiGLU (one input row), W2 + weighted sum over exactly 8 slots
     const int nx = (st.ld_in_slot ? st.topk : 1) * (st.k / 8);
-    if (silu && !st.ld_in_slot && nx <= 768) {
+    const int n_loc = (silu ? st.topk * (st.n / 2) : st.n) / c.G + 1;
+    if ((silu ? 3 : 9) * n_loc * 2 > MK_PF_OFFSET - MK_OUT_OFFSET) {
+      // outputs of one workgroup do not fit the LDS collection window: generic form below
+    } else if (silu && !st.ld_in_slot && nx <= 768) {
       if (st.k <= 1024) return stage_moe_linear_m1<2, 4, true>(st, c, smem);
       if (st.k <= 2048) return stage_moe_linear_m1<4, 3, true>(st, c, smem);
     } else if (!silu && (st.flags & MK_F_MOE_COMBINE) && st.ld_in_slot && st.topk == 8 && nx <= 768) {

@@ -23,6 +23,7 @@
 //   [24 KB, 25 KB)  reduction scratch
 //   [32 KB, 128 KB) weight prefetch rings of the worker wavefronts, filled by direct-to-LDS loads across the grid barrier
 #define MK_RED_OFFSET (24 * 1024)
+#define MK_OUT_OFFSET (25 * 1024)   // [25 KB, 32 KB): outputs of a single-token linear collected before they are written out
 #define MK_PF_OFFSET (32 * 1024)
 #define MK_PF_BYTES (96 * 1024)
 #define MK_LDS_BYTES (128 * 1024)
