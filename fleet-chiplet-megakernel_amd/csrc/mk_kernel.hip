@@ -576,9 +576,12 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
     for (int i = tid; i < o_end - o_begin; i += MK_THREADS) stc_u16(dst + i, so[i]);
     c.wrote_through = true;
   };
-  if (ctrl) {
-    flush();
-    return;
+  if (ctrl) {  // the control wavefront has done its part: it now streams rows like the others
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      uo[j] = take();
+      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+    }
   }
   const bool has_res = st.flags & MK_F_RES;
   const uint16_t *res = (const uint16_t *)st.res;
@@ -924,14 +927,36 @@ __device__ __forceinline__ void moe_route_wave(const uint16_t *logits, int E, in
         bv = p[j];
         be = j * 64 + lane;
       }
+    // arg-max over the wavefront (lower expert id wins ties): rotations inside the 16-lane rows, then the four row
+    // winners through scalar lane reads
+#define MK_ARGMAX_STEP(CTRL)                                                                                          \
+  {                                                                                                                   \
+    const float ov = dpp_f32<CTRL>(bv);                                                                               \
+    const int oe = __builtin_amdgcn_update_dpp(0, be, CTRL, 0xF, 0xF, true);                                          \
+    if (ov > bv || (ov == bv && oe < be)) {                                                                           \
+      bv = ov;                                                                                                        \
+      be = oe;                                                                                                        \
+    }                                                                                                                 \
+  }
+    MK_ARGMAX_STEP(0x128)
+    MK_ARGMAX_STEP(0x124)
+    MK_ARGMAX_STEP(0x122)
+    MK_ARGMAX_STEP(0x121)
+#undef MK_ARGMAX_STEP
+    {
+      float rv = lane_f32(bv, 0);
+      int re = __builtin_amdgcn_readlane(be, 0);
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(bv, o, 64);
-      const int oe = __shfl_xor(be, o, 64);
-      if (ov > bv || (ov == bv && oe < be)) {
-        bv = ov;
-        be = oe;
+      for (int r = 16; r < 64; r += 16) {
+        const float ov = lane_f32(bv, r);
+        const int oe = __builtin_amdgcn_readlane(be, r);
+        if (ov > rv || (ov == rv && oe < re)) {
+          rv = ov;
+          re = oe;
+        }
       }
+      bv = rv;
+      be = re;
     }
     tot += bv;
     if (lane == s) {
@@ -1316,13 +1341,11 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
       for (int i = lane; i < E; i += 64) __hip_atomic_store(st.moe_mask + i, i < topk ? L->act_e[i] : -1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
       if (lane == 0) __hip_atomic_store(st.moe_mask + E, topk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
-    flush();
-    return;
   }
   float ures[R];
 #pragma unroll
   for (int j = 0; j < R; j++) {
-    if (!reuse) {
+    if (!reuse || ctrl) {  // the control wavefront joins the streaming once its part is done
       ut[j] = take();
       if (ut[j] >= 0) load_ticket(ut[j], buf[j]);
     }
