@@ -1234,18 +1234,36 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
     t = __builtin_amdgcn_readfirstlane(t) + t_begin;
     return t < t_end ? t : -1;
   };
-  auto load_ticket = [&](int tk, u32x4 (&b)[NSUB][KL]) {
-    int a = 0, j = tk;
-    if (SILU) {
-      a = tk / NR;
-      j = tk - a * NR;
+  // W2 form: the weight base of every slot's expert, fixed for the whole stage (set once the expert list is known)
+  const u32x4 *eb[SILU ? 1 : TK];
+  bool ev[SILU ? 1 : TK];
+  auto set_bases = [&]() {
+    if (!SILU) {
+#pragma unroll
+      for (int h = 0; h < (SILU ? 1 : TK); h++) {
+        const int ei = __builtin_amdgcn_readfirstlane(L->act_e[h]);
+        ev[h] = ei >= 0;
+        eb[h] = W + (size_t)max(ei, 0) * st.n * k8 + lane;
+      }
     }
+  };
+  auto load_ticket = [&](int tk, u32x4 (&b)[NSUB][KL]) {
+    if (SILU) {
+      const int a = tk / NR, j = tk - a * NR;
+      const int ei = __builtin_amdgcn_readfirstlane(L->act_e[a]);
 #pragma unroll
-    for (int h = 0; h < NSUB; h++) {
-      const int ei = __builtin_amdgcn_readfirstlane(L->act_e[SILU ? a : h]);
-      const u32x4 *p = W + ((size_t)max(ei, 0) * st.n + (size_t)(j + (SILU ? h * NR : 0))) * k8;
+      for (int h = 0; h < NSUB; h++) {
+        const u32x4 *p = W + ((size_t)max(ei, 0) * st.n + (size_t)(j + h * NR)) * k8;
 #pragma unroll
-      for (int kc = 0; kc < KL; kc++) b[h][kc] = (ei >= 0 && kc * 64 + lane < k8) ? ldg_stream(p + kc * 64 + lane) : zero;
+        for (int kc = 0; kc < KL; kc++) b[h][kc] = (ei >= 0 && kc * 64 + lane < k8) ? ldg_stream(p + kc * 64 + lane) : zero;
+      }
+    } else {
+#pragma unroll
+      for (int h = 0; h < NSUB; h++) {
+        const u32x4 *p = eb[SILU ? 0 : h] + (size_t)tk * k8;
+#pragma unroll
+        for (int kc = 0; kc < KL; kc++) b[h][kc] = (ev[SILU ? 0 : h] && kc * 64 + lane < k8) ? ldg_stream(p + kc * 64) : zero;
+      }
     }
   };
   u32x4 buf[R][NSUB][KL];
@@ -1254,6 +1272,7 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
   for (int j = 0; j < R; j++) ut[j] = -1;
   if (!ctrl) {
     if (reuse) {
+      set_bases();
 #pragma unroll
       for (int j = 0; j < R; j++) {
         ut[j] = take();
@@ -1342,6 +1361,15 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
       if (lane == 0) __hip_atomic_store(st.moe_mask + E, topk, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     }
   }
+  if (!reuse || ctrl) set_bases();
+  // W2 form: the staged input rows of all slots stay in registers for the whole stage
+  u32x4 xr[SILU ? 1 : TK][KL];
+  if (!SILU) {
+#pragma unroll
+    for (int h = 0; h < (SILU ? 1 : TK); h++)
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) xr[h][kc] = (kc * 64 + lane < k8) ? xs4[(st.ld_in_slot ? h * k8 : 0) + kc * 64 + lane] : zero;
+  }
   float ures[R];
 #pragma unroll
   for (int j = 0; j < R; j++) {
@@ -1367,10 +1395,11 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
 #pragma unroll
         for (int h = 0; h < NSUB; h++) {
           acc[h] = 0.f;
-          const u32x4 *x = xs4 + ((!SILU && st.ld_in_slot) ? h * k8 : 0);
 #pragma unroll
           for (int kc = 0; kc < KL; kc++) {
-            const u32x4 xk = (kc * 64 + lane < k8) ? x[kc * 64 + lane] : zero;
+            u32x4 xk;
+            if (SILU) xk = (kc * 64 + lane < k8) ? xs4[kc * 64 + lane] : zero;
+            else xk = xr[SILU ? 0 : h][kc];
             acc[h] = dot8(buf[j][h][kc], xk, acc[h]);
           }
         }
