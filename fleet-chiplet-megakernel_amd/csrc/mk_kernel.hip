@@ -1362,14 +1362,12 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
     }
   }
   if (!reuse || ctrl) set_bases();
-  // W2 form: the staged input rows of all slots stay in registers for the whole stage
+  // the staged input row(s) stay in registers for the whole stage
   u32x4 xr[SILU ? 1 : TK][KL];
-  if (!SILU) {
 #pragma unroll
-    for (int h = 0; h < (SILU ? 1 : TK); h++)
+  for (int h = 0; h < (SILU ? 1 : TK); h++)
 #pragma unroll
-      for (int kc = 0; kc < KL; kc++) xr[h][kc] = (kc * 64 + lane < k8) ? xs4[(st.ld_in_slot ? h * k8 : 0) + kc * 64 + lane] : zero;
-  }
+    for (int kc = 0; kc < KL; kc++) xr[h][kc] = (kc * 64 + lane < k8) ? xs4[(st.ld_in_slot ? h * k8 : 0) + kc * 64 + lane] : zero;
   float ures[R];
 #pragma unroll
   for (int j = 0; j < R; j++) {
@@ -1397,10 +1395,7 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
           acc[h] = 0.f;
 #pragma unroll
           for (int kc = 0; kc < KL; kc++) {
-            u32x4 xk;
-            if (SILU) xk = (kc * 64 + lane < k8) ? xs4[kc * 64 + lane] : zero;
-            else xk = xr[SILU ? 0 : h][kc];
-            acc[h] = dot8(buf[j][h][kc], xk, acc[h]);
+            acc[h] = dot8(buf[j][h][kc], xr[SILU ? 0 : h][kc], acc[h]);
           }
         }
         const float r0 = ures[j];
