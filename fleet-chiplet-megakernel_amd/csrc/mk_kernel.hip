@@ -891,6 +891,37 @@ __device__ __forceinline__ float wave_max(float v) {
   return fmaxf(fmaxf(lane_f32(v, 0), lane_f32(v, 16)), fmaxf(lane_f32(v, 32), lane_f32(v, 48)));
 }
 
+// Arg-max of (value, index) pairs over the wavefront; equal values go to the lower index.  Every lane returns the winner.
+__device__ __forceinline__ void wave_argmax(float &bv, int &be) {
+#define MK_ARGMAX_STEP(CTRL)                                                 \
+  {                                                                          \
+    const float ov = dpp_f32<CTRL>(bv);                                      \
+    const int oe = __builtin_amdgcn_update_dpp(0, be, CTRL, 0xF, 0xF, true); \
+    if (ov > bv || (ov == bv && oe < be)) {                                  \
+      bv = ov;                                                               \
+      be = oe;                                                               \
+    }                                                                        \
+  }
+  MK_ARGMAX_STEP(0x128)
+  MK_ARGMAX_STEP(0x124)
+  MK_ARGMAX_STEP(0x122)
+  MK_ARGMAX_STEP(0x121)
+#undef MK_ARGMAX_STEP
+  float rv = lane_f32(bv, 0);
+  int re = __builtin_amdgcn_readlane(be, 0);
+#pragma unroll
+  for (int r = 16; r < 64; r += 16) {
+    const float ov = lane_f32(bv, r);
+    const int oe = __builtin_amdgcn_readlane(be, r);
+    if (ov > rv || (ov == rv && oe < re)) {
+      rv = ov;
+      re = oe;
+    }
+  }
+  bv = rv;
+  be = re;
+}
+
 // Route one token with one wavefront: fp32 softmax over all experts, `topk` rounds of arg-max (equal probabilities
 // go to the lower expert id), weights renormalised by the sum of the selected probabilities.  Lane l owns experts
 // l, l+64, ...: sel[j] becomes 1 + slot for a selected expert l + 64 j, 0 otherwise; lane s < topk returns the weight
@@ -927,37 +958,7 @@ __device__ __forceinline__ void moe_route_wave(const uint16_t *logits, int E, in
         bv = p[j];
         be = j * 64 + lane;
       }
-    // arg-max over the wavefront (lower expert id wins ties): rotations inside the 16-lane rows, then the four row
-    // winners through scalar lane reads
-#define MK_ARGMAX_STEP(CTRL)                                                                                          \
-  {                                                                                                                   \
-    const float ov = dpp_f32<CTRL>(bv);                                                                               \
-    const int oe = __builtin_amdgcn_update_dpp(0, be, CTRL, 0xF, 0xF, true);                                          \
-    if (ov > bv || (ov == bv && oe < be)) {                                                                           \
-      bv = ov;                                                                                                        \
-      be = oe;                                                                                                        \
-    }                                                                                                                 \
-  }
-    MK_ARGMAX_STEP(0x128)
-    MK_ARGMAX_STEP(0x124)
-    MK_ARGMAX_STEP(0x122)
-    MK_ARGMAX_STEP(0x121)
-#undef MK_ARGMAX_STEP
-    {
-      float rv = lane_f32(bv, 0);
-      int re = __builtin_amdgcn_readlane(be, 0);
-#pragma unroll
-      for (int r = 16; r < 64; r += 16) {
-        const float ov = lane_f32(bv, r);
-        const int oe = __builtin_amdgcn_readlane(be, r);
-        if (ov > rv || (ov == rv && oe < re)) {
-          rv = ov;
-          re = oe;
-        }
-      }
-      bv = rv;
-      be = re;
-    }
+    wave_argmax(bv, be);
     tot += bv;
     if (lane == s) {
       w_slot = bv;
@@ -1726,16 +1727,29 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       if (pos < a.cend) process_block(pk, pv, pos);
       pos += 16 * NPRE;
     }
-    for (; pos < a.cend; pos += 16 * NPRE) {
-      u32x4 kk[NPRE], vv[NPRE];
+    // later blocks: the next block's rows are in flight while the current one is reduced
+    auto load_block = [&](int p0, u32x4 (&kk)[NPRE], u32x4 (&vv)[NPRE]) {
 #pragma unroll
       for (int i = 0; i < NPRE; i++)
-        if (pos + 16 * i < a.cend) {
-          const size_t off = kvoff(a, pos + 16 * i);
+        if (p0 + 16 * i < a.cend) {
+          const size_t off = kvoff(a, p0 + 16 * i);
           kk[i] = kc[off];
           vv[i] = vc[off];
         }
-      process_block(kk, vv, pos);
+    };
+    if (pos < a.cend) {
+      u32x4 ka[NPRE], va[NPRE], kb[NPRE], vb[NPRE];
+      load_block(pos, ka, va);
+      while (true) {
+        if (pos + 16 * NPRE < a.cend) load_block(pos + 16 * NPRE, kb, vb);
+        process_block(ka, va, pos);
+        pos += 16 * NPRE;
+        if (pos >= a.cend) break;
+        if (pos + 16 * NPRE < a.cend) load_block(pos + 16 * NPRE, ka, va);
+        process_block(kb, vb, pos);
+        pos += 16 * NPRE;
+        if (pos >= a.cend) break;
+      }
     }
     for (int j = gg; j < a.n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
     // ---- phase C: merge the 16 groups through LDS
@@ -1879,8 +1893,6 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
 // (max, lowest index attaining it).  Reference task: tasks/mi300/argmax_mi300.cuh:78-127.
 __device__ __forceinline__ void stage_argmax_partial(CStage &st, Ctx &c, int M, char *smem) {
   barrier_wait(c);
-  float *sv = (float *)smem;
-  int *si = (int *)(smem + 1024);
   const int n = st.n;
   int per = (n + c.G - 1) / c.G;
   per = (per + 1) & ~1;  // even, so slices start on a dword
@@ -1888,45 +1900,42 @@ __device__ __forceinline__ void stage_argmax_partial(CStage &st, Ctx &c, int M, 
   float *pv = (float *)st.aux0;
   int *pi = (int *)st.aux1;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
-  for (int t = 0; t < M; t++) {
-    const uint16_t *row = (const uint16_t *)st.in + (size_t)t * st.ld_in;
-    float best = -INFINITY;
-    int bi = 0x7fffffff;
-    for (int i = c0 + 2 * (int)threadIdx.x; i < c1; i += 2 * MK_THREADS) {
-      const uint32_t w = ldc_u32(row + i);
-      const float v0 = bf_lo(w), v1 = bf_hi(w);
-      if (v0 > best) {
-        best = v0;
-        bi = i;
-      }
-      if (i + 1 < c1 && v1 > best) {
-        best = v1;
-        bi = i + 1;
-      }
-    }
+  constexpr int NDW = 5, TB = 4;  // dwords per lane per token, tokens in flight per wavefront
+  const int nd = (c1 - c0 + 1) / 2;
+  // one wavefront per token, TB tokens' slices requested together; slices longer than NDW * 64 dwords loop
+  for (int t0 = wave * TB; t0 < M; t0 += MK_WAVES * TB) {
+    uint32_t w[TB][NDW];
 #pragma unroll
-    for (int o = 32; o > 0; o >>= 1) {
-      const float ov = __shfl_xor(best, o, 64);
-      const int oi = __shfl_xor(bi, o, 64);
-      if (ov > best || (ov == best && oi < bi)) {
-        best = ov;
-        bi = oi;
-      }
-    }
-    __syncthreads();
-    if (lane == 0) {
-      sv[wave] = best;
-      si[wave] = bi;
-    }
-    __syncthreads();
-    if (threadIdx.x == 0) {
-      for (int w = 1; w < MK_WAVES; w++)
-        if (sv[w] > best || (sv[w] == best && si[w] < bi)) {
-          best = sv[w];
-          bi = si[w];
+    for (int k = 0; k < TB; k++)
+#pragma unroll
+      for (int j = 0; j < NDW; j++)
+        if (t0 + k < M && j * 64 + lane < nd) w[k][j] = ldc_u32((const uint16_t *)st.in + (size_t)(t0 + k) * st.ld_in + c0 + 2 * (j * 64 + lane));
+#pragma unroll
+    for (int k = 0; k < TB; k++) {
+      if (t0 + k >= M) break;
+      const uint16_t *row = (const uint16_t *)st.in + (size_t)(t0 + k) * st.ld_in;
+      float best = -INFINITY;
+      int bi = 0x7fffffff;
+      auto consider = [&](uint32_t u, int i) {
+        const float v0 = bf_lo(u), v1 = bf_hi(u);
+        if (v0 > best) {
+          best = v0;
+          bi = i;
         }
-      pv[t * c.G + c.vid] = best;
-      pi[t * c.G + c.vid] = bi;
+        if (i + 1 < c1 && v1 > best) {
+          best = v1;
+          bi = i + 1;
+        }
+      };
+#pragma unroll
+      for (int j = 0; j < NDW; j++)
+        if (j * 64 + lane < nd) consider(w[k][j], c0 + 2 * (j * 64 + lane));
+      for (int d = NDW * 64 + lane; d < nd; d += 64) consider(ldc_u32(row + c0 + 2 * d), c0 + 2 * d);
+      wave_argmax(best, bi);
+      if (lane == 0) {
+        pv[(t0 + k) * c.G + c.vid] = best;
+        pi[(t0 + k) * c.G + c.vid] = bi;
+      }
     }
   }
 }
