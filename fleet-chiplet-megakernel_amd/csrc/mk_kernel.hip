@@ -25,28 +25,7 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 
 #define MK_SPIN_LIMIT (1u << 24)
 
-// prefetch depth of the single-token linear: LDS ring bytes per workgroup and register rows per worker wavefront
-#ifndef MK_TUNE_PF_BYTES
-#define MK_TUNE_PF_BYTES 0  // measured: the ring does not pay once the poll sits on the control wavefront
-#endif
-#ifndef MK_DEBUG_ATTN
-#define MK_DEBUG_ATTN 0
-#endif
-#ifndef MK_DEBUG_LIN
-#define MK_DEBUG_LIN 0
-#endif
-#ifndef MK_TUNE_WT
-#define MK_TUNE_WT 1
-#endif
-#ifndef MK_TUNE_EVEN
-#define MK_TUNE_EVEN 1
-#endif
-#ifndef MK_TUNE_LOCALMERGE
-#define MK_TUNE_LOCALMERGE 1
-#endif
-#ifndef MK_TUNE_XFENCE
-#define MK_TUNE_XFENCE 0
-#endif
+// weight rows in flight per wavefront of the single-token linear (K = 4096 with SwiGLU / K = 4096 plain / K = 12288)
 #ifndef MK_TUNE_R8
 #define MK_TUNE_R8 4
 #endif
@@ -78,9 +57,6 @@ struct Ctx {
                       // MoE stage that last filled the workgroup's expert list (kept outside the stages' scratch LDS)
   int seq;            // stages executed so far by this workgroup
   bool wrote_through; // the stage that just ran wrote all its outputs with write-through stores: no L2 write-back at its barrier
-#if MK_DEBUG_LIN
-  long long *dbg;     // four debug timestamps of the instrumented stage
-#endif
 };
 
 // ----------------------------------------------------------------------------- small helpers
@@ -188,10 +164,8 @@ __device__ __forceinline__ void barrier_arrive(Ctx &c) {
   __syncthreads();
   c.epoch++;
   if (threadIdx.x == 0) {
-#if MK_TUNE_WT
     if (c.wrote_through) __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
     else
-#endif
       __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT);
   }
   c.wrote_through = false;
@@ -457,16 +431,8 @@ __device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32
   const u32x4 *xin = (const u32x4 *)st.in;
   u32x4 *xs4 = (u32x4 *)xs;
   u32x4 v[KL];
-#if MK_TUNE_XFENCE
-  // every workgroup reads the same few KB: one cache invalidate, then ordinary loads that share the row through the
-  // die's L2, instead of 256 workgroups each pulling it from memory with device-scope loads
-  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-#pragma unroll
-  for (int kc = 0; kc < KL; kc++) v[kc] = xin[kc * 64 + lane];
-#else
 #pragma unroll
   for (int kc = 0; kc < KL; kc++) v[kc] = ldc_16B(xin + kc * 64 + lane);
-#endif
   if (st.flags & MK_F_NORM) {
     float ss = 0.f;
 #pragma unroll
@@ -501,12 +467,13 @@ __device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32
 // packed bf16 and the products run on v_dot2_f32_bf16 with fp32 accumulation.
 //
 // Wavefront roles: wavefront 0 is the control wavefront -- it polls the grid barrier, then loads, normalises and
-// publishes x -- while wavefronts 1..3 stream weight rows.  A wavefront's vector loads return in order, so a
-// wavefront that has weight loads in flight cannot observe the barrier before they land; keeping the poll on a
-// wavefront without weight loads lets the weight prefetch and the barrier overlap.
-// KL = K/512 row segments per lane; per worker wavefront the first NPF rows are prefetched straight into its LDS
-// ring and the next R rows into registers, all BEFORE the previous stage is known to be complete (weights do not
-// depend on it), so the HBM pipe stays busy across the grid barrier; each register slot is refilled once consumed.
+// publishes x, and only then joins the streaming -- while wavefronts 1..3 stream weight rows from the start.  A
+// wavefront's vector loads return in order, so a wavefront that has weight loads in flight cannot observe the
+// barrier before they land; keeping the poll on a wavefront without weight loads lets the weight prefetch and the
+// barrier overlap.
+// KL = K/512 row segments per lane.  Every worker keeps U outputs' rows in flight in registers; the first U are
+// requested BEFORE the previous stage is known to be complete (weights do not depend on it), so the HBM pipe stays
+// busy across the grid barrier, and a slot is refilled from the workgroup's ticket counter as soon as it is consumed.
 // Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:359-576).
 template <int KL, int R, bool SILU>
@@ -559,9 +526,6 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
       for (int kc = 0; kc < KL; kc++) nwv[kc] = ((const u32x4 *)st.norm_w)[kc * 64 + lane];
     }
     if (c.pending && tid == 0) barrier_poll(c);
-#if MK_DEBUG_LIN
-    if (tid == 0 && c.dbg) c.dbg[0] = (long long)wall_clock64();
-#endif
     stage_x_m1_wave<KL>(st, c, xs, lane, nwv);
 
   }
@@ -623,9 +587,6 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
     if (!any) break;
   }
   flush();
-#if MK_DEBUG_LIN
-  if (lane == 0 && c.dbg) c.dbg[wave] = (long long)wall_clock64();
-#endif
 }
 
 // Generic single-token linear for reduction lengths that are not a multiple of 512 or have no tuned
@@ -675,8 +636,8 @@ __device__ __forceinline__ void stage_linear_m1_generic(CStage &st, Ctx &c, char
 
 __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
-  // the tuned forms collect a workgroup's outputs in the LDS window [MK_OUT_OFFSET, MK_PF_OFFSET)
-  const bool fits = ((silu ? st.n / 2 : st.n) / c.G + 1) * 2 <= MK_PF_OFFSET - MK_OUT_OFFSET;
+  // the tuned forms collect a workgroup's outputs in the LDS window [MK_OUT_OFFSET, MK_MOE_OFFSET)
+  const bool fits = ((silu ? st.n / 2 : st.n) / c.G + 1) * 2 <= MK_MOE_OFFSET - MK_OUT_OFFSET;
   if (!fits) {
     stage_linear_m1_generic(st, c, smem);
   } else if (st.k == 4096) {
@@ -872,7 +833,7 @@ __device__ __forceinline__ void stage_silu_mul(CStage &st, Ctx &c, int M) {
 }
 
 // ----------------------------------------------------------------------------- mixture of experts
-// Routing lists of one workgroup, kept in the LDS region above MK_PF_OFFSET.
+// Routing lists of one workgroup, kept in the LDS region above MK_MOE_OFFSET.
 struct MoeLds {
   int r[MK_MOE_MAX_EXPERTS];          // single-token routing: 1 + slot per expert
   int act_e[MK_MOE_MAX_EXPERTS];      // expert id of each active expert
@@ -1068,7 +1029,7 @@ template <int KL, int R, bool SILU>
 __device__ __forceinline__ void stage_moe_linear_t(CStage &st, Ctx &c, int M, char *smem) {
   constexpr int NROW = SILU ? 2 : 1;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  MoeLds *L = (MoeLds *)(smem + MK_PF_OFFSET);
+  MoeLds *L = (MoeLds *)(smem + MK_MOE_OFFSET);
   const int k8 = st.k / 8;
   const bool combine = !SILU && (st.flags & MK_F_MOE_COMBINE) && M == 1;
   const bool inline_topk = (st.flags & MK_F_MOE_INLINE_TOPK) && M == 1;
@@ -1216,7 +1177,7 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
   constexpr int TK = 8;
   constexpr int NSUB = SILU ? 2 : TK;
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-  MoeLds *L = (MoeLds *)(smem + MK_PF_OFFSET);
+  MoeLds *L = (MoeLds *)(smem + MK_MOE_OFFSET);
   const int k8 = st.k / 8, topk = st.topk, E = st.num_experts;
   const bool ctrl = wave == 0;
   const bool inline_topk = st.flags & MK_F_MOE_INLINE_TOPK;
@@ -1282,9 +1243,6 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
     }
   } else {
     if (c.pending && tid == 0) barrier_poll(c);
-#if MK_DEBUG_LIN
-    if (tid == 0 && c.dbg) c.dbg[0] = (long long)wall_clock64();
-#endif
     // input row(s): one row, or one row per slot (at most 12 16-byte segments per lane)
     const int nx = (st.ld_in_slot ? topk : 1) * k8;
     u32x4 xv[12];
@@ -1321,17 +1279,10 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
         }
       if (!SILU && lane < topk) L->w[lane] = ldc_f32(st.moe_topk_w + lane);
     }
-#if MK_DEBUG_LIN
-    if (tid == 0 && c.dbg) c.dbg[1] = (long long)wall_clock64();
-#endif
 #pragma unroll
     for (int i = 0; i < 12; i++)
       if (i * 64 + lane < nx) xs4[i * 64 + lane] = xv[i];
     if (lane == 0) c.sh_ticket[2] = c.seq;
-#if MK_DEBUG_LIN
-    asm volatile("s_waitcnt lgkmcnt(0)" ::: "memory");
-    if (tid == 0 && c.dbg) c.dbg[2] = (long long)wall_clock64();
-#endif
   }
   __syncthreads();
   barrier_done(c);
@@ -1437,7 +1388,7 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
     // tuned single-token forms: W13 + SwiGLU (one input row), W2 + weighted sum over exactly 8 slots
     const int nx = (st.ld_in_slot ? st.topk : 1) * (st.k / 8);
     const int n_loc = (silu ? st.topk * (st.n / 2) : st.n) / c.G + 1;
-    if ((silu ? 3 : 9) * n_loc * 2 > MK_PF_OFFSET - MK_OUT_OFFSET) {
+    if ((silu ? 3 : 9) * n_loc * 2 > MK_MOE_OFFSET - MK_OUT_OFFSET) {
       // outputs of one workgroup do not fit the LDS collection window: generic form below
     } else if (silu && !st.ld_in_slot && nx <= 768) {
       if (st.k <= 1024) return stage_moe_linear_m1<2, 4, true>(st, c, smem);
@@ -1635,10 +1586,6 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
     }
     __syncthreads();
-#if MK_DEBUG_ATTN
-    long long *dbg2 = rt.stage_prof ? rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + 5) : nullptr;
-    if (dbg2 && tid == 0) dbg2[0] = (long long)wall_clock64();
-#endif
     // the chunk that owns the newest position appends this token's K/V and publishes q
     if (a.cidx == C - 1) {
       const int j = p - a.new_lo;
@@ -1753,9 +1700,6 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     }
     for (int j = gg; j < a.n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
     // ---- phase C: merge the 16 groups through LDS
-#if MK_DEBUG_ATTN
-    if (dbg2 && tid == 0) dbg2[1] = (long long)wall_clock64();
-#endif
 #pragma unroll
     for (int hh = 0; hh < QPK; hh++) {
       float *pp = part + (gg * QPK + hh) * 132;
@@ -1767,14 +1711,11 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
     }
     __syncthreads();
-#if MK_DEBUG_ATTN
-    if (dbg2 && tid == 0) dbg2[2] = (long long)wall_clock64();
-#endif
     // When every chunk of this (token, kv head) runs on one die, the partials and the arrival counter never leave that
     // die's L2: workgroup-scope atomic, ordinary stores and loads (each stage has its own partial buffer and the L1 is
     // invalidated once per iteration, so a partial is never read from a stale line).  Otherwise device scope.
     const int item = u / cmax;
-    const bool local = MK_TUNE_LOCALMERGE && c.even_xcds && (item * cmax) / c.quota == (item * cmax + C - 1) / c.quota;
+    const bool local = c.even_xcds && (item * cmax) / c.quota == (item * cmax + C - 1) / c.quota;
     float *gpart = (float *)st.aux0 + (size_t)u * QPK * MK_ATTN_PSTRIDE;
     uint16_t *orow = (uint16_t *)st.out + (size_t)t * st.ld_out + (size_t)h * QPK * D;
     const int mh = tid / TPH, md = (tid - mh * TPH) * DPT;  // this thread merges dims [md, md+DPT) of head mh
@@ -1807,10 +1748,6 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     }
     if (C > 1) {
       // ---- phase D: the last chunk to finish merges all chunks of this (token, kv head)
-#if MK_DEBUG_ATTN
-      long long *dbg = rt.stage_prof ? rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + 1) : nullptr;
-      if (dbg && tid == 0) dbg[0] = (long long)wall_clock64();
-#endif
       asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
       __syncthreads();
       if (tid == 0) {
@@ -1825,9 +1762,6 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
           if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
         *sflag = last;
-#if MK_DEBUG_ATTN
-        if (dbg) dbg[1] = (long long)wall_clock64();
-#endif
       }
       __syncthreads();
       if (*sflag) {
@@ -1870,16 +1804,9 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
               return make_float2(__uint_as_float((uint32_t)u), __uint_as_float((uint32_t)(u >> 32)));
             });
         }
-#if MK_DEBUG_ATTN
-        if (dbg && tid == 0) dbg[2] = (long long)wall_clock64();
-#endif
 #pragma unroll
         for (int d = 0; d < DPT; d += 2)  // written through: the stage's barrier skips the L2 write-back
           __hip_atomic_store((uint32_t *)(orow + mh * D + md + d), pack2(os[d] / ls, os[d + 1] / ls), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-#if MK_DEBUG_ATTN
-        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-        if (dbg && tid == 0) dbg[3] = (long long)wall_clock64();
-#endif
       }
     }
   }
@@ -2075,9 +2002,6 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       const int op = st.op, flags = st.flags;
       if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
       const long long t_in = (long long)wall_clock64();
-#if MK_DEBUG_LIN
-      c.dbg = (rt.stage_prof && s == MK_DEBUG_LIN) ? rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + 1) : nullptr;
-#endif
       switch (op) {
         case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;

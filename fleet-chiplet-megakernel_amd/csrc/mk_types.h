@@ -19,13 +19,13 @@
 #define MK_ATTN_PSTRIDE 160   // floats per (work unit, q head) split-KV partial: 128 values + one 128-byte line of (max, sum)
 #define MK_MAX_NEW_PER_REQ 8  // prefill tokens per request per iteration (reference: MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
 // LDS map of one workgroup (dynamic, > 80 KB pins one workgroup per CU):
-//   [0, 24 KB)      input row(s) of the running stage / attention scratch (attention may run on into the ring)
+//   [0, 24 KB)      input row(s) of the running stage / attention scratch (attention may run on beyond 32 KB)
 //   [24 KB, 25 KB)  reduction scratch
-//   [32 KB, 128 KB) weight prefetch rings of the worker wavefronts, filled by direct-to-LDS loads across the grid barrier
+//   [25 KB, 32 KB)  outputs of a single-token linear, collected before they are written out
+//   [32 KB, 128 KB) routing lists of the mixture-of-experts stages, matrix-core reduction scratch
 #define MK_RED_OFFSET (24 * 1024)
 #define MK_OUT_OFFSET (25 * 1024)   // [25 KB, 32 KB): outputs of a single-token linear collected before they are written out
-#define MK_PF_OFFSET (32 * 1024)
-#define MK_PF_BYTES (96 * 1024)
+#define MK_MOE_OFFSET (32 * 1024)
 #define MK_LDS_BYTES (128 * 1024)
 
 enum MkOp {
