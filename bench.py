@@ -3,7 +3,7 @@
 A "step" is one decode iteration of the persistent megakernel for the whole batch.  The prompt (80 seeded random ids
 per request) is ingested and W warm-up decode steps run untimed; then EXACTLY K decode steps run inside ONE persistent
 launch, bracketed by torch.cuda.synchronize() on both sides.  Weights, KV cache and meta tensors are resident in HBM
-before the timed region.  Prints one JSON line (see README of the driver contract).
+before the timed region.  Prints one JSON line.
 
 roofline: the dominant (only) kernel is mk_persistent_kernel; its algorithmic bytes per launch are
 K x (all bf16 weight matrices once + the K/V rows of every cached position of every request), divided by the launch
@@ -96,7 +96,7 @@ def main():
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the decode megakernel on ONE GPU; --gpus must be 1 "
-              "(multi-GPU tensor parallelism is described in DESIGN.md, not built)", file=sys.stderr)
+              "(multi-GPU tensor parallelism is not built)", file=sys.stderr)
         sys.exit(2)
     if int(os.environ.get("WORLD_SIZE", "1")) != 1:
         print("bench.py: launched with WORLD_SIZE>1; this benchmark is single-GPU", file=sys.stderr)

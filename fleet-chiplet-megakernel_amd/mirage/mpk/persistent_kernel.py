@@ -518,7 +518,7 @@ class PersistentKernel:
                    [(input_value, (1, 0, -1), -1), (input_index, (1, 0, -1), -1), (output, (0, 1, -1), -1)],
                    [getattr(self, "argmax_partial_output_size", 0)])
 
-    # layers of the reference that are outside the one-GPU dense decode path
+    # layers of the reference that are outside the one-GPU decode path
     def allreduce_layer(self, *args, **kwargs):
         raise NotImplementedError("allreduce_layer: the MI355X megakernel runs on one GPU")
 
