@@ -974,12 +974,18 @@ __device__ __forceinline__ void moe_build_lists(CStage &st, MoeLds *L, int M, bo
     __syncthreads();
     return;
   }
+  // the expert's row of the routing table, all requested at once (the multi-token callers have done their acquire,
+  // but the table is tiny: device-scope loads keep this correct for any caller)
+  int rv[MK_MAX_TOKENS];
   int cnt = 0;
-  if (tid < E)
-    for (int t = 0; t < M; t++) {
-      const int r = ldc_i32(st.moe_routing + (size_t)tid * st.ld_routing + t);
-      cnt += r > 0 && r <= st.topk;
-    }
+  if (tid < E) {
+#pragma unroll
+    for (int t = 0; t < MK_MAX_TOKENS; t++)
+      if (t < M) rv[t] = ldc_i32(st.moe_routing + (size_t)tid * st.ld_routing + t);
+#pragma unroll
+    for (int t = 0; t < MK_MAX_TOKENS; t++)
+      if (t < M) cnt += rv[t] > 0 && rv[t] <= st.topk;
+  }
   int sc = cnt, sa = cnt > 0;  // inclusive scans inside the wavefront
 #pragma unroll
   for (int o = 1; o < 64; o <<= 1) {
@@ -1004,10 +1010,12 @@ __device__ __forceinline__ void moe_build_lists(CStage &st, MoeLds *L, int M, bo
     L->act_e[ai] = tid;
     L->pair_off[ai] = off;
     int i = off;
-    for (int t = 0; t < M; t++) {
-      const int r = ldc_i32(st.moe_routing + (size_t)tid * st.ld_routing + t);
-      if (r > 0 && r <= st.topk && i < MK_MAX_TOKENS * MK_MOE_MAX_TOPK) L->pair_ts[i++] = t | ((r - 1) << 8);
-    }
+#pragma unroll
+    for (int t = 0; t < MK_MAX_TOKENS; t++)
+      if (t < M) {
+        const int r = rv[t];
+        if (r > 0 && r <= st.topk && i < MK_MAX_TOKENS * MK_MOE_MAX_TOPK) L->pair_ts[i++] = t | ((r - 1) << 8);
+      }
   }
   if (tid == MK_THREADS - 1) {
     L->n_act = ba + sa;
@@ -1382,6 +1390,131 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
   flush();
 }
 
+// Multi-token per-expert linear.  Work units (active expert, row) in expert-major order are split evenly over the
+// workgroups (a workgroup then touches one or two experts) and drawn from the LDS ticket counter by all four
+// wavefronts; the input rows of the tokens routed to the workgroup's experts are staged in LDS once, so the inner
+// loop over an expert's tokens reads them at LDS latency while R units' weight rows are in flight.
+template <int KL, int R, bool SILU>
+__device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M, char *smem) {
+  constexpr int NROW = SILU ? 2 : 1;
+  const int tid = threadIdx.x, lane = tid & 63;
+  MoeLds *L = (MoeLds *)(smem + MK_MOE_OFFSET);
+  const int k8 = st.k / 8;
+  barrier_wait(c);
+  if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // activation rows are read with cached loads below
+  __syncthreads();
+  moe_build_lists(st, L, M, false);
+  const int n_act = L->n_act;
+  if (c.vid == 0 && st.moe_mask) {  // publish the active-expert list (its order is unspecified in the reference)
+    for (int i = tid; i < st.num_experts; i += MK_THREADS) st.moe_mask[i] = i < n_act ? L->act_e[i] : -1;
+    if (tid == 0) st.moe_mask[st.num_experts] = n_act;
+  }
+  const int NR = SILU ? st.n / 2 : st.n;  // units per expert
+  const int n_units = n_act * NR;
+  // A unit of expert a costs one row load plus one reduction per token routed to a: split the units so that every
+  // workgroup gets the same cost.  With w_a = tokens(a) + 1 the cost before expert a is NR * (pair_off[a] + a).
+  int *bnd = L->wtot[0];  // reused: the scans are done
+  if (tid < 2) bnd[tid] = 0;
+  __syncthreads();
+  const long long total = (long long)NR * (L->pair_off[n_act] + n_act);
+  const long long tgt0 = total * c.vid / c.G, tgt1 = total * (c.vid + 1) / c.G;
+  if (tid < n_act) {
+    const long long before = (long long)NR * (L->pair_off[tid] + tid);
+    if (before <= tgt0) __hip_atomic_fetch_max(&bnd[0], tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    if (before <= tgt1) __hip_atomic_fetch_max(&bnd[1], tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+  }
+  __syncthreads();
+  auto unit_at = [&](long long tgt, int a) -> int {
+    if (n_act == 0) return 0;
+    const long long before = (long long)NR * (L->pair_off[a] + a);
+    const int w = L->pair_off[a + 1] - L->pair_off[a] + 1;
+    return a * NR + min(NR, (int)((tgt - before) / w));
+  };
+  const int u_begin = unit_at(tgt0, bnd[0]);
+  const int u_end = c.vid == c.G - 1 ? n_units : unit_at(tgt1, bnd[1]);
+  // stage the input rows of the (token, slot) pairs of this workgroup's experts
+  u32x4 *xs4 = (u32x4 *)(smem + MK_MOE_X_OFFSET);
+  int p_base = 0, n_staged = 0;
+  if (u_begin < u_end) {
+    p_base = L->pair_off[u_begin / NR];
+    n_staged = min(L->pair_off[(u_end - 1) / NR + 1] - p_base, (MK_LDS_BYTES - MK_MOE_X_OFFSET) / (k8 * 16));
+  }
+  for (int i = tid; i < n_staged * k8; i += MK_THREADS) {
+    const int p = i / k8, o = i - p * k8;
+    const int ts = L->pair_ts[p_base + p], tok = ts & 255, slot = ts >> 8;
+    xs4[i] = ((const u32x4 *)((const uint16_t *)st.in + (size_t)tok * st.ld_in + (size_t)slot * st.ld_in_slot))[o];
+  }
+  __syncthreads();
+  int *ticket = c.sh_ticket + (c.seq & 1);
+  auto take = [&]() -> int {
+    int t = 0;
+    if (lane == 0) t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    t = __builtin_amdgcn_readfirstlane(t) + u_begin;
+    return t < u_end ? t : -1;
+  };
+  const u32x4 *W = (const u32x4 *)st.w.seg[0];
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  auto load_unit = [&](int u, u32x4 (&b)[NROW][KL]) {
+    const int a = u / NR, j = u - a * NR;
+    const size_t e = (size_t)__builtin_amdgcn_readfirstlane(L->act_e[a]);
+#pragma unroll
+    for (int h = 0; h < NROW; h++) {
+      const u32x4 *p = W + (e * st.n + (size_t)(j + h * NR)) * k8;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) b[h][kc] = (kc * 64 + lane < k8) ? ldg_stream(p + kc * 64 + lane) : zero;
+    }
+  };
+  u32x4 buf[R][NROW][KL];
+  int ut[R];
+#pragma unroll
+  for (int jj = 0; jj < R; jj++) {
+    ut[jj] = take();
+    if (ut[jj] >= 0) load_unit(ut[jj], buf[jj]);
+  }
+  uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
+  while (true) {
+    bool any = false;
+#pragma unroll
+    for (int jj = 0; jj < R; jj++) {
+      if (ut[jj] >= 0) {
+        any = true;
+        const int u = ut[jj], a = u / NR, j = u - a * NR;
+        const int p0 = __builtin_amdgcn_readfirstlane(L->pair_off[a]), p1 = __builtin_amdgcn_readfirstlane(L->pair_off[a + 1]);
+        for (int p = p0; p < p1; p++) {
+          const int ts = __builtin_amdgcn_readfirstlane(L->pair_ts[p]), tok = ts & 255, slot = ts >> 8;
+          const u32x4 *x = (p - p_base < n_staged) ? xs4 + (size_t)(p - p_base) * k8
+                                                   : (const u32x4 *)((const uint16_t *)st.in + (size_t)tok * st.ld_in + (size_t)slot * st.ld_in_slot);
+          float acc[NROW];
+#pragma unroll
+          for (int h = 0; h < NROW; h++) acc[h] = 0.f;
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) {
+            const u32x4 xv = (kc * 64 + lane < k8) ? x[kc * 64 + lane] : zero;
+#pragma unroll
+            for (int h = 0; h < NROW; h++) acc[h] = dot8(buf[jj][h][kc], xv, acc[h]);
+          }
+#pragma unroll
+          for (int h = 0; h < NROW; h++) acc[h] = wave_sum(acc[h]);
+          uint16_t *y = out + (size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot;
+          if (SILU) {
+            const uint32_t g = f2bf(acc[0]), up = f2bf(acc[NROW - 1]);
+            if (lane == 0) {
+              y[j] = (uint16_t)g;
+              y[j + NR] = (uint16_t)up;
+              out2[(size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
+            }
+          } else if (lane == 0) {
+            y[j] = (uint16_t)f2bf(acc[0]);
+          }
+        }
+        ut[jj] = take();
+        if (ut[jj] >= 0) load_unit(ut[jj], buf[jj]);
+      }
+    }
+    if (!any) break;
+  }
+}
+
 __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
   if (M == 1) {
@@ -1396,6 +1529,19 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
     } else if (!silu && (st.flags & MK_F_MOE_COMBINE) && st.ld_in_slot && st.topk == 8 && nx <= 768) {
       if (st.k <= 1024) return stage_moe_linear_m1<2, 2, false>(st, c, smem);
     }
+  }
+  if (M > 1) {
+    if (st.k <= 1024) {
+      if (silu) stage_moe_linear_multi<2, 4, true>(st, c, M, smem);
+      else stage_moe_linear_multi<2, 6, false>(st, c, M, smem);
+    } else if (st.k <= 2048) {
+      if (silu) stage_moe_linear_multi<4, 3, true>(st, c, M, smem);
+      else stage_moe_linear_multi<4, 4, false>(st, c, M, smem);
+    } else {
+      if (silu) stage_moe_linear_multi<8, 1, true>(st, c, M, smem);
+      else stage_moe_linear_multi<8, 2, false>(st, c, M, smem);
+    }
+    return;
   }
   if (st.k <= 1024) {
     if (silu) stage_moe_linear_t<2, 4, true>(st, c, M, smem);

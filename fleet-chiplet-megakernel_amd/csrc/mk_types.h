@@ -26,6 +26,7 @@
 #define MK_RED_OFFSET (24 * 1024)
 #define MK_OUT_OFFSET (25 * 1024)   // [25 KB, 32 KB): outputs of a single-token linear collected before they are written out
 #define MK_MOE_OFFSET (32 * 1024)
+#define MK_MOE_X_OFFSET (40 * 1024)  // [40 KB, 128 KB): input rows of a multi-token MoE linear's (token, slot) pairs
 #define MK_LDS_BYTES (128 * 1024)
 
 enum MkOp {
