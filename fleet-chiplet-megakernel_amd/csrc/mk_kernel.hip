@@ -109,13 +109,16 @@ __device__ __forceinline__ u32x4 ldg_stream(const u32x4 *p) { return __builtin_n
 // not coherent with each other, and the CU's vector L1 is not coherent with anything: producers write back
 // their L2 at the barrier (release by the XCD's last arriver), consumers read with device-scope loads
 // (sc1: miss the L1, coherent in L2), so no cache invalidate is ever issued.
+// (the pointers are cast to the global address space explicitly: an atomic through a generic pointer becomes a flat
+// access, which is counted against the LDS queue as well and waits for it)
+#define MK_GLOBAL __attribute__((address_space(1)))
 __device__ __forceinline__ uint32_t ldc_u32(const void *p) {
-  return __hip_atomic_load((const uint32_t *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_load((const MK_GLOBAL uint32_t *)(unsigned long long)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ int ldc_i32(const int *p) { return (int)ldc_u32(p); }
 __device__ __forceinline__ float ldc_f32(const float *p) { return __uint_as_float(ldc_u32(p)); }
 __device__ __forceinline__ unsigned long long ldc_u64(const void *p) {
-  return __hip_atomic_load((const unsigned long long *)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  return __hip_atomic_load((const MK_GLOBAL unsigned long long *)(unsigned long long)p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
 __device__ __forceinline__ u32x4 ldc_16B(const u32x4 *p) {
   const unsigned long long a = ldc_u64(p), b = ldc_u64((const unsigned long long *)p + 1);
@@ -124,9 +127,11 @@ __device__ __forceinline__ u32x4 ldc_16B(const u32x4 *p) {
 }
 // Stores that are written through to memory (device scope), for outputs of stages that skip the L2 write-back at
 // their barrier.
-__device__ __forceinline__ void stc_u16(uint16_t *p, uint16_t v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); }
+__device__ __forceinline__ void stc_u16(uint16_t *p, uint16_t v) {
+  __hip_atomic_store((__attribute__((address_space(1))) uint16_t *)(unsigned long long)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ void stc_16B(u32x4 *p, u32x4 v) {
-  unsigned long long *q = (unsigned long long *)p;
+  __attribute__((address_space(1))) unsigned long long *q = (__attribute__((address_space(1))) unsigned long long *)(unsigned long long)p;
   __hip_atomic_store(q, (unsigned long long)v.x | ((unsigned long long)v.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __hip_atomic_store(q + 1, (unsigned long long)v.z | ((unsigned long long)v.w << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
@@ -1390,30 +1395,26 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
   flush();
 }
 
-// Multi-token per-expert linear.  Work units (active expert, row) in expert-major order are split evenly over the
-// workgroups (a workgroup then touches one or two experts) and drawn from the LDS ticket counter by all four
-// wavefronts; the input rows of the tokens routed to the workgroup's experts are staged in LDS once, so the inner
-// loop over an expert's tokens reads them at LDS latency while R units' weight rows are in flight.
+// Multi-token per-expert linear.  Work units (active expert, row) in expert-major order are split over the workgroups
+// by cost (a workgroup then touches one or two experts) and drawn from the LDS ticket counter by all four wavefronts.
+// The input rows of the tokens routed to the workgroup's experts are staged in LDS once and the outputs are collected
+// in an LDS tile, so the loop over an expert's tokens contains NO vector-memory instruction: the compiler can then
+// count the weight-row loads in flight exactly, and R units' rows really stay in flight (with a store inside that
+// loop every unit waited for all outstanding loads).  The tile is written out at the end, one contiguous run of
+// rows per (token, slot).  A workgroup whose tile or staged rows do not fit runs a plain loop over the same units.
 template <int KL, int R, bool SILU>
 __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M, char *smem) {
   constexpr int NROW = SILU ? 2 : 1;
+  constexpr int NARR = SILU ? 3 : 1;
   const int tid = threadIdx.x, lane = tid & 63;
   MoeLds *L = (MoeLds *)(smem + MK_MOE_OFFSET);
   const int k8 = st.k / 8;
-  barrier_wait(c);
-  if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // activation rows are read with cached loads below
-  __syncthreads();
-  moe_build_lists(st, L, M, false);
   const int n_act = L->n_act;
-  if (c.vid == 0 && st.moe_mask) {  // publish the active-expert list (its order is unspecified in the reference)
-    for (int i = tid; i < st.num_experts; i += MK_THREADS) st.moe_mask[i] = i < n_act ? L->act_e[i] : -1;
-    if (tid == 0) st.moe_mask[st.num_experts] = n_act;
-  }
   const int NR = SILU ? st.n / 2 : st.n;  // units per expert
   const int n_units = n_act * NR;
   // A unit of expert a costs one row load plus one reduction per token routed to a: split the units so that every
   // workgroup gets the same cost.  With w_a = tokens(a) + 1 the cost before expert a is NR * (pair_off[a] + a).
-  int *bnd = L->wtot[0];  // reused: the scans are done
+  int *bnd = L->wtot[0];  // reused: the scans of the list building are done
   if (tid < 2) bnd[tid] = 0;
   __syncthreads();
   const long long total = (long long)NR * (L->pair_off[n_act] + n_act);
@@ -1430,16 +1431,56 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
     const int w = L->pair_off[a + 1] - L->pair_off[a] + 1;
     return a * NR + min(NR, (int)((tgt - before) / w));
   };
-  const int u_begin = unit_at(tgt0, bnd[0]);
-  const int u_end = c.vid == c.G - 1 ? n_units : unit_at(tgt1, bnd[1]);
+  const int u_begin = __builtin_amdgcn_readfirstlane(unit_at(tgt0, bnd[0]));
+  const int u_end = __builtin_amdgcn_readfirstlane(c.vid == c.G - 1 ? n_units : unit_at(tgt1, bnd[1]));
+  const int nu = u_end - u_begin;
+  int p_base = 0, n_pairs = 0, maxp = 0;
+  if (nu > 0) {
+    const int a0 = u_begin / NR, a1 = (u_end - 1) / NR;
+    p_base = L->pair_off[a0];
+    n_pairs = L->pair_off[a1 + 1] - p_base;
+    for (int a = a0; a <= a1; a++) maxp = max(maxp, L->pair_off[a + 1] - L->pair_off[a]);
+  }
+  // the decision below is per workgroup (uniform within it); either form covers exactly [u_begin, u_end)
+  const u32x4 zero = {0u, 0u, 0u, 0u};
+  const u32x4 *W = (const u32x4 *)st.w.seg[0];
+  if ((size_t)n_pairs * k8 * 16 > (size_t)(MK_LDS_BYTES - MK_MOE_X_OFFSET) || (size_t)NARR * maxp * nu * 2 > (size_t)MK_MOE_OFFSET) {
+    // too many tokens on this workgroup's experts for the LDS windows: plain form over the same unit range
+    const int wv = __builtin_amdgcn_readfirstlane(tid >> 6);
+    uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
+    for (int u = u_begin + wv; u < u_end; u += MK_WAVES) {
+      const int a = u / NR, j = u - a * NR;
+      const size_t e = (size_t)L->act_e[a];
+      for (int p = L->pair_off[a]; p < L->pair_off[a + 1]; p++) {
+        const int ts = L->pair_ts[p], tok = ts & 255, slot = ts >> 8;
+        const u32x4 *x = (const u32x4 *)((const uint16_t *)st.in + (size_t)tok * st.ld_in + (size_t)slot * st.ld_in_slot);
+        float acc[NROW];
+#pragma unroll
+        for (int h = 0; h < NROW; h++) {
+          acc[h] = 0.f;
+          const u32x4 *wr = W + (e * st.n + (size_t)(j + h * NR)) * k8;
+          for (int kc = lane; kc < k8; kc += 64) acc[h] = dot8(wr[kc], x[kc], acc[h]);
+          acc[h] = wave_sum(acc[h]);
+        }
+        uint16_t *y = out + (size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot;
+        if (SILU) {
+          const uint32_t g = f2bf(acc[0]), up = f2bf(acc[NROW - 1]);
+          if (lane == 0) {
+            y[j] = (uint16_t)g;
+            y[j + NR] = (uint16_t)up;
+            out2[(size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
+          }
+        } else if (lane == 0) {
+          y[j] = (uint16_t)f2bf(acc[0]);
+        }
+      }
+    }
+    return;
+  }
   // stage the input rows of the (token, slot) pairs of this workgroup's experts
   u32x4 *xs4 = (u32x4 *)(smem + MK_MOE_X_OFFSET);
-  int p_base = 0, n_staged = 0;
-  if (u_begin < u_end) {
-    p_base = L->pair_off[u_begin / NR];
-    n_staged = min(L->pair_off[(u_end - 1) / NR + 1] - p_base, (MK_LDS_BYTES - MK_MOE_X_OFFSET) / (k8 * 16));
-  }
-  for (int i = tid; i < n_staged * k8; i += MK_THREADS) {
+  uint16_t *so = (uint16_t *)smem;  // [array][pair of the expert][unit - u_begin]
+  for (int i = tid; i < n_pairs * k8; i += MK_THREADS) {
     const int p = i / k8, o = i - p * k8;
     const int ts = L->pair_ts[p_base + p], tok = ts & 255, slot = ts >> 8;
     xs4[i] = ((const u32x4 *)((const uint16_t *)st.in + (size_t)tok * st.ld_in + (size_t)slot * st.ld_in_slot))[o];
@@ -1452,8 +1493,6 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
     t = __builtin_amdgcn_readfirstlane(t) + u_begin;
     return t < u_end ? t : -1;
   };
-  const u32x4 *W = (const u32x4 *)st.w.seg[0];
-  const u32x4 zero = {0u, 0u, 0u, 0u};
   auto load_unit = [&](int u, u32x4 (&b)[NROW][KL]) {
     const int a = u / NR, j = u - a * NR;
     const size_t e = (size_t)__builtin_amdgcn_readfirstlane(L->act_e[a]);
@@ -1471,19 +1510,16 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
     ut[jj] = take();
     if (ut[jj] >= 0) load_unit(ut[jj], buf[jj]);
   }
-  uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
   while (true) {
     bool any = false;
 #pragma unroll
     for (int jj = 0; jj < R; jj++) {
       if (ut[jj] >= 0) {
         any = true;
-        const int u = ut[jj], a = u / NR, j = u - a * NR;
+        const int u = ut[jj], a = u / NR;
         const int p0 = __builtin_amdgcn_readfirstlane(L->pair_off[a]), p1 = __builtin_amdgcn_readfirstlane(L->pair_off[a + 1]);
-        for (int p = p0; p < p1; p++) {
-          const int ts = __builtin_amdgcn_readfirstlane(L->pair_ts[p]), tok = ts & 255, slot = ts >> 8;
-          const u32x4 *x = (p - p_base < n_staged) ? xs4 + (size_t)(p - p_base) * k8
-                                                   : (const u32x4 *)((const uint16_t *)st.in + (size_t)tok * st.ld_in + (size_t)slot * st.ld_in_slot);
+        for (int p = p0; p < p1; p++) {  // LDS only in here
+          const u32x4 *x = xs4 + (p - p_base) * k8;
           float acc[NROW];
 #pragma unroll
           for (int h = 0; h < NROW; h++) acc[h] = 0.f;
@@ -1495,16 +1531,16 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
           }
 #pragma unroll
           for (int h = 0; h < NROW; h++) acc[h] = wave_sum(acc[h]);
-          uint16_t *y = out + (size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot;
+          uint16_t *t0 = so + (size_t)(p - p0) * nu + (u - u_begin);
           if (SILU) {
             const uint32_t g = f2bf(acc[0]), up = f2bf(acc[NROW - 1]);
             if (lane == 0) {
-              y[j] = (uint16_t)g;
-              y[j + NR] = (uint16_t)up;
-              out2[(size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
+              t0[0] = (uint16_t)g;
+              t0[(size_t)maxp * nu] = (uint16_t)up;
+              t0[(size_t)2 * maxp * nu] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
             }
           } else if (lane == 0) {
-            y[j] = (uint16_t)f2bf(acc[0]);
+            t0[0] = (uint16_t)f2bf(acc[0]);
           }
         }
         ut[jj] = take();
@@ -1512,6 +1548,18 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
       }
     }
     if (!any) break;
+  }
+  __syncthreads();
+  // write the tile out: consecutive threads take consecutive rows of one (token, slot)
+  uint16_t *out = (uint16_t *)st.out, *out2 = (uint16_t *)st.out2;
+  for (int i = tid; i < NARR * maxp * nu; i += MK_THREADS) {
+    const int arr = i / (maxp * nu), r = i - arr * maxp * nu, pi = r / nu, ui = r - pi * nu;
+    const int u = u_begin + ui, a = u / NR, j = u - a * NR;
+    const int p = L->pair_off[a] + pi;
+    if (p >= L->pair_off[a + 1]) continue;
+    const int ts = L->pair_ts[p], tok = ts & 255, slot = ts >> 8;
+    if (SILU && arr == 2) out2[(size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j] = so[i];
+    else out[(size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot + j + (arr == 1 ? NR : 0)] = so[i];
   }
 }
 
@@ -1531,6 +1579,17 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
     }
   }
   if (M > 1) {
+    // common front: wait for the previous stage, one acquire (activation rows are read with cached loads), routing lists
+    MoeLds *L = (MoeLds *)(smem + MK_MOE_OFFSET);
+    barrier_wait(c);
+    if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    __syncthreads();
+    moe_build_lists(st, L, M, false);
+    if (c.vid == 0 && st.moe_mask) {  // publish the active-expert list (its order is unspecified in the reference)
+      const int n_act = L->n_act;
+      for (int i = threadIdx.x; i < st.num_experts; i += MK_THREADS) st.moe_mask[i] = i < n_act ? L->act_e[i] : -1;
+      if (threadIdx.x == 0) st.moe_mask[st.num_experts] = n_act;
+    }
     if (st.k <= 1024) {
       if (silu) stage_moe_linear_multi<2, 4, true>(st, c, M, smem);
       else stage_moe_linear_multi<2, 6, false>(st, c, M, smem);
