@@ -24,6 +24,9 @@ typedef const __attribute__((address_space(4))) MkStage CStage;
 typedef const __attribute__((address_space(4))) MkWeight CWeight;
 
 #define MK_SPIN_LIMIT (1u << 24)
+#ifndef MK_TUNE_POLL_SLEEP
+#define MK_TUNE_POLL_SLEEP 1
+#endif
 
 // weight rows in flight per wavefront of the single-token linear (K = 4096 with SwiGLU / K = 4096 plain / K = 12288)
 #ifndef MK_TUNE_R8
@@ -184,15 +187,21 @@ __device__ __forceinline__ void barrier_poll(Ctx &c) {
   MkSync *s = c.sync;
   const unsigned epoch = c.epoch;
   unsigned spins = 0;
-  while (true) {
-    unsigned v[8];
+  unsigned va[8];
+  auto issue = [&](unsigned (&v)[8]) {
 #pragma unroll
     for (int x = 0; x < 8; x++) v[x] = __hip_atomic_load(&s->local_ctr[x][0], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  };
+  auto done = [&](const unsigned (&v)[8]) -> bool {
     bool ok = true;
 #pragma unroll
     for (int x = 0; x < 8; x++) ok = ok && (v[x] >= c.quotas[x] * epoch);
-    if (ok || !spin_ok(s, spins, epoch)) break;
-    __builtin_amdgcn_s_sleep(1);
+    return ok;
+  };
+  while (true) {
+    issue(va);
+    if (done(va) || !spin_ok(s, spins, epoch)) break;
+    __builtin_amdgcn_s_sleep(MK_TUNE_POLL_SLEEP);
   }
   *c.sh_dead = (spins >= 1024u) ? (int)__hip_atomic_load(&s->abort_flag, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) : 0;
 }
