@@ -677,16 +677,14 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
 // weight row) against a 32(k) x 16(m) activation fragment that comes from the L2-resident activation rows.
 // Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
-#ifndef MK_TUNE_TG
-#define MK_TUNE_TG 6
+#ifndef MK_TUNE_NBN
+#define MK_TUNE_NBN 4
 #endif
-#ifndef MK_TUNE_NB
-#define MK_TUNE_NB 2
-#endif
-template <int MT>
+// TG = weight tiles per K sweep, NB = 64-wide k steps in flight per wavefront.  Two shapes are instantiated: wide
+// stages (several tiles per workgroup) run <6, 2>; narrow ones (one or two weight tiles per workgroup, e.g. N = 4096
+// on 256 workgroups) spend the registers on depth instead: <2, MK_TUNE_NBN>.
+template <int MT, int TG, int NB>
 __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, char *smem) {
-  constexpr int TG = MK_TUNE_TG;  // weight tiles per K sweep
-  constexpr int NB = MK_TUNE_NB;  // 64-wide k steps in flight per wavefront
   barrier_wait(c);
   // activations were produced by other workgroups: invalidate this CU's L1 once, then use cached loads so the rows
   // are shared through the XCD's L2
@@ -2221,10 +2219,21 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
         case MK_OP_LINEAR:
           if (M == 1) stage_linear_m1(st, c, smem);
-          else if (M <= 16) stage_linear_mfma<1>(st, c, M, smem);
-          else if (M <= 32) stage_linear_mfma<2>(st, c, M, smem);
-          else if (M <= 48) stage_linear_mfma<3>(st, c, M, smem);
-          else stage_linear_mfma<4>(st, c, M, smem);
+          else {
+            const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
+            const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
+            if (narrow) {
+              if (M <= 16) stage_linear_mfma<1, 2, 2 * MK_TUNE_NBN>(st, c, M, smem);
+              else if (M <= 32) stage_linear_mfma<2, 2, MK_TUNE_NBN + MK_TUNE_NBN / 2>(st, c, M, smem);
+              else if (M <= 48) stage_linear_mfma<3, 2, MK_TUNE_NBN>(st, c, M, smem);
+              else stage_linear_mfma<4, 2, MK_TUNE_NBN>(st, c, M, smem);
+            } else {
+              if (M <= 16) stage_linear_mfma<1, 6, 2>(st, c, M, smem);
+              else if (M <= 32) stage_linear_mfma<2, 6, 2>(st, c, M, smem);
+              else if (M <= 48) stage_linear_mfma<3, 6, 2>(st, c, M, smem);
+              else stage_linear_mfma<4, 6, 2>(st, c, M, smem);
+            }
+          }
           break;
         case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
         case MK_OP_ATTN:
