@@ -677,6 +677,172 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
 // weight row) against a 32(k) x 16(m) activation fragment that comes from the L2-resident activation rows.
 // Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
+// Few-token linear (2..MB tokens): the single-token structure with the token rows in LDS.  Every weight row is still
+// read once and dotted against all token rows (v_dot2, fp32); up to 8 tokens this stays under the streaming time, so
+// small batches cost little more than one token, where the matrix-core path (16-row tiles, one tile per workgroup
+// on the narrow stages) is bound by latency.  The rows were normalised by the preceding NORM stage when the stage
+// carries MK_F_NORM.  Outputs are collected in LDS [token][output] and written through.
+template <int KL, int R, bool SILU, int MB>
+__device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, char *smem) {
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  constexpr int K8 = KL * 64;
+  constexpr int NROW = SILU ? 2 : 1;
+  constexpr int U = R / NROW;
+  const bool ctrl = wave == 0;
+  const int n_out = SILU ? st.n / 2 : st.n;
+  const int oq = n_out / c.G, orem = n_out - oq * c.G;
+  const int o_begin = c.vid * oq + min(c.vid, orem), o_end = o_begin + oq + (c.vid < orem ? 1 : 0);
+  const int n_loc = o_end - o_begin;
+  int *ticket = c.sh_ticket + (c.seq & 1);
+  const int half = st.silu_half;
+  auto take = [&]() -> int {
+    int t = 0;
+    if (lane == 0) t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    t = __builtin_amdgcn_readfirstlane(t) + o_begin;
+    return t < o_end ? t : -1;
+  };
+  auto load_unit = [&](int o, u32x4 (&b)[NROW][KL]) {
+    int vr = o;
+    if (SILU) {
+      const int g = o / half;
+      vr = g * 2 * half + (o - g * half);
+    }
+#pragma unroll
+    for (int h = 0; h < NROW; h++) {
+      const u32x4 *p = weight_row(st.w, vr + h * half, K8) + lane;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) b[h][kc] = ldg_stream(p + kc * 64);
+    }
+  };
+  u32x4 buf[U][NROW][KL];
+  int uo[U];
+#pragma unroll
+  for (int j = 0; j < U; j++) uo[j] = -1;
+  if (!ctrl) {
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      uo[j] = take();
+      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+    }
+  } else {
+    if (c.pending && tid == 0) barrier_poll(c);
+    // the token rows come from other workgroups: one acquire, then ordinary loads that share them through the die's L2
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  }
+  __syncthreads();
+  barrier_done(c);
+  // all four wavefronts stage the token rows (the workers' requests queue behind their weight rows, which were issued
+  // long before)
+  const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
+  const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
+  u32x4 *xs4 = (u32x4 *)(smem + MK_MOE_X_OFFSET);  // [token][K8]
+  {
+    constexpr int NCH = MB * KL / MK_WAVES;  // 16-byte segments per lane
+    u32x4 xv[NCH];
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int ci = (i * MK_WAVES + wave) * 64 + lane, m = ci / K8, o = ci - m * K8;
+      if (m < M) xv[i] = ((const u32x4 *)(x + (size_t)m * ldx))[o];
+    }
+#pragma unroll
+    for (int i = 0; i < NCH; i++) {
+      const int ci = (i * MK_WAVES + wave) * 64 + lane;
+      if (ci / K8 < M) xs4[ci] = xv[i];
+    }
+  }
+  __syncthreads();
+  if (ctrl) {
+#pragma unroll
+    for (int j = 0; j < U; j++) {
+      uo[j] = take();
+      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+    }
+  }
+  const bool has_res = st.flags & MK_F_RES;
+  const uint16_t *res = (const uint16_t *)st.res;
+  uint16_t *so = (uint16_t *)smem;  // [token][output - o_begin]
+  // Plain rows are reduced two slots at a time: a token-row segment read from LDS is used for both slots' weight rows
+  // (half the LDS reads per output), while the other pair of slots has its rows in flight.
+  constexpr int Q = SILU ? 1 : 2;  // slots per group ([gate ; up] pairs already share the segment)
+  static_assert(U % Q == 0, "slots are processed in groups");
+  while (true) {
+    bool any = false;
+#pragma unroll
+    for (int j = 0; j < U; j += Q) {
+      if (uo[j] >= 0 || uo[j + Q - 1] >= 0) {
+        any = true;
+        float a[Q][NROW][MB];
+#pragma unroll
+        for (int m = 0; m < MB; m++) {
+#pragma unroll
+          for (int q = 0; q < Q; q++)
+#pragma unroll
+            for (int h = 0; h < NROW; h++) a[q][h][m] = 0.f;
+          if (m < M) {
+#pragma unroll
+            for (int kc = 0; kc < KL; kc++) {
+              const u32x4 xk = xs4[m * K8 + kc * 64 + lane];
+#pragma unroll
+              for (int q = 0; q < Q; q++)
+#pragma unroll
+                for (int h = 0; h < NROW; h++) a[q][h][m] = dot8(buf[j + q][h][kc], xk, a[q][h][m]);
+            }
+          }
+        }
+        int o2[Q];
+#pragma unroll
+        for (int q = 0; q < Q; q++) {
+          o2[q] = uo[j + q];
+          uo[j + q] = take();
+          if (uo[j + q] >= 0) load_unit(uo[j + q], buf[j + q]);
+        }
+#pragma unroll
+        for (int q = 0; q < Q; q++)
+          if (o2[q] >= 0) {
+#pragma unroll
+            for (int m = 0; m < MB; m++)
+              if (m < M) {
+#pragma unroll
+                for (int h = 0; h < NROW; h++) a[q][h][m] = wave_sum(a[q][h][m]);
+                float v;
+                if (SILU) v = silu_mul(a[q][0][m], a[q][NROW - 1][m]);
+                else v = has_res ? a[q][0][m] + bf2f(res[(size_t)m * st.ld_res + o2[q]]) : a[q][0][m];
+                if (lane == 0) so[m * n_loc + (o2[q] - o_begin)] = (uint16_t)f2bf(v);
+              }
+          }
+      }
+    }
+    if (!any) break;
+  }
+  __syncthreads();
+  uint16_t *dst = (uint16_t *)st.out + o_begin;
+  for (int i = tid; i < M * n_loc; i += MK_THREADS) {
+    const int m = i / n_loc, r = i - m * n_loc;
+    stc_u16(dst + (size_t)m * st.ld_out + r, so[i]);
+  }
+  c.wrote_through = true;
+}
+
+// Whether the few-token form can run this stage: reduction length with a tuned instantiation, token rows within the
+// LDS window above MK_MOE_X_OFFSET, collected outputs within the window below MK_MOE_OFFSET.
+__device__ __forceinline__ bool linear_small_ok(CStage &st, const Ctx &c, int M) {
+  if (M > 8 || (st.k != 4096 && st.k != 2048)) return false;
+  const int n_out = (st.flags & MK_F_SILU) ? st.n / 2 : st.n;
+  return (size_t)M * st.k * 2 <= (size_t)(MK_LDS_BYTES - MK_MOE_X_OFFSET) && (size_t)M * (n_out / c.G + 1) * 2 <= (size_t)MK_MOE_OFFSET;
+}
+
+template <int MB>
+__device__ __forceinline__ void stage_linear_small_dispatch(CStage &st, Ctx &c, int M, char *smem) {
+  const bool silu = st.flags & MK_F_SILU;
+  if (st.k == 4096) {
+    if (silu) stage_linear_small<8, 4, true, MB>(st, c, M, smem);
+    else stage_linear_small<8, 4, false, MB>(st, c, M, smem);
+  } else {
+    if (silu) stage_linear_small<4, 4, true, MB>(st, c, M, smem);
+    else stage_linear_small<4, 4, false, MB>(st, c, M, smem);
+  }
+}
+
 #ifndef MK_TUNE_NBN
 #define MK_TUNE_NBN 4
 #endif
@@ -2219,7 +2385,11 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
         case MK_OP_LINEAR:
           if (M == 1) stage_linear_m1(st, c, smem);
-          else {
+          else if (linear_small_ok(st, c, M)) {
+            if (M <= 2) stage_linear_small_dispatch<2>(st, c, M, smem);
+            else if (M <= 4) stage_linear_small_dispatch<4>(st, c, M, smem);
+            else stage_linear_small_dispatch<8>(st, c, M, smem);
+          } else {
             const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
             const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
             if (narrow) {
