@@ -1203,6 +1203,10 @@ int mk_compile(mk_graph *g) {
   g->d_stages = (MkStage *)p;
   rt.stages = g->d_stages;
   if (!g->stages.empty()) HIP_TRY(hipMemcpy(g->d_stages, g->stages.data(), sizeof(MkStage) * g->stages.size(), hipMemcpyHostToDevice));
+  if ((rc = dev_alloc(g, &p, (size_t)g->G * 4 * 4 * 64 * 16, false))) return rc;
+  rt.splitk_part = p;
+  if ((rc = dev_alloc(g, &p, (size_t)g->G * 32 * sizeof(unsigned)))) return rc;
+  rt.splitk_cnt = (unsigned *)p;
   g->timing_cap = 8192;
   if ((rc = dev_alloc(g, &p, sizeof(long long) * (g->timing_cap + 2)))) return rc;
   rt.timing = g->d_timing = (long long *)p;

@@ -10,6 +10,7 @@
 // (include/mirage/persistent_kernel/tasks/mi300/*.cuh).
 #include <hip/hip_runtime.h>
 #include <stdint.h>
+#include <type_traits>
 #include "mk_types.h"
 
 typedef unsigned u32x4 __attribute__((ext_vector_type(4)));
@@ -840,6 +841,169 @@ __device__ __forceinline__ void stage_linear_small_dispatch(CStage &st, Ctx &c, 
   } else {
     if (silu) stage_linear_small<4, 4, true, MB>(st, c, M, smem);
     else stage_linear_small<4, 4, false, MB>(st, c, M, smem);
+  }
+}
+
+// Split-K matrix-core linear for stages with few output tiles (N = 4096 on 256 workgroups is one 16-column tile per
+// workgroup): S workgroups share a group of four output tiles, each takes a K/S slice; inside a workgroup every
+// wavefront owns ONE tile and all four use the same token-row slice, which is staged once per 64-wide step in LDS
+// (double-buffered, laid out so that the matrix-core operand reads are linear in the lane index) instead of being
+// pulled from L2 by every wavefront.  A workgroup thus reads 1/S of the token rows; weight steps sit NB deep in
+// registers.  The S partial tiles go through a write-through buffer; the last workgroup of a group to arrive sums
+// them in slice order (deterministic), applies the residual and stores bf16.
+// Reference tasks: splitk_linear (tasks/mi300/linear_ck_mi300.cuh split-K variants), gang_splitk_linear_res_mi300.
+#ifndef MK_TUNE_SPLITK_MAXS
+#define MK_TUNE_SPLITK_MAXS 8
+#endif
+#ifndef MK_TUNE_SPLITK_INV
+#define MK_TUNE_SPLITK_INV 0
+#endif
+#define MK_SPLITK_NB 8  // 64-wide k steps held in registers per wavefront; a workgroup's K slice is a multiple of it
+template <int MT>
+__device__ __forceinline__ void stage_linear_mfma_splitk(CStage &st, Ctx &c, const MkRuntime &rt, int M, int S, char *smem) {
+  constexpr int NB = MK_SPLITK_NB;
+  constexpr int NXC = (MT * 128 + MK_THREADS - 1) / MK_THREADS;  // 16-byte token-row segments per thread and step
+  barrier_wait(c);
+  if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+  __syncthreads();
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const int K = st.k, k8 = K / 8, n_out = st.n;
+  const int ntiles = (n_out + 15) / 16;
+  const int g = c.vid / S, sl = c.vid - g * S;
+  if (g * 4 >= ntiles) return;  // workgroups beyond the last group have nothing to do in this stage
+  const int tile = g * 4 + wave;
+  const bool has_tile = tile < ntiles;
+  const int kslice = K / S, kbeg = sl * kslice, nsteps = kslice >> 6;
+  const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
+  const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
+  const uint16_t *wrow = (const uint16_t *)weight_row(st.w, min(tile * 16 + lr, n_out - 1), k8) + kbeg + lg * 16;
+  u32x4 *xl = (u32x4 *)smem;  // two buffers of [MT][2][64] 16-byte operands
+  int *sflag = (int *)(smem + 2 * MT * 2048);
+  // this thread's token-row segments: segment ci -> token ci / 8, 16-byte piece ci % 8 of the 128-byte step
+  const uint16_t *xsrc[NXC];
+  int xdst[NXC];
+#pragma unroll
+  for (int i = 0; i < NXC; i++) {
+    const int ci = tid + i * MK_THREADS, m = ci >> 3, cc = ci & 7;
+    xsrc[i] = x + (size_t)min(m, M - 1) * ldx + kbeg + cc * 8;
+    xdst[i] = (((m >> 4) * 2 + (cc & 1)) * 64) + (cc >> 1) * 16 + (m & 15);
+  }
+  auto x_load = [&](int step, u32x4 (&q)[NXC]) {
+#pragma unroll
+    for (int i = 0; i < NXC; i++) q[i] = *(const u32x4 *)(xsrc[i] + (step << 6));  // unconditional (surplus threads re-read the last token's row): a load under a branch spoils the wait counts
+  };
+  auto x_store = [&](int buf, const u32x4 (&q)[NXC]) {
+#pragma unroll
+    for (int i = 0; i < NXC; i++)
+      if ((i + 1) * MK_THREADS <= MT * 128 || tid + i * MK_THREADS < MT * 128) xl[buf * MT * 128 + xdst[i]] = q[i];
+  };
+  bf16x8 a[NB][2];
+  auto w_load = [&](int step, bf16x8 (&aa)[2]) {
+    aa[0] = __builtin_nontemporal_load((const bf16x8 *)(wrow + (step << 6)));
+    aa[1] = __builtin_nontemporal_load((const bf16x8 *)(wrow + (step << 6) + 8));
+  };
+  // Loads return in issue order, so token-row segments are prefetched exactly as deep as the weights (a wait for a
+  // younger token-row load would drain every older weight load with it).
+  u32x4 xq[NB][NXC];
+#pragma unroll
+  for (int j = 0; j < NB; j++) {
+    w_load(j, a[j]);  // wavefronts without a tile load a clamped row and ignore it
+    x_load(j, xq[j]);
+  }
+  x_store(0, xq[0]);
+  __syncthreads();
+  f32x4 acc[MT];
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+  // nsteps is a multiple of NB: every block but the last refills its ring slots unconditionally, so the compiler's
+  // wait counts stay exact (a load under a condition makes every later wait a full drain).
+  auto block = [&](int s0, auto refill) {
+    constexpr bool REFILL = decltype(refill)::value;
+#pragma unroll
+    for (int j = 0; j < NB; j++) {
+      const int step = s0 + j;
+      if (REFILL || j + 1 < NB) x_store((step + 1) & 1, xq[(j + 1) % NB]);  // that buffer was last read before the previous barrier
+      if (has_tile) {
+        const u32x4 *xb = xl + (step & 1) * MT * 128;
+        u32x4 b[2][MT];
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++) b[h][mt] = xb[(mt * 2 + h) * 64 + lane];
+        __builtin_amdgcn_sched_barrier(0);  // all operand reads in flight before the first matrix instruction waits
+#pragma unroll
+        for (int h = 0; h < 2; h++)
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++)
+            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][h], __builtin_bit_cast(bf16x8, b[h][mt]), acc[mt], 0, 0, 0);
+      }
+      if (REFILL) {
+        w_load(step + NB, a[j]);
+        x_load(step + NB, xq[j]);
+      }
+      __syncthreads();
+    }
+  };
+  int s0 = 0;
+  for (; s0 + NB < nsteps; s0 += NB) block(s0, std::true_type{});
+  block(s0, std::false_type{});
+  // ---- combine the S slices
+  if (S > 1) {
+    u32x4 *part = (u32x4 *)rt.splitk_part;
+    if (has_tile) {
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) stc_16B(part + (((size_t)c.vid * 4 + wave) * 4 + mt) * 64 + lane, __builtin_bit_cast(u32x4, acc[mt]));
+    }
+    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    __syncthreads();
+    if (tid == 0) {
+      unsigned *cnt = rt.splitk_cnt + (size_t)g * 32;
+      const int last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(S - 1);
+      if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+      if (MK_TUNE_SPLITK_INV && last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      *sflag = last;
+    }
+    __syncthreads();
+    if (!*sflag) return;
+    if (has_tile) {
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int q0 = 0; q0 < S; q0 += 4) {  // four slices requested at once; summed in slice order
+        u32x4 pv[4][MT];
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          if (q0 + q < S) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) pv[q][mt] = ldc_16B(part + (((size_t)(g * S + q0 + q) * 4 + wave) * 4 + mt) * 64 + lane);
+          }
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          if (q0 + q < S) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++) acc[mt] += __builtin_bit_cast(f32x4, pv[q][mt]);
+          }
+      }
+    }
+  }
+  if (!has_tile) return;
+  // ---- epilogue: lane l holds token m = mt * 16 + (l & 15), output columns tile * 16 + (l >> 4) * 4 .. + 3
+#pragma unroll
+  for (int mt = 0; mt < MT; mt++) {
+    const int m = mt * 16 + lr;
+    if (m < M) {
+      uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
+      const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
+#pragma unroll
+      for (int i = 0; i < 4; i++) {
+        const int n = tile * 16 + lg * 4 + i;
+        if (n < n_out) {
+          float r = acc[mt][i];
+          if (st.flags & MK_F_RES) r += bf2f(rrow[n]);
+          orow[n] = (uint16_t)f2bf(r);
+        }
+      }
+    }
   }
 }
 
@@ -2139,7 +2303,8 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
           last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(C - 1);
           if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        *sflag = last;
+        if (MK_TUNE_SPLITK_INV && last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+      *sflag = last;
       }
       __syncthreads();
       if (*sflag) {
@@ -2392,7 +2557,19 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
           } else {
             const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
             const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
-            if (narrow) {
+            // split-K form: groups of four tiles, S workgroups per group
+            const int groups = (wt + 3) / 4;
+            int S = 0;
+            if (!(flags & MK_F_SILU) && groups <= c.G && st.k % (64 * MK_SPLITK_NB) == 0) {
+              S = 1;
+              while (S < MK_TUNE_SPLITK_MAXS && groups * S * 2 <= c.G && st.k % (S * 2 * 64 * MK_SPLITK_NB) == 0) S *= 2;
+            }
+            if (narrow && S >= 1) {
+              if (M <= 16) stage_linear_mfma_splitk<1>(st, c, rt, M, S, smem);
+              else if (M <= 32) stage_linear_mfma_splitk<2>(st, c, rt, M, S, smem);
+              else if (M <= 48) stage_linear_mfma_splitk<3>(st, c, rt, M, S, smem);
+              else stage_linear_mfma_splitk<4>(st, c, rt, M, S, smem);
+            } else if (narrow) {
               if (M <= 16) stage_linear_mfma<1, 2, 2 * MK_TUNE_NBN>(st, c, M, smem);
               else if (M <= 32) stage_linear_mfma<2, 2, MK_TUNE_NBN + MK_TUNE_NBN / 2>(st, c, M, smem);
               else if (M <= 48) stage_linear_mfma<3, 2, MK_TUNE_NBN>(st, c, M, smem);

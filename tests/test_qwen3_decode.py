@@ -151,12 +151,16 @@ def test_batched_decode_independent_prompts(B, R_total, mode):
 
 def test_batch_rows_with_same_prompt_agree():
     """The reference driver's self-check (demo/qwen3/demo.py:1281-1301): identical prompts in every slot must produce
-    identical tokens in every row."""
+    identical tokens in every row.  As in that driver the token budget holds every prompt at once, so all rows prefill
+    in one iteration and decode in lockstep: every row then sees the same batch size in every iteration and therefore
+    the same kernel forms and summation orders, and the rows must agree bit for bit.  (With a smaller budget the rows
+    finish in different iterations, the stragglers run at smaller batch sizes through other kernel forms, and tokens
+    with a tiny top-2 margin may legitimately differ.)"""
     from oracle.qwen3_ref import make_model_weights, make_prompt
     cfg = _small_cfg()
     w = make_model_weights(cfg, seed=22)
-    prompt = make_prompt(cfg, 11, 7)
-    dec = _decoder(cfg, w, max_num_batched_tokens=8, max_num_batched_requests=8, max_seq_length=36, page_size=16)
+    prompt = make_prompt(cfg, 8, 7)
+    dec = _decoder(cfg, w, max_num_batched_tokens=64, max_num_batched_requests=8, max_seq_length=36, page_size=16)
     toks, _ = dec.generate([prompt] * 8)
     for r in range(1, 8):
         assert torch.equal(toks[r], toks[0]), f"row {r} differs from row 0"
