@@ -862,7 +862,7 @@ __device__ __forceinline__ void stage_linear_small_dispatch(CStage &st, Ctx &c, 
 template <int MT>
 __device__ __forceinline__ void stage_linear_mfma_splitk(CStage &st, Ctx &c, const MkRuntime &rt, int M, int S, char *smem) {
   constexpr int NB = MK_SPLITK_NB;
-  constexpr int NXC = (MT * 128 + MK_THREADS - 1) / MK_THREADS;  // 16-byte token-row segments per thread and step
+  constexpr int NXC = 2;  // 16-byte token-row segments per thread and step
   barrier_wait(c);
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   __syncthreads();
@@ -880,23 +880,19 @@ __device__ __forceinline__ void stage_linear_mfma_splitk(CStage &st, Ctx &c, con
   const uint16_t *wrow = (const uint16_t *)weight_row(st.w, min(tile * 16 + lr, n_out - 1), k8) + kbeg + lg * 16;
   u32x4 *xl = (u32x4 *)smem;  // two buffers of [MT][2][64] 16-byte operands
   int *sflag = (int *)(smem + 2 * MT * 2048);
-  // this thread's token-row segments: segment ci -> token ci / 8, 16-byte piece ci % 8 of the 128-byte step
-  const uint16_t *xsrc[NXC];
-  int xdst[NXC];
-#pragma unroll
-  for (int i = 0; i < NXC; i++) {
-    const int ci = tid + i * MK_THREADS, m = ci >> 3, cc = ci & 7;
-    xsrc[i] = x + (size_t)min(m, M - 1) * ldx + kbeg + cc * 8;
-    xdst[i] = (((m >> 4) * 2 + (cc & 1)) * 64) + (cc >> 1) * 16 + (m & 15);
-  }
-  auto x_load = [&](int step, u32x4 (&q)[NXC]) {
-#pragma unroll
-    for (int i = 0; i < NXC; i++) q[i] = *(const u32x4 *)(xsrc[i] + (step << 6));  // unconditional (surplus threads re-read the last token's row): a load under a branch spoils the wait counts
+  // token rows: wavefront w stages token tile w, every lane the same 32 contiguous bytes it would feed the matrix core
+  // with, stored at its own lane slot of the operand block (consecutive 16-byte slots: no bank conflicts either way)
+  const uint16_t *xsrc = x + (size_t)min(min(wave, MT - 1) * 16 + lr, M - 1) * ldx + kbeg + lg * 16;
+  const int xdst = min(wave, MT - 1) * 128 + lane;
+  auto x_load = [&](int step, u32x4 (&q)[NXC]) {  // unconditional (surplus wavefronts re-read a row): a load under a branch spoils the wait counts
+    q[0] = *(const u32x4 *)(xsrc + (step << 6));
+    q[1] = *(const u32x4 *)(xsrc + (step << 6) + 8);
   };
   auto x_store = [&](int buf, const u32x4 (&q)[NXC]) {
-#pragma unroll
-    for (int i = 0; i < NXC; i++)
-      if ((i + 1) * MK_THREADS <= MT * 128 || tid + i * MK_THREADS < MT * 128) xl[buf * MT * 128 + xdst[i]] = q[i];
+    if (wave < MT) {
+      xl[buf * MT * 128 + xdst] = q[0];
+      xl[buf * MT * 128 + xdst + 64] = q[1];
+    }
   };
   bf16x8 a[NB][2];
   auto w_load = [&](int step, bf16x8 (&aa)[2]) {
@@ -1995,6 +1991,9 @@ __device__ __forceinline__ void head_row_finish(float x0, float x1, uint16_t *ds
   dst[lane + 64] = (uint16_t)f2bf(x1);
 }
 
+#ifndef MK_TUNE_NPRE
+#define MK_TUNE_NPRE 4
+#endif
 struct AttnUnit {
   int t, h, cidx, C, start, end, p, p0, t0, new_lo, n_new, cend;
   const int *pages;
@@ -2018,7 +2017,7 @@ struct AttnUnit {
 template <int QPK>
 __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
   constexpr int D = 128;
-  constexpr int NPRE = 4;                     // positions per lane group requested ahead
+  constexpr int NPRE = MK_TUNE_NPRE;          // positions per lane group requested ahead
   constexpr int DPT = QPK * D / MK_THREADS;   // merged outputs per thread (all of one head)
   constexpr int TPH = D / DPT;                // threads per head in the merges
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -2217,24 +2216,25 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       pos += 16 * NPRE;
     }
     // later blocks: the next block's rows are in flight while the current one is reduced
+    // Every load is issued unconditionally (positions beyond the chunk re-read its last row and are masked in
+    // process_block): a load under a branch would turn the wait for the current block into a wait for the next one too.
     auto load_block = [&](int p0, u32x4 (&kk)[NPRE], u32x4 (&vv)[NPRE]) {
 #pragma unroll
-      for (int i = 0; i < NPRE; i++)
-        if (p0 + 16 * i < a.cend) {
-          const size_t off = kvoff(a, p0 + 16 * i);
-          kk[i] = kc[off];
-          vv[i] = vc[off];
-        }
+      for (int i = 0; i < NPRE; i++) {
+        const size_t off = kvoff(a, min(p0 + 16 * i, a.cend - 1));
+        kk[i] = kc[off];
+        vv[i] = vc[off];
+      }
     };
     if (pos < a.cend) {
       u32x4 ka[NPRE], va[NPRE], kb[NPRE], vb[NPRE];
       load_block(pos, ka, va);
       while (true) {
-        if (pos + 16 * NPRE < a.cend) load_block(pos + 16 * NPRE, kb, vb);
+        load_block(pos + 16 * NPRE, kb, vb);
         process_block(ka, va, pos);
         pos += 16 * NPRE;
         if (pos >= a.cend) break;
-        if (pos + 16 * NPRE < a.cend) load_block(pos + 16 * NPRE, ka, va);
+        load_block(pos + 16 * NPRE, ka, va);
         process_block(kb, vb, pos);
         pos += 16 * NPRE;
         if (pos >= a.cend) break;
