@@ -1203,7 +1203,7 @@ int mk_compile(mk_graph *g) {
   g->d_stages = (MkStage *)p;
   rt.stages = g->d_stages;
   if (!g->stages.empty()) HIP_TRY(hipMemcpy(g->d_stages, g->stages.data(), sizeof(MkStage) * g->stages.size(), hipMemcpyHostToDevice));
-  if ((rc = dev_alloc(g, &p, (size_t)g->G * 4 * 4 * 64 * 16, false))) return rc;
+  if ((rc = dev_alloc(g, &p, (size_t)g->G * 4 * 4 * 4 * 64 * 16, false))) return rc;
   rt.splitk_part = p;
   if ((rc = dev_alloc(g, &p, (size_t)g->G * 32 * sizeof(unsigned)))) return rc;
   rt.splitk_cnt = (unsigned *)p;

@@ -542,7 +542,6 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
     }
     if (c.pending && tid == 0) barrier_poll(c);
     stage_x_m1_wave<KL>(st, c, xs, lane, nwv);
-
   }
   __syncthreads();
   barrier_done(c);
@@ -844,161 +843,270 @@ __device__ __forceinline__ void stage_linear_small_dispatch(CStage &st, Ctx &c, 
   }
 }
 
-// Split-K matrix-core linear for stages with few output tiles (N = 4096 on 256 workgroups is one 16-column tile per
-// workgroup): S workgroups share a group of four output tiles, each takes a K/S slice; inside a workgroup every
-// wavefront owns ONE tile and all four use the same token-row slice, which is staged once per 64-wide step in LDS
-// (double-buffered, laid out so that the matrix-core operand reads are linear in the lane index) instead of being
-// pulled from L2 by every wavefront.  A workgroup thus reads 1/S of the token rows; weight steps sit NB deep in
-// registers.  The S partial tiles go through a write-through buffer; the last workgroup of a group to arrive sums
-// them in slice order (deterministic), applies the residual and stores bf16.
-// Reference tasks: splitk_linear (tasks/mi300/linear_ck_mi300.cuh split-K variants), gang_splitk_linear_res_mi300.
+// Matrix-core linear for several tokens.  A workgroup owns a range of 16-row weight tiles and one K slice (S slices
+// per range when a stage has too few tiles to fill the machine, S = 1 otherwise).  The range is worked off in sweeps:
+// every wavefront holds TW tiles of the sweep over the whole slice, and all four share the token rows of the slice,
+// which one pass stages per 64-wide step in LDS (double-buffered, in matrix-core operand order, so the reads are linear
+// in the lane index).  Token-row traffic per weight byte is M / (64 TW); weight steps sit NB deep in registers.
+//
+// Every load is unconditional and the step loop has a fixed trip structure (slices are multiples of NB steps; slots
+// past the range re-read its last tile): a load under a branch makes the compiler's wait counts drain everything
+// younger, which costs the whole prefetch depth.  Loads return in issue order, so token rows are prefetched exactly as
+// deep as the weights.
+//
+// With S > 1 the partial tiles go through a write-through buffer; the last workgroup of a group to arrive sums them in
+// slice order (deterministic), applies SwiGLU / residual and stores bf16.  SwiGLU stages number their weight tiles
+// gate, up, gate, up ... so that a pair always sits in one wavefront.
+// Reference tasks: linear / linear_with_residual / splitk_linear (tasks/mi300/linear_ck_mi300.cuh), silu_mul_linear.
 #ifndef MK_TUNE_SPLITK_MAXS
 #define MK_TUNE_SPLITK_MAXS 8
 #endif
-#ifndef MK_TUNE_SPLITK_INV
-#define MK_TUNE_SPLITK_INV 0
+#ifndef MK_TUNE_TPU
+#define MK_TUNE_TPU 4  // tiles per workgroup a split stage aims for
 #endif
-#define MK_SPLITK_NB 8  // 64-wide k steps held in registers per wavefront; a workgroup's K slice is a multiple of it
+#ifndef MK_TUNE_NB1
+#define MK_TUNE_NB1 8
+#endif
+#ifndef MK_TUNE_NB2
+#define MK_TUNE_NB2 4
+#endif
+#ifndef MK_TUNE_NB4
+#define MK_TUNE_NB4 2
+#endif
+#ifndef MK_TUNE_TILES_MIN_TPW
+#define MK_TUNE_TILES_MIN_TPW 16
+#endif
+#define MK_TILES_NB 4  // a K slice is a multiple of 64 * 2 * MK_TILES_NB (the deepest instantiation's ring)
+
+struct TilePlan {
+  int S;       // K slices per tile range (0: this form cannot run the stage)
+  int groups;  // tile ranges
+  int wt;      // weight tiles of the stage
+};
+__device__ __forceinline__ TilePlan linear_tiles_plan(CStage &st, const Ctx &c) {
+  TilePlan p;
+  const bool silu = st.flags & MK_F_SILU;
+  const int n_out = silu ? st.n / 2 : st.n;
+  const int unit = silu ? 2 : 1;                      // ranges are made of whole gate/up pairs
+  p.wt = ((n_out + 15) / 16) * unit;
+  p.S = 0;
+  p.groups = 0;
+  if (st.k % (64 * 2 * MK_TILES_NB) != 0) return p;
+  const int tpw = (p.wt + c.G - 1) / c.G;            // tiles per workgroup without a K split
+  int S = 1;
+  while (S < MK_TUNE_SPLITK_MAXS && tpw * S < MK_TUNE_TPU && st.k % (S * 2 * 64 * 2 * MK_TILES_NB) == 0) S *= 2;
+  int tpu = (p.wt * S + c.G - 1) / c.G;              // tiles per range
+  tpu = (tpu + unit - 1) / unit * unit;
+  if (S > 1 && tpu > 16) return p;                    // a split range is a single sweep
+  if (S == 1 && tpw < MK_TUNE_TILES_MIN_TPW) return p;  // a few tiles per workgroup without a K split: the form that splits K inside the workgroup
+  p.groups = (p.wt + tpu - 1) / tpu;
+  p.S = S;
+  return p;
+}
+
 template <int MT>
-__device__ __forceinline__ void stage_linear_mfma_splitk(CStage &st, Ctx &c, const MkRuntime &rt, int M, int S, char *smem) {
-  constexpr int NB = MK_SPLITK_NB;
-  constexpr int NXC = 2;  // 16-byte token-row segments per thread and step
+__device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, const MkRuntime &rt, int M, const TilePlan plan, char *smem) {
   barrier_wait(c);
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   __syncthreads();
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
-  const int K = st.k, k8 = K / 8, n_out = st.n;
-  const int ntiles = (n_out + 15) / 16;
+  const bool silu = st.flags & MK_F_SILU;
+  const int K = st.k, k8 = K / 8;
+  const int n_out = silu ? st.n / 2 : st.n;
+  const int half = st.silu_half;
+  const int S = plan.S, unit = silu ? 2 : 1;
   const int g = c.vid / S, sl = c.vid - g * S;
-  if (g * 4 >= ntiles) return;  // workgroups beyond the last group have nothing to do in this stage
-  const int tile = g * 4 + wave;
-  const bool has_tile = tile < ntiles;
+  if (g >= plan.groups) return;  // workgroups beyond the last range have nothing to do in this stage
+  // balanced ranges of whole units
+  const int nun = plan.wt / unit;
+  const int tb = (int)(((long long)g * nun) / plan.groups) * unit, te = (int)(((long long)(g + 1) * nun) / plan.groups) * unit;
   const int kslice = K / S, kbeg = sl * kslice, nsteps = kslice >> 6;
   const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
   const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
-  const uint16_t *wrow = (const uint16_t *)weight_row(st.w, min(tile * 16 + lr, n_out - 1), k8) + kbeg + lg * 16;
   u32x4 *xl = (u32x4 *)smem;  // two buffers of [MT][2][64] 16-byte operands
   int *sflag = (int *)(smem + 2 * MT * 2048);
   // token rows: wavefront w stages token tile w, every lane the same 32 contiguous bytes it would feed the matrix core
   // with, stored at its own lane slot of the operand block (consecutive 16-byte slots: no bank conflicts either way)
   const uint16_t *xsrc = x + (size_t)min(min(wave, MT - 1) * 16 + lr, M - 1) * ldx + kbeg + lg * 16;
   const int xdst = min(wave, MT - 1) * 128 + lane;
-  auto x_load = [&](int step, u32x4 (&q)[NXC]) {  // unconditional (surplus wavefronts re-read a row): a load under a branch spoils the wait counts
-    q[0] = *(const u32x4 *)(xsrc + (step << 6));
-    q[1] = *(const u32x4 *)(xsrc + (step << 6) + 8);
-  };
-  auto x_store = [&](int buf, const u32x4 (&q)[NXC]) {
-    if (wave < MT) {
-      xl[buf * MT * 128 + xdst] = q[0];
-      xl[buf * MT * 128 + xdst + 64] = q[1];
+  // first weight row of weight tile ti for this lane
+  auto tile_row = [&](int ti) -> const uint16_t * {
+    int o, vr;
+    if (silu) {
+      o = min((ti >> 1) * 16 + lr, n_out - 1);
+      const int gi = o / half;
+      vr = gi * 2 * half + (o - gi * half) + ((ti & 1) ? half : 0);
+    } else {
+      o = min(ti * 16 + lr, n_out - 1);
+      vr = o;
     }
+    return (const uint16_t *)weight_row(st.w, vr, k8) + kbeg + lg * 16;
   };
-  bf16x8 a[NB][2];
-  auto w_load = [&](int step, bf16x8 (&aa)[2]) {
-    aa[0] = __builtin_nontemporal_load((const bf16x8 *)(wrow + (step << 6)));
-    aa[1] = __builtin_nontemporal_load((const bf16x8 *)(wrow + (step << 6) + 8));
-  };
-  // Loads return in issue order, so token-row segments are prefetched exactly as deep as the weights (a wait for a
-  // younger token-row load would drain every older weight load with it).
-  u32x4 xq[NB][NXC];
+  u32x4 *part = (u32x4 *)rt.splitk_part;
+
+  auto sweep = [&](int t0, auto twc) {
+    constexpr int TW = decltype(twc)::value;
+    constexpr int NB = TW == 1 ? MK_TUNE_NB1 : (TW == 2 ? MK_TUNE_NB2 : MK_TUNE_NB4);
+    const int tw0 = t0 + wave * TW;           // this wavefront's first tile
+    const bool has_tile = tw0 < te;           // wavefronts without one only stage token rows and keep the barriers
+    const uint16_t *wrow[TW];
 #pragma unroll
-  for (int j = 0; j < NB; j++) {
-    w_load(j, a[j]);  // wavefronts without a tile load a clamped row and ignore it
-    x_load(j, xq[j]);
-  }
-  x_store(0, xq[0]);
-  __syncthreads();
-  f32x4 acc[MT];
+    for (int t = 0; t < TW; t++) wrow[t] = tile_row(min(tw0 + t, te - 1));
+    bf16x8 a[NB][TW][2];
+    u32x4 xq[NB][2];
+    auto w_load = [&](int step, bf16x8 (&aa)[TW][2]) {
 #pragma unroll
-  for (int mt = 0; mt < MT; mt++) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-  // nsteps is a multiple of NB: every block but the last refills its ring slots unconditionally, so the compiler's
-  // wait counts stay exact (a load under a condition makes every later wait a full drain).
-  auto block = [&](int s0, auto refill) {
-    constexpr bool REFILL = decltype(refill)::value;
+      for (int t = 0; t < TW; t++) {
+        aa[t][0] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + (step << 6)));
+        aa[t][1] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + (step << 6) + 8));
+      }
+    };
+    auto x_load = [&](int step, u32x4 (&q)[2]) {
+      q[0] = *(const u32x4 *)(xsrc + (step << 6));
+      q[1] = *(const u32x4 *)(xsrc + (step << 6) + 8);
+    };
+    auto x_store = [&](int buf, const u32x4 (&q)[2]) {
+      if (wave < MT) {
+        xl[buf * MT * 128 + xdst] = q[0];
+        xl[buf * MT * 128 + xdst + 64] = q[1];
+      }
+    };
+    f32x4 acc[TW][MT];
 #pragma unroll
-    for (int j = 0; j < NB; j++) {
-      const int step = s0 + j;
-      if (REFILL || j + 1 < NB) x_store((step + 1) & 1, xq[(j + 1) % NB]);  // that buffer was last read before the previous barrier
+    for (int t = 0; t < TW; t++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    // Two copies of the step loop, for wavefronts with and without tiles: a branch around the weight loads inside one
+    // copy would spoil its wait counts.  Both execute the same barriers.
+    auto pipeline = [&](auto htc) {
+      constexpr bool HT = decltype(htc)::value;
+      __syncthreads();  // the previous sweep has finished with the LDS buffers
+#pragma unroll
+      for (int j = 0; j < NB; j++) {
+        if (HT) w_load(j, a[j]);
+        x_load(j, xq[j]);
+      }
+      x_store(0, xq[0]);
+      __syncthreads();
+      auto block = [&](int s0, auto refill) {
+        constexpr bool REFILL = decltype(refill)::value;
+#pragma unroll
+        for (int j = 0; j < NB; j++) {
+          const int step = s0 + j;
+          if (REFILL || j + 1 < NB) x_store((step + 1) & 1, xq[(j + 1) % NB]);  // that buffer was last read before the previous barrier
+          if (HT) {
+            const u32x4 *xb = xl + (step & 1) * MT * 128;
+            u32x4 b[2][MT];
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+              for (int mt = 0; mt < MT; mt++) b[h][mt] = xb[(mt * 2 + h) * 64 + lane];
+            __builtin_amdgcn_sched_barrier(0);  // all operand reads in flight before the first matrix instruction waits
+#pragma unroll
+            for (int h = 0; h < 2; h++)
+#pragma unroll
+              for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+                for (int t = 0; t < TW; t++)
+                  acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][t][h], __builtin_bit_cast(bf16x8, b[h][mt]), acc[t][mt], 0, 0, 0);
+          }
+          if (REFILL) {
+            if (HT) w_load(step + NB, a[j]);
+            x_load(step + NB, xq[j]);
+          }
+          __syncthreads();
+        }
+      };
+      int s0 = 0;
+      for (; s0 + NB < nsteps; s0 += NB) block(s0, std::true_type{});
+      block(s0, std::false_type{});
+    };
+    if (has_tile) pipeline(std::true_type{});
+    else pipeline(std::false_type{});
+
+    // ---- combine the S slices (a split range is a single sweep, so slots are indexed by wavefront and tile only)
+    if (S > 1) {
       if (has_tile) {
-        const u32x4 *xb = xl + (step & 1) * MT * 128;
-        u32x4 b[2][MT];
 #pragma unroll
-        for (int h = 0; h < 2; h++)
-#pragma unroll
-          for (int mt = 0; mt < MT; mt++) b[h][mt] = xb[(mt * 2 + h) * 64 + lane];
-        __builtin_amdgcn_sched_barrier(0);  // all operand reads in flight before the first matrix instruction waits
-#pragma unroll
-        for (int h = 0; h < 2; h++)
+        for (int t = 0; t < TW; t++)
 #pragma unroll
           for (int mt = 0; mt < MT; mt++)
-            acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a[j][h], __builtin_bit_cast(bf16x8, b[h][mt]), acc[mt], 0, 0, 0);
+            stc_16B(part + ((((size_t)c.vid * 4 + wave) * 4 + t) * 4 + mt) * 64 + lane, __builtin_bit_cast(u32x4, acc[t][mt]));
       }
-      if (REFILL) {
-        w_load(step + NB, a[j]);
-        x_load(step + NB, xq[j]);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0) {
+        unsigned *cnt = rt.splitk_cnt + (size_t)g * 32;
+        const int last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(S - 1);
+        if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        *sflag = last;
       }
       __syncthreads();
-    }
-  };
-  int s0 = 0;
-  for (; s0 + NB < nsteps; s0 += NB) block(s0, std::true_type{});
-  block(s0, std::false_type{});
-  // ---- combine the S slices
-  if (S > 1) {
-    u32x4 *part = (u32x4 *)rt.splitk_part;
-    if (has_tile) {
+      if (!*sflag || !has_tile) return;
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) stc_16B(part + (((size_t)c.vid * 4 + wave) * 4 + mt) * 64 + lane, __builtin_bit_cast(u32x4, acc[mt]));
-    }
-    asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
-    __syncthreads();
-    if (tid == 0) {
-      unsigned *cnt = rt.splitk_cnt + (size_t)g * 32;
-      const int last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(S - 1);
-      if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
-      if (MK_TUNE_SPLITK_INV && last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      *sflag = last;
-    }
-    __syncthreads();
-    if (!*sflag) return;
-    if (has_tile) {
+      for (int t = 0; t < TW; t++) {
 #pragma unroll
-      for (int mt = 0; mt < MT; mt++) acc[mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-      for (int q0 = 0; q0 < S; q0 += 4) {  // four slices requested at once; summed in slice order
-        u32x4 pv[4][MT];
+        for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+        for (int q0 = 0; q0 < S; q0 += 4) {  // four slices requested at once; summed in slice order
+          u32x4 pv[4][MT];
 #pragma unroll
-        for (int q = 0; q < 4; q++)
-          if (q0 + q < S) {
+          for (int q = 0; q < 4; q++)
+            if (q0 + q < S) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) pv[q][mt] = ldc_16B(part + (((size_t)(g * S + q0 + q) * 4 + wave) * 4 + mt) * 64 + lane);
-          }
+              for (int mt = 0; mt < MT; mt++) pv[q][mt] = ldc_16B(part + ((((size_t)(g * S + q0 + q) * 4 + wave) * 4 + t) * 4 + mt) * 64 + lane);
+            }
 #pragma unroll
-        for (int q = 0; q < 4; q++)
-          if (q0 + q < S) {
+          for (int q = 0; q < 4; q++)
+            if (q0 + q < S) {
 #pragma unroll
-            for (int mt = 0; mt < MT; mt++) acc[mt] += __builtin_bit_cast(f32x4, pv[q][mt]);
-          }
-      }
-    }
-  }
-  if (!has_tile) return;
-  // ---- epilogue: lane l holds token m = mt * 16 + (l & 15), output columns tile * 16 + (l >> 4) * 4 .. + 3
-#pragma unroll
-  for (int mt = 0; mt < MT; mt++) {
-    const int m = mt * 16 + lr;
-    if (m < M) {
-      uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
-      const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
-#pragma unroll
-      for (int i = 0; i < 4; i++) {
-        const int n = tile * 16 + lg * 4 + i;
-        if (n < n_out) {
-          float r = acc[mt][i];
-          if (st.flags & MK_F_RES) r += bf2f(rrow[n]);
-          orow[n] = (uint16_t)f2bf(r);
+              for (int mt = 0; mt < MT; mt++) acc[t][mt] += __builtin_bit_cast(f32x4, pv[q][mt]);
+            }
         }
       }
+    }
+    if (!has_tile) return;
+    // ---- epilogue: lane l holds token m = mt * 16 + (l & 15), output columns tile * 16 + (l >> 4) * 4 .. + 3
+    constexpr int OT = TW >= 2 ? TW / 2 : 1;
+#pragma unroll
+    for (int u = 0; u < (TW >= 2 ? TW : 1); u++) {
+      if (silu && u >= OT) break;
+      const int ti = silu ? tw0 + 2 * u : tw0 + u;
+      if (ti >= te) break;
+      const int otile = silu ? (ti >> 1) : ti;
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int m = mt * 16 + lr;
+        if (m < M) {
+          uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
+          const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int n = otile * 16 + lg * 4 + i;
+            if (n < n_out) {
+              float r;
+              if (silu) r = TW >= 2 ? silu_mul(acc[(2 * u) % TW][mt][i], acc[(2 * u + 1) % TW][mt][i]) : 0.f;
+              else r = acc[u][mt][i];
+              if (st.flags & MK_F_RES) r += bf2f(rrow[n]);
+              orow[n] = (uint16_t)f2bf(r);
+            }
+          }
+        }
+      }
+    }
+  };
+
+  for (int t0 = tb; t0 < te;) {
+    const int r = te - t0;
+    if (r > 8) {
+      sweep(t0, std::integral_constant<int, 4>{});
+      t0 += 16;
+    } else if (r > 4 || silu) {
+      sweep(t0, std::integral_constant<int, 2>{});
+      t0 += 8;
+    } else {
+      sweep(t0, std::integral_constant<int, 1>{});
+      t0 += 4;
     }
   }
 }
@@ -2303,8 +2411,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
           last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELEASE, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(C - 1);
           if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
         }
-        if (MK_TUNE_SPLITK_INV && last) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-      *sflag = last;
+        *sflag = last;
       }
       __syncthreads();
       if (*sflag) {
@@ -2557,18 +2664,12 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
           } else {
             const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
             const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
-            // split-K form: groups of four tiles, S workgroups per group
-            const int groups = (wt + 3) / 4;
-            int S = 0;
-            if (!(flags & MK_F_SILU) && groups <= c.G && st.k % (64 * MK_SPLITK_NB) == 0) {
-              S = 1;
-              while (S < MK_TUNE_SPLITK_MAXS && groups * S * 2 <= c.G && st.k % (S * 2 * 64 * MK_SPLITK_NB) == 0) S *= 2;
-            }
-            if (narrow && S >= 1) {
-              if (M <= 16) stage_linear_mfma_splitk<1>(st, c, rt, M, S, smem);
-              else if (M <= 32) stage_linear_mfma_splitk<2>(st, c, rt, M, S, smem);
-              else if (M <= 48) stage_linear_mfma_splitk<3>(st, c, rt, M, S, smem);
-              else stage_linear_mfma_splitk<4>(st, c, rt, M, S, smem);
+            const TilePlan plan = linear_tiles_plan(st, c);
+            if (plan.S >= 1) {
+              if (M <= 16) stage_linear_mfma_tiles<1>(st, c, rt, M, plan, smem);
+              else if (M <= 32) stage_linear_mfma_tiles<2>(st, c, rt, M, plan, smem);
+              else if (M <= 48) stage_linear_mfma_tiles<3>(st, c, rt, M, plan, smem);
+              else stage_linear_mfma_tiles<4>(st, c, rt, M, plan, smem);
             } else if (narrow) {
               if (M <= 16) stage_linear_mfma<1, 2, 2 * MK_TUNE_NBN>(st, c, M, smem);
               else if (M <= 32) stage_linear_mfma<2, 2, MK_TUNE_NBN + MK_TUNE_NBN / 2>(st, c, M, smem);

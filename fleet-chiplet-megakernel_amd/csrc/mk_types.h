@@ -159,7 +159,7 @@ struct MkRuntime {
   // attention split-KV workspace
   float *attn_part;     // [units][qpk][head_dim + 2]
   unsigned *attn_cnt;   // [max_tokens * num_kv_heads][32]: one 128-byte line per counter
-  void *splitk_part;    // [workgroups][4 wavefronts][4 token tiles][64 lanes] f32x4: K-slice partials of the split-K linear
+  void *splitk_part;    // [workgroups][4 wavefronts][4 weight tiles][4 token tiles][64 lanes] f32x4: K-slice partials of the split-K linear
   unsigned *splitk_cnt; // [workgroups][32]: arrival counter per split-K group (one 128-byte line each)
   long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end
   int timing_cap, pad0;
