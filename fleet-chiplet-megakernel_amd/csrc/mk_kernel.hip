@@ -733,10 +733,42 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
   barrier_done(c);
   // all four wavefronts stage the token rows (the workers' requests queue behind their weight rows, which were issued
   // long before)
-  const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
-  const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
+  const uint16_t *x = (const uint16_t *)st.in;
+  const int ldx = st.ld_in;
   u32x4 *xs4 = (u32x4 *)(smem + MK_MOE_X_OFFSET);  // [token][K8]
-  {
+  if (st.flags & MK_F_NORM) {
+    // Fused RMSNorm (the standalone NORM stage in front is skipped for these batch sizes): every workgroup normalises
+    // all rows itself, a wavefront per row, exactly as the single-token form does; virtual workgroup 0 also stores the
+    // normalised rows, which are the norm task's output tensor.
+    const u32x4 *nw4 = (const u32x4 *)st.norm_w;
+    for (int m = wave; m < M; m += MK_WAVES) {
+      const u32x4 *xr = (const u32x4 *)(x + (size_t)m * ldx);
+      u32x4 v[KL];
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) v[kc] = xr[kc * 64 + lane];
+      float ss = 0.f;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) {
+#pragma unroll
+        for (int e = 0; e < 4; e++) {
+          const uint32_t u = v[kc][e];
+          ss += bf_lo(u) * bf_lo(u) + bf_hi(u) * bf_hi(u);
+        }
+      }
+      ss = wave_sum(ss);
+      const float r = rsqrtf(ss / (float)(KL * 512) + st.eps);
+      u32x4 *no = (c.vid == 0) ? (u32x4 *)((uint16_t *)st.norm_out + (size_t)m * st.ld_norm) : nullptr;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) {
+        const u32x4 g = nw4[kc * 64 + lane];
+        u32x4 y;
+#pragma unroll
+        for (int e = 0; e < 4; e++) y[e] = pack2((bf_lo(v[kc][e]) * r) * bf_lo(g[e]), (bf_hi(v[kc][e]) * r) * bf_hi(g[e]));
+        xs4[m * K8 + kc * 64 + lane] = y;
+        if (no) stc_16B(no + kc * 64 + lane, y);
+      }
+    }
+  } else {
     constexpr int NCH = MB * KL / MK_WAVES;  // 16-byte segments per lane
     u32x4 xv[NCH];
 #pragma unroll
@@ -2651,6 +2683,11 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       CStage &st = ((CStage *)(unsigned long long)rt.stages)[s];
       const int op = st.op, flags = st.flags;
       if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
+      if ((flags & MK_F_ONLY_MULTI) && op == MK_OP_NORM && s + 1 < rt.num_stages) {
+        // the few-token linear normalises its rows itself
+        CStage &nx = ((CStage *)(unsigned long long)rt.stages)[s + 1];
+        if (nx.op == MK_OP_LINEAR && (nx.flags & MK_F_NORM) && nx.in == st.in && linear_small_ok(nx, c, M)) continue;
+      }
       const long long t_in = (long long)wall_clock64();
       switch (op) {
         case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
