@@ -695,11 +695,14 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
   const int n_loc = o_end - o_begin;
   int *ticket = c.sh_ticket + (c.seq & 1);
   const int half = st.silu_half;
-  auto take = [&]() -> int {
+  // Plain rows are drawn and reduced two at a time: a token-row segment read from LDS is used for both weight rows
+  // (half the LDS reads per output); a [gate ; up] pair already shares the segment.
+  constexpr int Q = SILU ? 1 : 2;  // outputs per ticket
+  static_assert(U == 2 * Q, "two groups of rows in flight");
+  auto take = [&]() -> int {  // first output of the next group of this workgroup (may lie at or beyond o_end)
     int t = 0;
-    if (lane == 0) t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    t = __builtin_amdgcn_readfirstlane(t) + o_begin;
-    return t < o_end ? t : -1;
+    if (lane == 0) t = __hip_atomic_fetch_add(ticket, Q, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __builtin_amdgcn_readfirstlane(t) + o_begin;
   };
   auto load_unit = [&](int o, u32x4 (&b)[NROW][KL]) {
     int vr = o;
@@ -714,16 +717,25 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
       for (int kc = 0; kc < KL; kc++) b[h][kc] = ldg_stream(p + kc * 64);
     }
   };
-  u32x4 buf[U][NROW][KL];
-  int uo[U];
+  // Every load is unconditional: a group at or beyond the end of the range re-reads the range's last row and its
+  // results are dropped.  (A load under a branch would turn every wait for one group into a drain of the other too.)
+  // The residual values of a group travel with its rows: lane (q * 8 + m) loads the one of output q, token m (stages
+  // without a residual read a valid dummy location instead, so that this load is unconditional too).
+  const bool has_res = st.flags & MK_F_RES;
+  const uint16_t *rbase = has_res ? (const uint16_t *)st.res + (size_t)min(lane & 7, M - 1) * st.ld_res : (const uint16_t *)st.in;
+  auto load_group = [&](int o, u32x4 (&b)[Q][NROW][KL], uint16_t &r) {
 #pragma unroll
-  for (int j = 0; j < U; j++) uo[j] = -1;
+    for (int q = 0; q < Q; q++) load_unit(max(min(o + q, o_end - 1), 0), b[q]);
+    r = rbase[has_res ? max(min(o + ((lane >> 3) & (Q - 1)), o_end - 1), 0) : 0];
+  };
+  u32x4 bufA[Q][NROW][KL], bufB[Q][NROW][KL];
+  uint16_t rA = 0, rB = 0;
+  int gA = 0, gB = 0;
   if (!ctrl) {
-#pragma unroll
-    for (int j = 0; j < U; j++) {
-      uo[j] = take();
-      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
-    }
+    gA = take();
+    load_group(gA, bufA, rA);
+    gB = take();
+    load_group(gB, bufB, rB);
   } else {
     if (c.pending && tid == 0) barrier_poll(c);
     // the token rows come from other workgroups: one acquire, then ordinary loads that share them through the die's L2
@@ -784,67 +796,70 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
   }
   __syncthreads();
   if (ctrl) {
-#pragma unroll
-    for (int j = 0; j < U; j++) {
-      uo[j] = take();
-      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
-    }
+    gA = take();
+    load_group(gA, bufA, rA);
+    gB = take();
+    load_group(gB, bufB, rB);
   }
-  const bool has_res = st.flags & MK_F_RES;
-  const uint16_t *res = (const uint16_t *)st.res;
   uint16_t *so = (uint16_t *)smem;  // [token][output - o_begin]
-  // Plain rows are reduced two slots at a time: a token-row segment read from LDS is used for both slots' weight rows
-  // (half the LDS reads per output), while the other pair of slots has its rows in flight.
-  constexpr int Q = SILU ? 1 : 2;  // slots per group ([gate ; up] pairs already share the segment)
-  static_assert(U % Q == 0, "slots are processed in groups");
-  while (true) {
-    bool any = false;
+  auto reduce_group = [&](const u32x4 (&b)[Q][NROW][KL], uint16_t r, int o) {
+    const float rf = has_res ? bf2f(r) : 0.f;
+    // the LDS addresses of the token rows are rebuilt from the lane index in every call: hoisted out of the loop they
+    // would be long-lived registers that get spilled, and a spill reload in this loop is a vector-memory wait
+    int lo = lane;
+    asm volatile("" : "+v"(lo));
+    float a[Q][NROW][MB];
+    // the segments of token m + 1 are read from LDS while token m is reduced (rows beyond M re-read row M - 1)
+    u32x4 xk[2][KL];
 #pragma unroll
-    for (int j = 0; j < U; j += Q) {
-      if (uo[j] >= 0 || uo[j + Q - 1] >= 0) {
-        any = true;
-        float a[Q][NROW][MB];
+    for (int kc = 0; kc < KL; kc++) xk[0][kc] = xs4[kc * 64 + lo];
 #pragma unroll
-        for (int m = 0; m < MB; m++) {
+    for (int m = 0; m < MB; m++) {
+#pragma unroll
+      for (int q = 0; q < Q; q++)
+#pragma unroll
+        for (int h = 0; h < NROW; h++) a[q][h][m] = 0.f;
+      if (m + 1 < MB) {
+        const int mn = min(m + 1, M - 1);
+#pragma unroll
+        for (int kc = 0; kc < KL; kc++) xk[(m + 1) & 1][kc] = xs4[mn * K8 + kc * 64 + lo];
+      }
+      __builtin_amdgcn_sched_barrier(0);
+      if (m < M) {
+#pragma unroll
+        for (int kc = 0; kc < KL; kc++) {
 #pragma unroll
           for (int q = 0; q < Q; q++)
 #pragma unroll
-            for (int h = 0; h < NROW; h++) a[q][h][m] = 0.f;
-          if (m < M) {
-#pragma unroll
-            for (int kc = 0; kc < KL; kc++) {
-              const u32x4 xk = xs4[m * K8 + kc * 64 + lane];
-#pragma unroll
-              for (int q = 0; q < Q; q++)
-#pragma unroll
-                for (int h = 0; h < NROW; h++) a[q][h][m] = dot8(buf[j + q][h][kc], xk, a[q][h][m]);
-            }
-          }
+            for (int h = 0; h < NROW; h++) a[q][h][m] = dot8(b[q][h][kc], xk[m & 1][kc], a[q][h][m]);
         }
-        int o2[Q];
-#pragma unroll
-        for (int q = 0; q < Q; q++) {
-          o2[q] = uo[j + q];
-          uo[j + q] = take();
-          if (uo[j + q] >= 0) load_unit(uo[j + q], buf[j + q]);
-        }
-#pragma unroll
-        for (int q = 0; q < Q; q++)
-          if (o2[q] >= 0) {
-#pragma unroll
-            for (int m = 0; m < MB; m++)
-              if (m < M) {
-#pragma unroll
-                for (int h = 0; h < NROW; h++) a[q][h][m] = wave_sum(a[q][h][m]);
-                float v;
-                if (SILU) v = silu_mul(a[q][0][m], a[q][NROW - 1][m]);
-                else v = has_res ? a[q][0][m] + bf2f(res[(size_t)m * st.ld_res + o2[q]]) : a[q][0][m];
-                if (lane == 0) so[m * n_loc + (o2[q] - o_begin)] = (uint16_t)f2bf(v);
-              }
-          }
       }
     }
-    if (!any) break;
+#pragma unroll
+    for (int q = 0; q < Q; q++)
+      if (o + q < o_end) {
+#pragma unroll
+        for (int m = 0; m < MB; m++)
+          if (m < M) {
+#pragma unroll
+            for (int h = 0; h < NROW; h++) a[q][h][m] = wave_sum(a[q][h][m]);
+            float v;
+            if (SILU) v = silu_mul(a[q][0][m], a[q][NROW - 1][m]);
+            else v = a[q][0][m] + lane_f32(rf, q * 8 + m);
+            if (lane == 0) so[m * n_loc + (o + q - o_begin)] = (uint16_t)f2bf(v);
+          }
+      }
+  };
+  // two groups in flight: while one is reduced the other one's rows are landing; tickets only grow, so the first
+  // group found beyond the range ends the loop
+  while (gA < o_end) {
+    reduce_group(bufA, rA, gA);
+    gA = take();
+    load_group(gA, bufA, rA);
+    if (gB >= o_end) break;
+    reduce_group(bufB, rB, gB);
+    gB = take();
+    load_group(gB, bufB, rB);
   }
   __syncthreads();
   uint16_t *dst = (uint16_t *)st.out + o_begin;
