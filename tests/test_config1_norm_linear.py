@@ -96,3 +96,62 @@ def test_norm_linear_multi_token(M, H, N, res):
     assert float(y[M:].abs().sum()) == 0.0, "rows beyond the batch must not be written"
     assert mpk.stats()["aborted"] == 0
     mpk.finalize()
+
+
+@pytest.mark.parametrize("M", [16, 50])
+def test_linear_wide_range_sweeps(M):
+    """A stage with many tiles per workgroup (LM-head-like: 70000 rows, not a multiple of 16) on the matrix-core path:
+    each workgroup works its tile range off in several sweeps, the last one ragged."""
+    import mirage as mi
+    from oracle.qwen3_ref import linear_k
+    H, N = 1024, 70000
+    g = torch.Generator().manual_seed(M)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    W = (0.02 * torch.randn(N, H, generator=g)).to(torch.bfloat16)
+    B = 64
+    meta = make_meta(1, 64, B, B, B)
+    mpk = make_mpk(meta, 64, B, B, B, 64, mode="onepass")
+    xd = torch.cat([x, torch.zeros(B - M, H, dtype=x.dtype)]).cuda()
+    tx, tW = mpk.attach_input(xd, "x"), mpk.attach_input(W.cuda(), "W")
+    ty = mpk.new_tensor((B, N), dtype=mi.bfloat16, name="y")
+    mpk.linear_layer(input=tx, weight=tW, output=ty, grid_dim=(64, 1, 1), block_dim=(128, 1, 1))
+    mpk.compile()
+    mpk.run_once(list(range(M)), [0] * M)
+    y = ty.to_torch().cpu()
+    y_ref = linear_k(x, W)
+    frac = float((y[:M].float() != y_ref.float()).float().mean())
+    ulp, mabs = bf16_ulp_diff(y[:M], y_ref, floor=1.0 / 16)
+    assert ulp <= 1.0 and frac < 0.02, f"{frac:.4f} of outputs differ, max {ulp} ulp ({mabs})"
+    assert float(y[M:].abs().sum()) == 0.0, "rows beyond the batch must not be written"
+    assert mpk.stats()["aborted"] == 0
+    mpk.finalize()
+
+
+@pytest.mark.parametrize("M", [16, 64])
+def test_linear_silu_split_k(M):
+    """A SwiGLU linear with few tiles per workgroup (2048 interleaved [gate ; up] rows, K = 4096) on the matrix-core
+    path: the reduction is split over workgroups, the gate and up partial sums are combined before the activation."""
+    import mirage as mi
+    from oracle.qwen3_ref import linear_silu_k
+    H, I, TN = 4096, 1024, 128  # a physically interleaved weight uses the reference layout [gate128 ; up128]
+    g = torch.Generator().manual_seed(100 + M)
+    x = torch.randn(M, H, generator=g).to(torch.bfloat16)
+    Wg = (0.02 * torch.randn(I, H, generator=g)).to(torch.bfloat16)
+    Wu = (0.02 * torch.randn(I, H, generator=g)).to(torch.bfloat16)
+    W = torch.cat([torch.cat([Wg[i:i + TN], Wu[i:i + TN]]) for i in range(0, I, TN)])  # [gate ; up] groups of TN rows
+    B = 64
+    meta = make_meta(1, 64, B, B, B)
+    mpk = make_mpk(meta, 64, B, B, B, 64, mode="onepass")
+    xd = torch.cat([x, torch.zeros(B - M, H, dtype=x.dtype)]).cuda()
+    tx, tW = mpk.attach_input(xd, "x"), mpk.attach_input(W.cuda(), "W")
+    ty = mpk.new_tensor((B, I), dtype=mi.bfloat16, name="y")
+    mpk.linear_silu_layer(input=tx, weight=tW, output=ty, output_stride=I, tile_n=64)
+    mpk.compile()
+    mpk.run_once(list(range(M)), [0] * M)
+    y = ty.to_torch().cpu()
+    y_ref = linear_silu_k(x, Wg, Wu)
+    frac = float((y[:M].float() != y_ref.float()).float().mean())
+    ulp, mabs = bf16_ulp_diff(y[:M], y_ref, floor=1.0 / 16)
+    assert ulp <= 1.0 and frac < 0.02, f"{frac:.4f} of outputs differ, max {ulp} ulp ({mabs})"
+    assert mpk.stats()["aborted"] == 0
+    mpk.finalize()
