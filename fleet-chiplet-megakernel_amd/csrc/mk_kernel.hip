@@ -1975,67 +1975,83 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
   }
   __syncthreads();
   int *ticket = c.sh_ticket + (c.seq & 1);
-  auto take = [&]() -> int {
+  auto take = [&](int n) -> int {  // first of the next n units of this workgroup (may lie at or beyond u_end)
     int t = 0;
-    if (lane == 0) t = __hip_atomic_fetch_add(ticket, 1, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
-    t = __builtin_amdgcn_readfirstlane(t) + u_begin;
-    return t < u_end ? t : -1;
+    if (lane == 0) t = __hip_atomic_fetch_add(ticket, n, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
+    return __builtin_amdgcn_readfirstlane(t) + u_begin;
   };
-  auto load_unit = [&](int u, u32x4 (&b)[NROW][KL]) {
+  // Every row load is unconditional: a unit at or beyond the end of the range re-reads the range's last unit and is
+  // not reduced.  (With the loads under a branch every wait for one unit's rows drained the other units' loads too.)
+  auto load_unit = [&](int u_, u32x4 (&b)[NROW][KL]) {
+    const int u = min(u_, u_end - 1);
     const int a = u / NR, j = u - a * NR;
     const size_t e = (size_t)__builtin_amdgcn_readfirstlane(L->act_e[a]);
 #pragma unroll
     for (int h = 0; h < NROW; h++) {
       const u32x4 *p = W + (e * st.n + (size_t)(j + h * NR)) * k8;
 #pragma unroll
-      for (int kc = 0; kc < KL; kc++) b[h][kc] = (kc * 64 + lane < k8) ? ldg_stream(p + kc * 64 + lane) : zero;
+      for (int kc = 0; kc < KL; kc++) b[h][kc] = ldg_stream(p + min(kc * 64 + lane, k8 - 1));  // lanes past the row re-read its last segment; their products are dropped below
     }
   };
-  u32x4 buf[R][NROW][KL];
-  int ut[R];
+  auto reduce_unit = [&](const u32x4 (&b)[NROW][KL], int u) {
+    const int a = u / NR;
+    const int p0 = __builtin_amdgcn_readfirstlane(L->pair_off[a]), p1 = __builtin_amdgcn_readfirstlane(L->pair_off[a + 1]);
+    for (int p = p0; p < p1; p++) {  // LDS only in here
+      const u32x4 *x = xs4 + (p - p_base) * k8;
+      float acc[NROW];
 #pragma unroll
-  for (int jj = 0; jj < R; jj++) {
-    ut[jj] = take();
-    if (ut[jj] >= 0) load_unit(ut[jj], buf[jj]);
-  }
-  while (true) {
-    bool any = false;
+      for (int h = 0; h < NROW; h++) acc[h] = 0.f;
 #pragma unroll
-    for (int jj = 0; jj < R; jj++) {
-      if (ut[jj] >= 0) {
-        any = true;
-        const int u = ut[jj], a = u / NR;
-        const int p0 = __builtin_amdgcn_readfirstlane(L->pair_off[a]), p1 = __builtin_amdgcn_readfirstlane(L->pair_off[a + 1]);
-        for (int p = p0; p < p1; p++) {  // LDS only in here
-          const u32x4 *x = xs4 + (p - p_base) * k8;
-          float acc[NROW];
+      for (int kc = 0; kc < KL; kc++) {
+        const u32x4 xv = (kc * 64 + lane < k8) ? x[kc * 64 + lane] : zero;
 #pragma unroll
-          for (int h = 0; h < NROW; h++) acc[h] = 0.f;
+        for (int h = 0; h < NROW; h++) acc[h] = dot8(b[h][kc], xv, acc[h]);
+      }
 #pragma unroll
-          for (int kc = 0; kc < KL; kc++) {
-            const u32x4 xv = (kc * 64 + lane < k8) ? x[kc * 64 + lane] : zero;
-#pragma unroll
-            for (int h = 0; h < NROW; h++) acc[h] = dot8(buf[jj][h][kc], xv, acc[h]);
-          }
-#pragma unroll
-          for (int h = 0; h < NROW; h++) acc[h] = wave_sum(acc[h]);
-          uint16_t *t0 = so + (size_t)(p - p0) * nu + (u - u_begin);
-          if (SILU) {
-            const uint32_t g = f2bf(acc[0]), up = f2bf(acc[NROW - 1]);
-            if (lane == 0) {
-              t0[0] = (uint16_t)g;
-              t0[(size_t)maxp * nu] = (uint16_t)up;
-              t0[(size_t)2 * maxp * nu] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
-            }
-          } else if (lane == 0) {
-            t0[0] = (uint16_t)f2bf(acc[0]);
-          }
+      for (int h = 0; h < NROW; h++) acc[h] = wave_sum(acc[h]);
+      uint16_t *t0 = so + (size_t)(p - p0) * nu + (u - u_begin);
+      if (SILU) {
+        const uint32_t g = f2bf(acc[0]), up = f2bf(acc[NROW - 1]);
+        if (lane == 0) {
+          t0[0] = (uint16_t)g;
+          t0[(size_t)maxp * nu] = (uint16_t)up;
+          t0[(size_t)2 * maxp * nu] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)g), bf2f((uint16_t)up)));
         }
-        ut[jj] = take();
-        if (ut[jj] >= 0) load_unit(ut[jj], buf[jj]);
+      } else if (lane == 0) {
+        t0[0] = (uint16_t)f2bf(acc[0]);
       }
     }
-    if (!any) break;
+  };
+  // two groups of units in flight: while one is reduced the other one's rows are landing; tickets only grow, so the
+  // first group found beyond the range ends the loop
+  constexpr int QA = (R + 1) / 2, QB = R / 2;
+  if (nu > 0) {
+    u32x4 bufA[QA][NROW][KL], bufB[QB > 0 ? QB : 1][NROW][KL];
+    int gA = take(QA), gB = u_end;
+#pragma unroll
+    for (int q = 0; q < QA; q++) load_unit(gA + q, bufA[q]);
+    if (QB > 0) {
+      gB = take(QB);
+#pragma unroll
+      for (int q = 0; q < QB; q++) load_unit(gB + q, bufB[q]);
+    }
+    while (gA < u_end) {
+#pragma unroll
+      for (int q = 0; q < QA; q++)
+        if (gA + q < u_end) reduce_unit(bufA[q], gA + q);
+      gA = take(QA);
+#pragma unroll
+      for (int q = 0; q < QA; q++) load_unit(gA + q, bufA[q]);
+      if (QB > 0) {
+        if (gB >= u_end) break;
+#pragma unroll
+        for (int q = 0; q < QB; q++)
+          if (gB + q < u_end) reduce_unit(bufB[q], gB + q);
+        gB = take(QB);
+#pragma unroll
+        for (int q = 0; q < QB; q++) load_unit(gB + q, bufB[q]);
+      }
+    }
   }
   __syncthreads();
   // write the tile out: consecutive threads take consecutive rows of one (token, slot)
