@@ -680,8 +680,9 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
 // Few-token linear (2..MB tokens): the single-token structure with the token rows in LDS.  Every weight row is still
 // read once and dotted against all token rows (v_dot2, fp32); up to 8 tokens this stays under the streaming time, so
 // small batches cost little more than one token, where the matrix-core path (16-row tiles, one tile per workgroup
-// on the narrow stages) is bound by latency.  The rows were normalised by the preceding NORM stage when the stage
-// carries MK_F_NORM.  Outputs are collected in LDS [token][output] and written through.
+// on the narrow stages) is bound by latency.  A stage that carries MK_F_NORM normalises the rows itself while staging
+// them (the standalone NORM stage in front is skipped for these batch sizes).  Outputs are collected in LDS
+// [token][output] and written through.
 template <int KL, int R, bool SILU, int MB>
 __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, char *smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
