@@ -670,13 +670,6 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
 }
 
 
-// Multi-token linear on the matrix cores: out[m, n] = bf16(sum_k x[m,k] * W[n,k] (+ res[m,n])) for 2..64 token rows,
-// optional SwiGLU epilogue.  A workgroup owns a contiguous range of 16-row weight tiles and ALL token rows, so every
-// weight byte is still read from HBM exactly once; its four wavefronts split K and are reduced through LDS.  One
-// v_mfma_f32_16x16x32_bf16 consumes a 16(n) x 32(k) weight fragment (one 16-byte load per lane, 64 contiguous bytes per
-// weight row) against a 32(k) x 16(m) activation fragment that comes from the L2-resident activation rows.
-// Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
-// (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
 // Few-token linear (2..MB tokens): the single-token structure with the token rows in LDS.  Every weight row is still
 // read once and dotted against all token rows (v_dot2, fp32); up to 8 tokens this stays under the streaming time, so
 // small batches cost little more than one token, where the matrix-core path (16-row tiles, one tile per workgroup
@@ -1162,6 +1155,13 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
 #ifndef MK_TUNE_NBN
 #define MK_TUNE_NBN 4
 #endif
+// Multi-token linear on the matrix cores, K split inside the workgroup: out[m, n] = bf16(sum_k x[m,k] * W[n,k] (+ res[m,n])) for 2..64 token rows,
+// optional SwiGLU epilogue.  A workgroup owns a contiguous range of 16-row weight tiles and ALL token rows, so every
+// weight byte is still read from HBM exactly once; its four wavefronts split K and are reduced through LDS.  One
+// v_mfma_f32_16x16x32_bf16 consumes a 16(n) x 32(k) weight fragment (one 16-byte load per lane, 64 contiguous bytes per
+// weight row) against a 32(k) x 16(m) activation fragment that comes from the L2-resident activation rows.
+// Reference tasks: linear_kernel_ck tile tiers (tasks/mi300/linear_ck_mi300.cuh:306-332), gang_linear_kernel
+// (tasks/mi300/gang_linear_mi300.cuh:47-108), gang_linear_silu_kernel (:359-576).
 // TG = weight tiles per K sweep, NB = 64-wide k steps in flight per wavefront.  Two shapes are instantiated: wide
 // stages (several tiles per workgroup) run <6, 2>; narrow ones (one or two weight tiles per workgroup, e.g. N = 4096
 // on 256 workgroups) spend the registers on depth instead: <2, MK_TUNE_NBN>.
