@@ -36,6 +36,9 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_R8N
 #define MK_TUNE_R8N 4
 #endif
+#ifndef MK_TUNE_NL
+#define MK_TUNE_NL 2
+#endif
 #ifndef MK_TUNE_R24
 #define MK_TUNE_R24 2
 #endif
@@ -527,12 +530,39 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   };
   u32x4 buf[U][NROW][KL];
   int uo[U];
+  // LDS side of the prefetch: NL further outputs per worker wavefront whose rows are parked in the LDS window above
+  // MK_MOE_OFFSET while the barrier is awaited (the registers alone hold about 3.5 us of streaming, the barrier and the
+  // staging of the input row take longer).  They are reduced from LDS right after the barrier.
+  constexpr int NLFIT = 32 / (KL * NROW);  // rows of KL KB that fit a wavefront's 32 KB share of the window
+  constexpr int NL = NLFIT < MK_TUNE_NL ? NLFIT : MK_TUNE_NL;
+  u32x4 *lrows = (u32x4 *)(smem + MK_MOE_OFFSET) + (size_t)(wave > 0 ? wave - 1 : 0) * (NL > 0 ? NL : 1) * NROW * K8;
+  int lo_[NL > 0 ? NL : 1];
   if (!ctrl) {
-    // weights do not depend on the previous stage: the first U outputs' rows are requested before its barrier completes
+    // weights do not depend on the previous stage: the first outputs' rows are requested before its barrier completes
+    if (NL > 0) {
+      u32x4 lb[NL > 0 ? NL : 1][NROW][KL];
 #pragma unroll
-    for (int j = 0; j < U; j++) {
-      uo[j] = take();
-      if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+      for (int i = 0; i < NL; i++) {
+        lo_[i] = take();
+        load_unit(lo_[i] >= 0 ? lo_[i] : min(o_begin, n_out - 1), lb[i]);  // unconditional (an exhausted ticket re-reads a valid row)
+      }
+#pragma unroll
+      for (int j = 0; j < U; j++) {
+        uo[j] = take();
+        if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+      }
+#pragma unroll
+      for (int i = 0; i < NL; i++)
+#pragma unroll
+        for (int h = 0; h < NROW; h++)
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) lrows[((i * NROW + h) * KL + kc) * 64 + lane] = lb[i][h][kc];
+    } else {
+#pragma unroll
+      for (int j = 0; j < U; j++) {
+        uo[j] = take();
+        if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+      }
     }
   } else {
     u32x4 nwv[KL];
@@ -571,6 +601,25 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   if (KL <= 8) {
 #pragma unroll
     for (int kc = 0; kc < (KL <= 8 ? KL : 1); kc++) xr[kc] = xs4[kc * 64 + lane];
+  }
+  if (NL > 0 && !ctrl) {  // the parked rows first: no memory traffic, the register slots keep landing meanwhile
+#pragma unroll
+    for (int i = 0; i < NL; i++) {
+      if (lo_[i] >= 0) {
+        float a[NROW];
+#pragma unroll
+        for (int h = 0; h < NROW; h++) {
+          a[h] = 0.f;
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) a[h] = dot8(lrows[((i * NROW + h) * KL + kc) * 64 + lane], KL <= 8 ? xr[KL <= 8 ? kc : 0] : xs4[kc * 64 + lane], a[h]);
+        }
+#pragma unroll
+        for (int h = 0; h < NROW; h++) a[h] = wave_sum(a[h]);
+        const float r = has_res ? bf2f(ldc_u16(res + lo_[i])) : 0.f;
+        const float v = SILU ? silu_mul(a[0], a[NROW - 1]) : a[0] + r;
+        if (lane == 0) so[lo_[i] - o_begin] = (uint16_t)f2bf(v);
+      }
+    }
   }
   while (true) {
     bool any = false;
