@@ -541,15 +541,16 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
     // weights do not depend on the previous stage: the first outputs' rows are requested before its barrier completes
     if (NL > 0) {
       u32x4 lb[NL > 0 ? NL : 1][NROW][KL];
-#pragma unroll
-      for (int i = 0; i < NL; i++) {
-        lo_[i] = take();
-        load_unit(lo_[i] >= 0 ? lo_[i] : min(o_begin, n_out - 1), lb[i]);  // unconditional (an exhausted ticket re-reads a valid row)
-      }
+      // the register slots draw first, so a short range is held in registers and only the surplus is parked
 #pragma unroll
       for (int j = 0; j < U; j++) {
         uo[j] = take();
         if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+      }
+#pragma unroll
+      for (int i = 0; i < NL; i++) {
+        lo_[i] = take();
+        load_unit(lo_[i] >= 0 ? lo_[i] : min(o_begin, n_out - 1), lb[i]);  // unconditional (an exhausted ticket re-reads a valid row)
       }
 #pragma unroll
       for (int i = 0; i < NL; i++)
