@@ -1,4 +1,4 @@
-"""BASELINE config 1: RMSNorm(4096) -> linear 4096x4096, BS=1 bf16, as a two-task graph through the C ABI.
+"""Headline configuration 1: RMSNorm(4096) -> linear 4096x4096, BS=1 bf16, as a two-task graph through the C ABI.
 
 Closest reference checks (CUDA-only, formula only): tests/runtime_python/test_norm_linear.py:13-19."""
 import pytest

@@ -1,4 +1,4 @@
-"""BASELINE config 2 (one Qwen3-8B-shaped decoder layer, 512 cached positions, one new token, BS=1) and smaller /
+"""Headline configuration 2 (one Qwen3-8B-shaped decoder layer, 512 cached positions, one new token, BS=1) and smaller /
 multi-token variants of the same layer, GPU vs the kernel-order CPU oracle, through the PersistentKernel API."""
 import pytest
 import torch
