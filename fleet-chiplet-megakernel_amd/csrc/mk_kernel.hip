@@ -36,6 +36,9 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_R8N
 #define MK_TUNE_R8N 4
 #endif
+#ifndef MK_TUNE_MOE_R2
+#define MK_TUNE_MOE_R2 12
+#endif
 #ifndef MK_TUNE_NL
 #define MK_TUNE_NL 2
 #endif
@@ -2147,7 +2150,7 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
     }
     if (st.k <= 1024) {
       if (silu) stage_moe_linear_multi<2, 4, true>(st, c, M, smem);
-      else stage_moe_linear_multi<2, 6, false>(st, c, M, smem);
+      else stage_moe_linear_multi<2, MK_TUNE_MOE_R2, false>(st, c, M, smem);
     } else if (st.k <= 2048) {
       if (silu) stage_moe_linear_multi<4, 3, true>(st, c, M, smem);
       else stage_moe_linear_multi<4, 4, false>(st, c, M, smem);
