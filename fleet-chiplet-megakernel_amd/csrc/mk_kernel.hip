@@ -109,6 +109,45 @@ __device__ __forceinline__ float wave_sum(float v) {
   v = group16_sum(v);
   return (lane_f32(v, 0) + lane_f32(v, 16)) + (lane_f32(v, 32) + lane_f32(v, 48));
 }
+// Transposing wavefront reduction: every lane holds partial sums of NV values (NV a power of two <= 16); on return lane
+// l holds the wavefront total of value l & (NV - 1).  Stage b pairs the values up and exchanges one of each pair with
+// the lane whose bit b differs (one DPP move per pair), so 16 values cost about 50 instructions instead of 16 full
+// reductions; the four 16-lane rows are combined with two cross-row permutes at the end.
+template <int NV>
+__device__ __forceinline__ float transpose_sum(float (&v)[NV], int lane) {
+  static_assert(NV == 1 || NV == 2 || NV == 4 || NV == 8 || NV == 16, "power of two");
+  if constexpr (NV >= 2) {
+    const bool b = lane & 1;
+#pragma unroll
+    for (int j = 0; j < NV / 2; j++) v[j] = (b ? v[2 * j + 1] : v[2 * j]) + dpp_f32<0xB1>(b ? v[2 * j] : v[2 * j + 1]);  // quad_perm [1,0,3,2]
+  }
+  if constexpr (NV >= 4) {
+    const bool b = lane & 2;
+#pragma unroll
+    for (int j = 0; j < NV / 4; j++) v[j] = (b ? v[2 * j + 1] : v[2 * j]) + dpp_f32<0x4E>(b ? v[2 * j] : v[2 * j + 1]);  // quad_perm [2,3,0,1]
+  }
+  if constexpr (NV >= 8) {
+    const bool b = lane & 4;
+#pragma unroll
+    for (int j = 0; j < NV / 8; j++) {
+      const float give = b ? v[2 * j] : v[2 * j + 1];
+      const float up = dpp_f32<0x104>(give), down = dpp_f32<0x114>(give);  // row_shl:4 (from lane + 4), row_shr:4 (from lane - 4)
+      v[j] = (b ? v[2 * j + 1] : v[2 * j]) + (b ? down : up);
+    }
+  }
+  if constexpr (NV >= 16) {
+    const bool b = lane & 8;
+    v[0] = (b ? v[1] : v[0]) + dpp_f32<0x128>(b ? v[0] : v[1]);  // row_ror:8
+  }
+  float r = v[0];
+  if (NV < 16) r += dpp_f32<0x128>(r);
+  if (NV < 8) r += dpp_f32<0x124>(r);
+  if (NV < 4) r += dpp_f32<0x122>(r);
+  if (NV < 2) r += dpp_f32<0x121>(r);
+  r += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, r)));
+  r += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, r)));
+  return r;
+}
 __device__ __forceinline__ unsigned xcc_id() {
   // HW_REG_XCC_ID (id 20), bits [3:0]
   return __builtin_amdgcn_s_getreg((3 << 11) | (0 << 6) | 20) & 7u;  // MI355X: 8 XCDs
@@ -766,14 +805,14 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
   };
   // Every load is unconditional: a group at or beyond the end of the range re-reads the range's last row and its
   // results are dropped.  (A load under a branch would turn every wait for one group into a drain of the other too.)
-  // The residual values of a group travel with its rows: lane (q * 8 + m) loads the one of output q, token m (stages
+  // The residual values of a group travel with its rows: lane (q * MB + m) loads the one of output q, token m (stages
   // without a residual read a valid dummy location instead, so that this load is unconditional too).
   const bool has_res = st.flags & MK_F_RES;
-  const uint16_t *rbase = has_res ? (const uint16_t *)st.res + (size_t)min(lane & 7, M - 1) * st.ld_res : (const uint16_t *)st.in;
+  const uint16_t *rbase = has_res ? (const uint16_t *)st.res + (size_t)min(lane & (MB - 1), M - 1) * st.ld_res : (const uint16_t *)st.in;
   auto load_group = [&](int o, u32x4 (&b)[Q][NROW][KL], uint16_t &r) {
 #pragma unroll
     for (int q = 0; q < Q; q++) load_unit(max(min(o + q, o_end - 1), 0), b[q]);
-    r = rbase[has_res ? max(min(o + ((lane >> 3) & (Q - 1)), o_end - 1), 0) : 0];
+    r = rbase[has_res ? max(min(o + ((lane / MB) & (Q - 1)), o_end - 1), 0) : 0];
   };
   u32x4 bufA[Q][NROW][KL], bufB[Q][NROW][KL];
   uint16_t rA = 0, rB = 0;
@@ -882,20 +921,21 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
         }
       }
     }
+    // all Q * NROW * MB sums are reduced together; lane q * MB + m (plain) / h * MB + m ([gate ; up]) gets the total
+    constexpr int NV = Q * NROW * MB;
+    float vv[NV];
 #pragma unroll
     for (int q = 0; q < Q; q++)
-      if (o + q < o_end) {
 #pragma unroll
-        for (int m = 0; m < MB; m++)
-          if (m < M) {
+      for (int h = 0; h < NROW; h++)
 #pragma unroll
-            for (int h = 0; h < NROW; h++) a[q][h][m] = wave_sum(a[q][h][m]);
-            float v;
-            if (SILU) v = silu_mul(a[q][0][m], a[q][NROW - 1][m]);
-            else v = a[q][0][m] + lane_f32(rf, q * 8 + m);
-            if (lane == 0) so[m * n_loc + (o + q - o_begin)] = (uint16_t)f2bf(v);
-          }
-      }
+        for (int m = 0; m < MB; m++) vv[(q * NROW + h) * MB + m] = a[q][h][m];
+    const float tot = transpose_sum<NV>(vv, lane);
+    const int m = lane & (MB - 1), q = SILU ? 0 : lane / MB;
+    float v;
+    if (SILU) v = silu_mul(tot, dpp_f32<0x100 + MB>(tot));  // row_shl:MB: the up sum sits MB lanes above the gate sum
+    else v = tot + rf;
+    if (lane < Q * MB && m < M && o + q < o_end) so[m * n_loc + (o + q - o_begin)] = (uint16_t)f2bf(v);
   };
   // two groups in flight: while one is reduced the other one's rows are landing; tickets only grow, so the first
   // group found beyond the range ends the loop
