@@ -1111,24 +1111,25 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
     for (int t = 0; t < TW; t++)
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
-    // Two copies of the step loop, for wavefronts with and without tiles: a branch around the weight loads inside one
-    // copy would spoil its wait counts.  Both execute the same barriers.
-    auto pipeline = [&](auto htc) {
+    // Copies of the step loop for wavefronts with / without tiles and with / without a token tile to stage: a branch
+    // around loads inside one copy would spoil its wait counts.  All copies execute the same barriers.
+    auto pipeline = [&](auto htc, auto xlc) {
       constexpr bool HT = decltype(htc)::value;
+      constexpr bool XL = decltype(xlc)::value;  // this wavefront stages a token tile (wavefront index < MT)
       __syncthreads();  // the previous sweep has finished with the LDS buffers
 #pragma unroll
       for (int j = 0; j < NB; j++) {
         if (HT) w_load(j, a[j]);
-        x_load(j, xq[j]);
+        if (XL) x_load(j, xq[j]);
       }
-      x_store(0, xq[0]);
+      if (XL) x_store(0, xq[0]);
       __syncthreads();
       auto block = [&](int s0, auto refill) {
         constexpr bool REFILL = decltype(refill)::value;
 #pragma unroll
         for (int j = 0; j < NB; j++) {
           const int step = s0 + j;
-          if (REFILL || j + 1 < NB) x_store((step + 1) & 1, xq[(j + 1) % NB]);  // that buffer was last read before the previous barrier
+          if (XL && (REFILL || j + 1 < NB)) x_store((step + 1) & 1, xq[(j + 1) % NB]);  // that buffer was last read before the previous barrier
           if (HT) {
             const u32x4 *xb = xl + (step & 1) * MT * 128;
             u32x4 b[2][MT];
@@ -1147,7 +1148,7 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
           }
           if (REFILL) {
             if (HT) w_load(step + NB, a[j]);
-            x_load(step + NB, xq[j]);
+            if (XL) x_load(step + NB, xq[j]);
           }
           __syncthreads();
         }
@@ -1156,8 +1157,14 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
       for (; s0 + NB < nsteps; s0 += NB) block(s0, std::true_type{});
       block(s0, std::false_type{});
     };
-    if (has_tile) pipeline(std::true_type{});
-    else pipeline(std::false_type{});
+    const bool stages_x = wave < MT;
+    if (MT == MK_WAVES || stages_x) {
+      if (has_tile) pipeline(std::true_type{}, std::true_type{});
+      else pipeline(std::false_type{}, std::true_type{});
+    } else {
+      if (has_tile) pipeline(std::true_type{}, std::false_type{});
+      else pipeline(std::false_type{}, std::false_type{});
+    }
 
     // ---- combine the S slices (a split range is a single sweep, so slots are indexed by wavefront and tile only)
     if (S > 1) {
