@@ -172,3 +172,13 @@ def test_full_width_layer_prefill_chunk_mpk_mode():
     cfg = Qwen3Config(num_layers=1)
     res = _run_layer(cfg, 40, 8, "mpk", seed=9)
     _check(res, cfg, 40, 8)
+
+
+@pytest.mark.parametrize("n_new", [2, 4, 7])
+def test_full_width_layer_few_tokens_fleet_mode(n_new):
+    """Full-width layer with 2..8 new tokens in the gang configuration: the few-token linears (token rows in LDS, fused
+    RMSNorm, fused SwiGLU, residual travelling with the rows) for every token-count instantiation."""
+    from oracle.qwen3_ref import Qwen3Config
+    cfg = Qwen3Config(num_layers=1)
+    res = _run_layer(cfg, 24, n_new, "fleet", seed=40 + n_new)
+    _check(res, cfg, 24, n_new)
