@@ -2123,6 +2123,53 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
       }
     }
   };
+  // The units of a group are consecutive rows, nearly always of one expert: they are then reduced jointly per (token,
+  // slot) pair -- the pair's input segments are read from LDS once for all of them and their sums are reduced together
+  // (transposing reduction, lane q * NROW + h gets unit q's sum h).  A group that straddles two experts takes the
+  // unit-by-unit form.
+  auto reduce_group = [&](auto &bufs, int g, auto nqc) {
+    constexpr int NQ = decltype(nqc)::value;
+    constexpr int NVAL = NQ * NROW;
+    constexpr int NV = NVAL <= 1 ? 1 : (NVAL <= 2 ? 2 : (NVAL <= 4 ? 4 : (NVAL <= 8 ? 8 : 16)));
+    static_assert(NVAL <= 16, "group size");
+    const int nvalid = min(NQ, u_end - g);
+    const int a = g / NR;
+    if ((g + nvalid - 1) / NR != a) {
+#pragma unroll
+      for (int q = 0; q < NQ; q++)
+        if (q < nvalid) reduce_unit(bufs[q], g + q);
+      return;
+    }
+    const int p0 = __builtin_amdgcn_readfirstlane(L->pair_off[a]), p1 = __builtin_amdgcn_readfirstlane(L->pair_off[a + 1]);
+    for (int p = p0; p < p1; p++) {  // LDS only in here
+      const u32x4 *x = xs4 + (p - p_base) * k8;
+      float vv[NV];
+#pragma unroll
+      for (int i = 0; i < NV; i++) vv[i] = 0.f;
+#pragma unroll
+      for (int kc = 0; kc < KL; kc++) {
+        const u32x4 xv = (kc * 64 + lane < k8) ? x[kc * 64 + lane] : zero;
+#pragma unroll
+        for (int q = 0; q < NQ; q++)
+#pragma unroll
+          for (int h = 0; h < NROW; h++) vv[q * NROW + h] = dot8(bufs[q][h][kc], xv, vv[q * NROW + h]);
+      }
+      const float tot = transpose_sum<NV>(vv, lane);
+      const int q = lane / NROW;
+      uint16_t *t0 = so + (size_t)(p - p0) * nu + (g + q - u_begin);
+      if (SILU) {
+        const float upv = dpp_f32<0x101>(tot);  // row_shl:1: the up sum sits one lane above the gate sum
+        const uint32_t gb = f2bf(tot), ub = f2bf(upv);
+        if (lane < NVAL && (lane & 1) == 0 && q < nvalid) {
+          t0[0] = (uint16_t)gb;
+          t0[(size_t)maxp * nu] = (uint16_t)ub;
+          t0[(size_t)2 * maxp * nu] = (uint16_t)f2bf(silu_mul(bf2f((uint16_t)gb), bf2f((uint16_t)ub)));
+        }
+      } else if (lane < NVAL && q < nvalid) {
+        t0[0] = (uint16_t)f2bf(tot);
+      }
+    }
+  };
   // two groups of units in flight: while one is reduced the other one's rows are landing; tickets only grow, so the
   // first group found beyond the range ends the loop
   constexpr int QA = (R + 1) / 2, QB = R / 2;
@@ -2137,17 +2184,13 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
       for (int q = 0; q < QB; q++) load_unit(gB + q, bufB[q]);
     }
     while (gA < u_end) {
-#pragma unroll
-      for (int q = 0; q < QA; q++)
-        if (gA + q < u_end) reduce_unit(bufA[q], gA + q);
+      reduce_group(bufA, gA, std::integral_constant<int, QA>{});
       gA = take(QA);
 #pragma unroll
       for (int q = 0; q < QA; q++) load_unit(gA + q, bufA[q]);
       if (QB > 0) {
         if (gB >= u_end) break;
-#pragma unroll
-        for (int q = 0; q < QB; q++)
-          if (gB + q < u_end) reduce_unit(bufB[q], gB + q);
+        reduce_group(bufB, gB, std::integral_constant<int, (QB > 0 ? QB : 1)>{});
         gB = take(QB);
 #pragma unroll
         for (int q = 0; q < QB; q++) load_unit(gB + q, bufB[q]);
