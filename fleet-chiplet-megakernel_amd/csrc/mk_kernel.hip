@@ -36,8 +36,11 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_R8N
 #define MK_TUNE_R8N 4
 #endif
+#ifndef MK_TUNE_MOE_R13
+#define MK_TUNE_MOE_R13 4
+#endif
 #ifndef MK_TUNE_MOE_R2
-#define MK_TUNE_MOE_R2 12
+#define MK_TUNE_MOE_R2 16
 #endif
 #ifndef MK_TUNE_NL
 #define MK_TUNE_NL 2
@@ -2242,7 +2245,7 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
       if (silu) stage_moe_linear_multi<2, 4, true>(st, c, M, smem);
       else stage_moe_linear_multi<2, MK_TUNE_MOE_R2, false>(st, c, M, smem);
     } else if (st.k <= 2048) {
-      if (silu) stage_moe_linear_multi<4, 3, true>(st, c, M, smem);
+      if (silu) stage_moe_linear_multi<4, MK_TUNE_MOE_R13, true>(st, c, M, smem);
       else stage_moe_linear_multi<4, 4, false>(st, c, M, smem);
     } else {
       if (silu) stage_moe_linear_multi<8, 1, true>(st, c, M, smem);
