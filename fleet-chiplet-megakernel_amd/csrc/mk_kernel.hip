@@ -431,6 +431,46 @@ __device__ __forceinline__ float block_sum(float v, float *red) {
 // single-token iterations fuse the norm into the consuming linear).  y = bf16((x * r) * w) with
 // r = rsqrt(mean(x^2) + eps) in fp32.  Reference task: tasks/mi300/rmsnorm_mi300.cuh:37-188.
 __device__ __forceinline__ void stage_norm(CStage &st, Ctx &c, int M, char *smem) {
+  const int k8 = st.k / 8;
+  if ((st.k & 7) == 0 && k8 <= 6 * MK_THREADS && (st.ld_in & 7) == 0 && (st.ld_out & 7) == 0) {
+    // Row per workgroup, up to six 16-byte segments per thread: the norm weights are requested before the barrier is
+    // awaited, the row is read with device-scope loads and written through, so the arrival needs no L2 write-back.
+    constexpr int NS = 6;
+    const int tid = threadIdx.x;
+    float *red = (float *)smem;
+    const u32x4 *w4 = (const u32x4 *)st.norm_w;
+    u32x4 g[NS], v[NS];
+#pragma unroll
+    for (int j = 0; j < NS; j++)
+      if (j * MK_THREADS < k8) g[j] = w4[min(tid + j * MK_THREADS, k8 - 1)];
+    barrier_wait(c);
+    for (int t = c.vid; t < M; t += c.G) {
+      const u32x4 *x = (const u32x4 *)((const uint16_t *)st.in + (size_t)t * st.ld_in);
+      u32x4 *y = (u32x4 *)((uint16_t *)st.out + (size_t)t * st.ld_out);
+      float ss = 0.f;
+#pragma unroll
+      for (int j = 0; j < NS; j++)
+        if (j * MK_THREADS < k8) {
+          const bool ok = tid + j * MK_THREADS < k8;
+          v[j] = ldc_16B(x + min(tid + j * MK_THREADS, k8 - 1));
+#pragma unroll
+          for (int e = 0; e < 4; e++) ss += ok ? bf_lo(v[j][e]) * bf_lo(v[j][e]) + bf_hi(v[j][e]) * bf_hi(v[j][e]) : 0.f;
+        }
+      ss = block_sum(ss, red);
+      const float r = rsqrtf(ss / (float)st.k + st.eps);
+#pragma unroll
+      for (int j = 0; j < NS; j++)
+        if (tid + j * MK_THREADS < k8) {
+          u32x4 o;
+#pragma unroll
+          for (int e = 0; e < 4; e++) o[e] = pack2((bf_lo(v[j][e]) * r) * bf_lo(g[j][e]), (bf_hi(v[j][e]) * r) * bf_hi(g[j][e]));
+          stc_16B(y + tid + j * MK_THREADS, o);
+        }
+      __syncthreads();
+    }
+    c.wrote_through = true;
+    return;
+  }
   barrier_wait(c);
   float *red = (float *)smem;
   uint32_t *xs = (uint32_t *)(smem + 1024);
