@@ -187,6 +187,18 @@ __device__ __forceinline__ void stc_16B(u32x4 *p, u32x4 v) {
   __hip_atomic_store(q, (unsigned long long)v.x | ((unsigned long long)v.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   __hip_atomic_store(q + 1, (unsigned long long)v.z | ((unsigned long long)v.w << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+// four consecutive bf16 outputs of one token row, written through: one 8-byte store when the run is whole and aligned
+__device__ __forceinline__ void stc_bf16x4(uint16_t *row, int n0, int n_out, const float (&r)[4]) {
+  uint16_t *p = row + n0;
+  if (n0 + 3 < n_out && (((unsigned long long)p) & 7) == 0) {
+    const unsigned long long v = (unsigned long long)pack2(r[0], r[1]) | ((unsigned long long)pack2(r[2], r[3]) << 32);
+    __hip_atomic_store((__attribute__((address_space(1))) unsigned long long *)(unsigned long long)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+  } else {
+#pragma unroll
+    for (int i = 0; i < 4; i++)
+      if (n0 + i < n_out) stc_u16(p + i, (uint16_t)f2bf(r[i]));
+  }
+}
 __device__ __forceinline__ uint16_t ldc_u16(const uint16_t *p) {
   const uintptr_t a = (uintptr_t)p;
   const uint32_t w = ldc_u32((const void *)(a & ~(uintptr_t)3));
@@ -1084,6 +1096,7 @@ __device__ __forceinline__ TilePlan linear_tiles_plan(CStage &st, const Ctx &c) 
 template <int MT>
 __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, const MkRuntime &rt, int M, const TilePlan plan, char *smem) {
   barrier_wait(c);
+  c.wrote_through = true;  // partial tiles and outputs are all written through: no L2 write-back at this stage's arrival
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   __syncthreads();
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
@@ -1264,17 +1277,17 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
         if (m < M) {
           uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
           const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
+          float rr[4];
 #pragma unroll
           for (int i = 0; i < 4; i++) {
             const int n = otile * 16 + lg * 4 + i;
-            if (n < n_out) {
-              float r;
-              if (silu) r = TW >= 2 ? silu_mul(acc[(2 * u) % TW][mt][i], acc[(2 * u + 1) % TW][mt][i]) : 0.f;
-              else r = acc[u][mt][i];
-              if (st.flags & MK_F_RES) r += bf2f(rrow[n]);
-              orow[n] = (uint16_t)f2bf(r);
-            }
+            float r;
+            if (silu) r = TW >= 2 ? silu_mul(acc[(2 * u) % TW][mt][i], acc[(2 * u + 1) % TW][mt][i]) : 0.f;
+            else r = acc[u][mt][i];
+            if ((st.flags & MK_F_RES) && n < n_out) r += bf2f(rrow[n]);
+            rr[i] = r;
           }
+          stc_bf16x4(orow, otile * 16 + lg * 4, n_out, rr);
         }
       }
     }
@@ -1311,6 +1324,7 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
 template <int MT, int TG, int NB>
 __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, char *smem) {
   barrier_wait(c);
+  c.wrote_through = true;  // outputs are written through: no L2 write-back at this stage's arrival
   // activations were produced by other workgroups: invalidate this CU's L1 once, then use cached loads so the rows
   // are shared through the XCD's L2
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
@@ -1439,15 +1453,15 @@ __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, cha
       if (m < M) {
         uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
         const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
+        float rr[4];
 #pragma unroll
         for (int i = 0; i < 4; i++) {
           const int n = n0 + i;
-          if (n < n_out) {
-            float r = silu ? silu_mul(v[i], v2[i]) : v[i];
-            if (st.flags & MK_F_RES) r += bf2f(rrow[n]);
-            orow[n] = (uint16_t)f2bf(r);
-          }
+          float r = silu ? silu_mul(v[i], v2[i]) : v[i];
+          if ((st.flags & MK_F_RES) && n < n_out) r += bf2f(rrow[n]);
+          rr[i] = r;
         }
+        stc_bf16x4(orow, n0, n_out, rr);
       }
     }
   }
