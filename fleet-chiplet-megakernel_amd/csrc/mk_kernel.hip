@@ -1597,11 +1597,12 @@ __device__ __forceinline__ void stage_moe_topk(CStage &st, Ctx &c, int M) {
     float w;
     int e;
     moe_route_wave((const uint16_t *)st.moe_logits + (size_t)t * st.ld_logits, E, st.topk, lane, sel, w, e);
-    if (lane < st.topk) st.moe_topk_w[(size_t)t * st.ld_topk_w + lane] = w;
+    if (lane < st.topk) __hip_atomic_store(st.moe_topk_w + (size_t)t * st.ld_topk_w + lane, w, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 #pragma unroll
     for (int j = 0; j < 4; j++)
-      if (j * 64 + lane < E) st.moe_routing[(size_t)(j * 64 + lane) * st.ld_routing + t] = sel[j];
+      if (j * 64 + lane < E) __hip_atomic_store(st.moe_routing + (size_t)(j * 64 + lane) * st.ld_routing + t, sel[j], __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
   }
+  c.wrote_through = true;  // written through: no L2 write-back at this stage's arrival
 }
 
 // Build the active-expert list and the (token, slot) pairs of every active expert from the routing table.
@@ -2263,9 +2264,10 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
     const int p = L->pair_off[a] + pi;
     if (p >= L->pair_off[a + 1]) continue;
     const int ts = L->pair_ts[p], tok = ts & 255, slot = ts >> 8;
-    if (SILU && arr == 2) out2[(size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j] = so[i];
-    else out[(size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot + j + (arr == 1 ? NR : 0)] = so[i];
+    if (SILU && arr == 2) stc_u16(out2 + (size_t)tok * st.ld_out2 + (size_t)slot * st.ld_out2_slot + j, so[i]);
+    else stc_u16(out + (size_t)tok * st.ld_out + (size_t)slot * st.ld_out_slot + j + (arr == 1 ? NR : 0), so[i]);
   }
+  c.wrote_through = true;  // (the plain form above returns before this and keeps the write-back)
 }
 
 __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char *smem) {
@@ -2332,8 +2334,9 @@ __device__ __forceinline__ void stage_moe_combine(CStage &st, Ctx &c, int M) {
     float s = bf2f(ldc_u16(res + (size_t)t * st.ld_res + j));
     for (int k = 0; k < st.topk; k++)
       s = fmaf(bf2f(ldc_u16(in + (size_t)t * st.ld_in + (size_t)k * st.ld_in_slot + j)), ldc_f32(st.moe_topk_w + (size_t)t * st.ld_topk_w + k), s);
-    out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(s);
+    stc_u16(out + (size_t)t * st.ld_out + j, (uint16_t)f2bf(s));
   }
+  c.wrote_through = true;
 }
 
 // Per-head RMSNorm + rotate-half RoPE of one 128-wide head row by one wavefront (lane l owns elements
