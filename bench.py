@@ -3,7 +3,9 @@
 A "step" is one decode iteration of the persistent megakernel for the whole batch.  The prompt (80 seeded random ids
 per request) is ingested and W warm-up decode steps run untimed; then EXACTLY K decode steps run inside ONE persistent
 launch, bracketed by torch.cuda.synchronize() on both sides.  Weights, KV cache and meta tensors are resident in HBM
-before the timed region.  Prints one JSON line.
+before the timed region.  Prints one JSON line.  The metric is quoted at two batch sizes: the default run times BS=1
+(the line's `value`, `ms_per_step`, `roofline`) and then BS=64 on the same weights (the line's "bs64" object, with its
+own ms_per_step, context range and roofline); --batch N runs one batch size only.
 
 roofline: the dominant (only) kernel is mk_persistent_kernel; its algorithmic bytes per launch are
 K x (all bf16 weight matrices once + the K/V rows of every cached position of every request), divided by the launch
@@ -80,45 +82,15 @@ def cpu_baseline(shape, n_layers_sample=2, steps=3, context=80):
                       f"extrapolated to {shape.num_layers} layers; torch-order bf16 oracle"}
 
 
-def main():
-    ap = argparse.ArgumentParser()
-    ap.add_argument("--gpus", type=int, default=1)
-    ap.add_argument("--steps", type=int, default=1024)
-    ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--batch", type=int, default=1, help="requests decoded concurrently (BS)")
-    ap.add_argument("--layers", type=int, default=36)
-    ap.add_argument("--prompt-length", type=int, default=80)
-    ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
-    ap.add_argument("--model", choices=["qwen3-8b", "qwen3-30b-a3b"], default="qwen3-8b",
-                    help="qwen3-8b: the headline dense shape; qwen3-30b-a3b: the mixture-of-experts shape (128 experts, top-8), reported alongside")
-    ap.add_argument("--no-cpu-baseline", action="store_true")
-    ap.add_argument("--calib-copy", action="store_true", help="also run one 1 GiB device-to-device copy (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
-    args = ap.parse_args()
-    if args.gpus != 1:
-        print("bench.py: this build runs the decode megakernel on ONE GPU; --gpus must be 1 "
-              "(multi-GPU tensor parallelism is not built)", file=sys.stderr)
-        sys.exit(2)
-    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
-        print("bench.py: launched with WORLD_SIZE>1; this benchmark is single-GPU", file=sys.stderr)
-        sys.exit(2)
-    import torch
-    from demo_qwen3 import Qwen3Decoder, Qwen3Shape, random_weights
-    if not torch.cuda.is_available():
-        print("bench.py: no GPU visible; the megakernel has no CPU path", file=sys.stderr)
-        sys.exit(1)
-    torch.cuda.set_device(0)
-    moe = args.model == "qwen3-30b-a3b"
-    shape = Qwen3Shape.qwen3_30b_a3b(min(args.layers, 48) if args.layers != 36 else 48) if moe else Qwen3Shape(num_layers=args.layers)
-    B, K, W, P = args.batch, args.steps, args.warmup, args.prompt_length
-    max_seq = max(1200, P + W + K + 2)
-    if args.calib_copy:
-        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
-        dst = torch.empty_like(src)
-        dst.copy_(src)
-        torch.cuda.synchronize()
-        del src, dst
-    weights = random_weights(shape, seed=0)
-    dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
+# HBM bytes per decode step as the counters saw them (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE, both scaled by a
+# 1 GiB copy in the same run; the passes and their commands are in profiles/mk_persistent_kernel_qwen3-8b_bs1.md and
+# ..._bs64.md).  Counter passes cannot run inside a timed benchmark, so the bench line carries these per-step figures
+# times the steps of its launch; a batch size without a committed counter pass reports null.
+MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): 15.183e9 + 13.5e6}
+
+
+def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
+    """Ingest B prompts of P tokens, run W untimed decode steps, then time exactly K decode steps in ONE persistent launch."""
     prompts = [torch.randint(0, shape.vocab_size, (P,), generator=torch.Generator().manual_seed(r)) for r in range(B)]
     dec.load_prompts(prompts)
     # prompt ingestion: run until every request has consumed its prompt (first decode token produced), then warm up
@@ -141,7 +113,7 @@ def main():
     t1 = time.perf_counter()
     st = dec.mpk.stats()
     assert not finished, "requests finished inside the timed region; lower --steps"
-    assert int(dec.meta["step"].min().item()) == ctx0 + K, "timed region did not run exactly K decode steps"
+    assert int(dec.meta["step"].min().item()) == ctx0 + K and int(dec.meta["step"].max().item()) == ctx0 + K, "timed region did not run exactly K decode steps"
     wall_ms = (t1 - t0) * 1e3
     kernel_ms = st["last_launch_ms"]
     ms_per_step = wall_ms / K
@@ -149,25 +121,89 @@ def main():
     kv_positions = sum(ctx0 + 1 + i for i in range(K))
     # mixture of experts: a step streams the experts its tokens select; B tokens choosing top-k of E uniformly touch
     # E * (1 - (1 - k/E)^B) distinct experts per layer in expectation (exactly k for one token)
+    moe = shape.num_experts > 0
     distinct = None
     if moe and B > 1:
         distinct = shape.num_experts * (1.0 - (1.0 - shape.num_experts_per_tok / shape.num_experts) ** B)
     bytes_total = int(K * shape.weight_bytes_per_token(distinct) + B * kv_positions * shape.kv_bytes_per_position())
     achieved = bytes_total / (kernel_ms * 1e-3) / 1e9
-    out = {
-        "metric": f"decode TPOT ms/token {'Qwen3-30B-A3B' if moe else 'Qwen3-8B'}-shape bf16", "value": round(ms_per_step, 4), "unit": "ms/token", "n_gpus": 1, "steps": K,
-        "warmup": W, "ms_per_step": round(ms_per_step, 4), "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
-        "data": "synthetic (random-init weights ~N(0,0.02), seeded random prompts)",
-        "config": {"workload": f"{'Qwen3-30B-A3B (128 experts, top-8)' if moe else 'Qwen3-8B'} shape, {shape.num_layers} layers, vocab {shape.vocab_size}, BS={B}, prompt {P}, "
-                               f"context {ctx0}..{ctx0 + K}, max_seq_len {max_seq}, page_size 4096, graph mode {args.mode}",
-                   "batch": B, "tokens_per_s": round(B * 1e3 / ms_per_step, 1), "prefill_iterations": prefill_iters},
+    per_step = MEASURED_TRAFFIC_BYTES_PER_STEP.get((model, B))
+    return {
+        "batch": B, "ms_per_step": round(ms_per_step, 4), "tokens_per_s": round(B * 1e3 / ms_per_step, 1), "steps": K, "warmup": W,
+        "workload": f"{'Qwen3-30B-A3B (128 experts, top-8)' if moe else 'Qwen3-8B'} shape, {shape.num_layers} layers, vocab {shape.vocab_size}, BS={B}, prompt {P}, "
+                    f"context {ctx0}..{ctx0 + K}, max_seq_len {max_seq}, page_size 4096, graph mode {mode}",
+        "prefill_iterations": prefill_iters,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
-                     "traffic": None, "kernel": "mk_persistent_kernel", "kernel_ms_per_launch": round(kernel_ms, 3),
-                     "algorithmic_bytes_per_launch": bytes_total},
+                     "traffic": None if per_step is None else int(per_step * K),
+                     "traffic_source": None if per_step is None else "per-step FETCH_SIZE/WRITE_SIZE counter passes in profiles/ x steps of this launch",
+                     "kernel": "mk_persistent_kernel", "kernel_ms_per_launch": round(kernel_ms, 3), "algorithmic_bytes_per_launch": bytes_total},
     }
-    dec.mpk.finalize()
-    del dec, weights
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=1024)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--batch", type=int, default=None,
+                    help="requests decoded concurrently (BS).  Default: the metric's two batch sizes, 1 (the headline `value`) and 64 (reported under \"bs64\")")
+    ap.add_argument("--layers", type=int, default=36)
+    ap.add_argument("--prompt-length", type=int, default=80)
+    ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
+    ap.add_argument("--model", choices=["qwen3-8b", "qwen3-30b-a3b"], default="qwen3-8b",
+                    help="qwen3-8b: the headline dense shape; qwen3-30b-a3b: the mixture-of-experts shape (128 experts, top-8), reported alongside")
+    ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--calib-copy", action="store_true", help="also run one 1 GiB device-to-device copy (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this build runs the decode megakernel on ONE GPU; --gpus must be 1 "
+              "(multi-GPU tensor parallelism is not built)", file=sys.stderr)
+        sys.exit(2)
+    if int(os.environ.get("WORLD_SIZE", "1")) != 1:
+        print("bench.py: launched with WORLD_SIZE>1; this benchmark is single-GPU", file=sys.stderr)
+        sys.exit(2)
+    import torch
+    from demo_qwen3 import Qwen3Decoder, Qwen3Shape, random_weights
+    if not torch.cuda.is_available():
+        print("bench.py: no GPU visible; the megakernel has no CPU path", file=sys.stderr)
+        sys.exit(1)
+    torch.cuda.set_device(0)
+    from mirage import _capi
+    # where the library is mapped (a crash report of the process can be matched against it)
+    print(f"bench.py: pid {os.getpid()}, {_capi.LIB_PATH} at {_capi.load_address():#x}", file=sys.stderr, flush=True)
+    moe = args.model == "qwen3-30b-a3b"
+    shape = Qwen3Shape.qwen3_30b_a3b(min(args.layers, 48) if args.layers != 36 else 48) if moe else Qwen3Shape(num_layers=args.layers)
+    K, W, P = args.steps, args.warmup, args.prompt_length
+    batches = [args.batch] if args.batch else ([1, 64] if not moe else [1])
+    max_seq = max(1200, P + W + K + 2)
+    if args.calib_copy:
+        src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
+        dst = torch.empty_like(src)
+        dst.copy_(src)
+        torch.cuda.synchronize()
+        del src, dst
+    weights = random_weights(shape, seed=0)
+    legs = []
+    for B in batches:
+        dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
+        legs.append(run_leg(torch, dec, shape, args.model, B, K, W, P, max_seq, args.mode))
+        dec.mpk.finalize()
+        del dec
+    del weights
     torch.cuda.synchronize()
+    torch.cuda.empty_cache()
+    head = legs[0]
+    name = "Qwen3-30B-A3B" if moe else "Qwen3-8B"
+    out = {
+        "metric": f"decode TPOT ms/token @BS={','.join(str(l['batch']) for l in legs)} {name}-shape bf16; % of HBM roofline",
+        "value": head["ms_per_step"], "unit": "ms/token", "n_gpus": 1, "steps": K,
+        "warmup": W, "ms_per_step": head["ms_per_step"], "higher_is_better": False, "scaling": "weak", "vs_baseline": None, "dtype": "bf16",
+        "data": "synthetic (random-init weights ~N(0,0.02), seeded random prompts)",
+        "config": {"workload": head["workload"], "batch": head["batch"], "tokens_per_s": head["tokens_per_s"], "prefill_iterations": head["prefill_iterations"]},
+        "roofline": head["roofline"],
+    }
+    for leg in legs[1:]:
+        out[f"bs{leg['batch']}"] = leg  # the metric's other batch size: same model, same steps, its own roofline
     if not args.no_cpu_baseline:
         out["cpu_baseline"] = cpu_baseline(shape)
     print(json.dumps(out), flush=True)

@@ -114,6 +114,7 @@ struct mk_graph {
   int64_t weight_bytes = 0;
   size_t attn_cnt_n = 0;
   int num_ref_tasks = 0, num_ref_events = 0;
+  int last_linear_task = -1, last_linear_stage = -1;  // lowering: the most recent linear task and the stage it became
 };
 
 namespace {
@@ -226,7 +227,20 @@ int lower_linear(mk_graph *g, size_t &i) {
   if (!linear_kind(lt.name, &res, &silu, &extra)) return fail(MK_EINVAL, "internal: '%s' is not a linear", lt.name.c_str());
   const size_t need_ops = 3 + (res ? 1 : 0) + extra;
   if (lt.ops.size() != need_ops) return fail(MK_EINVAL, "task '%s' expects %zu operands, got %zu", lt.name.c_str(), need_ops, lt.ops.size());
-  const int in_id = lt.ops[0], w_id = lt.ops[1], res_id = res ? lt.ops[2] : -1, out_id = lt.ops.back();
+  const int in_id = lt.ops[0], w_id = lt.ops[1];
+  int res_id = res ? lt.ops[2] : -1, out_id = lt.ops.back();
+  size_t consumed_linear = 1;
+  if (lt.name == "splitk_linear_mi300" && g->tensors[out_id].dtype == MK_DT_F32) {
+    // the reference's two-task split-K: partial products into an fp32 workspace, then splitk_reduce [workspace, residual,
+    // output] sums the slices and adds the residual.  The pair is one stage here; the workspace is never written.
+    const Task *rd = i + 1 < g->tasks.size() ? &g->tasks[i + 1] : nullptr;
+    if (!rd || rd->name != "splitk_reduce_mi300" || rd->ops.size() != 3 || rd->ops[0] != out_id)
+      return fail(MK_EUNSUPPORTED, "splitk_linear_mi300 into an fp32 workspace must be followed by splitk_reduce_mi300 over that workspace");
+    res = true;
+    res_id = rd->ops[1];
+    out_id = rd->ops[2];
+    consumed_linear = 2;
+  }
   const Tensor &tin = g->tensors[in_id];
   Tensor &tout = g->tensors[out_id];
   if (tin.ndims != 2 || tout.ndims != 2) return fail(MK_EINVAL, "task '%s': input/output must be 2-D", lt.name.c_str());
@@ -310,20 +324,123 @@ int lower_linear(mk_graph *g, size_t &i) {
                               (st.flags & MK_F_SILU) ? "+silu" : "", tin.name.c_str(), g->tensors[w_id].name.c_str(), tfo.name.c_str(), st.n, st.k,
                               st.w.nseg));
   g->weight_bytes += (int64_t)st.n * st.k * 2;
-  i += act ? 2 : 1;
+  g->last_linear_task = (int)i;
+  g->last_linear_stage = (int)g->stages.size() - 1;
+  i += act ? 2 : consumed_linear;
   return MK_OK;
 }
 
+// silu_mul_linear_with_residual [input [tokens, 2I], weight [H, I], residual, output]: out = silu_mul(input) W^T + residual.
+// When `input` was produced by the linear stage right before it, the activation moves into that stage's epilogue
+// (single rounding, like the fused gate/up task) writing a library-owned [tokens, I] tensor, and the gate/up tensor
+// itself is no longer written; which rows are gate and which are up comes from the producer's weight view (a
+// shuffled [gate ; up] view) or, for a physically interleaved weight, from the producer's grid (one block per
+// half-group, which is how the reference drivers size it).  Otherwise a standalone activation stage reads `input` as
+// [gate | up] halves, the layout the reference task kernel reads (tasks/ampere/silu_mul_linear.cuh:78-80).
+int lower_silu_mul_linear(mk_graph *g, size_t &i) {
+  const Task &t = g->tasks[i];
+  if (t.ops.size() != 4) return fail(MK_EINVAL, "silu_mul_linear_with_residual expects 4 operands");
+  const Tensor &x = g->tensors[t.ops[0]], &w = g->tensors[t.ops[1]], &r = g->tensors[t.ops[2]], &o = g->tensors[t.ops[3]];
+  const int B = g->cfg.max_num_batched_tokens;
+  if (x.ndims != 2 || w.ndims != 2 || r.ndims != 2 || o.ndims != 2 || x.dtype != MK_DT_BF16 || o.dtype != MK_DT_BF16 || r.dtype != MK_DT_BF16)
+    return fail(MK_EINVAL, "silu_mul_linear_with_residual: operands must be 2-D bf16");
+  const int I = (int)w.dims[1], H = (int)w.dims[0];
+  if (x.dims[1] != 2 * (int64_t)I || o.dims[1] < H || r.dims[1] < H || x.dims[0] < B || o.dims[0] < B || r.dims[0] < B)
+    return fail(MK_EINVAL, "silu_mul_linear_with_residual: input must be [tokens, 2*%d], residual/output [tokens, >=%d]", I, H);
+  if (I % 8 || (B > 1 && I % 32)) return fail(MK_EINVAL, "silu_mul_linear_with_residual: intermediate size %d must be a multiple of 8 (32 when batching)", I);
+  void *mid = nullptr;
+  int rc = dev_alloc(g, &mid, (size_t)B * I * 2);
+  if (rc) return rc;
+  const bool have_producer = g->last_linear_stage >= 0 && g->last_linear_stage == (int)g->stages.size() - 1;
+  MkStage *prev = have_producer ? &g->stages.back() : nullptr;
+  if (prev && prev->op == MK_OP_LINEAR && prev->out == x.ptr && !(prev->flags & (MK_F_SILU | MK_F_RES)) && prev->n == 2 * I) {
+    int half = 0;
+    if (prev->w.nseg == 2 && prev->w.seg_rows[0] == prev->w.seg_rows[1]) {
+      half = prev->w.seg_rows[0];
+    } else if (prev->w.nseg == 1) {
+      const Task &pt = g->tasks[g->last_linear_task];
+      const int blocks = pt.grid[0] * pt.grid[1] * pt.grid[2];
+      half = (blocks >= 2 && (2 * I) % blocks == 0) ? 2 * I / blocks : I;
+    }
+    if (half <= 0 || (2 * I) % (2 * half)) return fail(MK_EINVAL, "silu_mul_linear_with_residual: cannot tell gate rows from up rows of '%s'", x.name.c_str());
+    prev->flags |= MK_F_SILU;
+    prev->silu_half = half;
+    prev->out = mid;
+    prev->ld_out = I;
+    g->stage_desc.back() += fmt(" [+silu half=%d folded in from silu_mul_linear_with_residual; output is library-owned]", half);
+  } else {
+    MkStage a;
+    memset(&a, 0, sizeof(a));
+    a.op = MK_OP_SILU_MUL;
+    a.n = I;
+    a.silu_half = I;
+    a.groups = 1;
+    a.in = x.ptr;
+    a.ld_in = (int)x.strides[0];
+    a.out = mid;
+    a.ld_out = I;
+    g->stages.push_back(a);
+    g->stage_desc.push_back(fmt("SILU_MUL %s -> (library) n=%d half=%d", x.name.c_str(), I, I));
+  }
+  MkStage st;
+  memset(&st, 0, sizeof(st));
+  st.op = MK_OP_LINEAR;
+  st.flags = MK_F_RES;
+  st.k = I;
+  int64_t rows;
+  int halfw;
+  rc = resolve_weight(g, t.ops[1], I, &st.w, &rows, &halfw);
+  if (rc) return rc;
+  st.n = (int)rows;
+  st.eps = g->cfg.rms_eps;
+  st.in = mid;
+  st.ld_in = I;
+  st.out = o.ptr;
+  st.ld_out = (int)o.strides[0];
+  st.res = r.ptr;
+  st.ld_res = (int)r.strides[0];
+  g->stages.push_back(st);
+  g->stage_desc.push_back(fmt("LINEAR+res silu_mul(%s) x %s -> %s n=%d k=%d", x.name.c_str(), w.name.c_str(), o.name.c_str(), st.n, st.k));
+  g->weight_bytes += (int64_t)st.n * st.k * 2;
+  i++;
+  return MK_OK;
+}
+
+// A merge task that closes a split-KV attention task: [lse, chunked output, final output].  Returns the final
+// output's tensor id when task `j` is such a merge over the attention's chunked output, -1 otherwise.
+int merge_output_of(mk_graph *g, size_t j, const char *merge_name, int chunked_out_id) {
+  if (j >= g->tasks.size()) return -1;
+  const Task &m = g->tasks[j];
+  if (m.name != merge_name || m.ops.size() != 3 || m.ops[1] != chunked_out_id) return -1;
+  return m.ops[2];
+}
+
+// Every attention flavour of the API becomes ONE stage (q/k-norm, RoPE, KV append, attention over a KV split the stage
+// chooses itself, merge): the fused tasks directly, kv_cache_update + attention as a pair, and any of them built with
+// num_kv_chunks > 1 together with the merge task that must follow (the stage writes the merge's output; the chunked
+// accumulator and the log-sum-exp tensor of the reference's two-task form are never touched).
 int lower_attention(mk_graph *g, size_t &i) {
   const Task &t0 = g->tasks[i];
-  int in_id, kc_id, vc_id, qn_id, kn_id, cos_id, sin_id, out_id, qws_id = -1, nq = 0;
+  int in_id, kc_id, vc_id, qn_id, kn_id, cos_id, sin_id, out_id, qws_id = -1, nq = 0, chunks = 1;
   size_t consumed = 1;
+  const char *merge = nullptr;
   if (t0.name == "gang_attn_split_kv_mi300") {
     if (t0.ops.size() != 10 || t0.params.size() < 10) return fail(MK_EINVAL, "gang_attn_split_kv_mi300 expects 10 operands / 10 params");
     in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
     out_id = t0.ops[8]; qws_id = t0.ops[9];
     nq = t0.params[0];
-    if (t0.params[6] != 1) return fail(MK_EUNSUPPORTED, "num_kv_chunks=%d: the kernel splits KV internally; pass 1 and drop the merge layer", t0.params[6]);
+    chunks = t0.params[6];
+    merge = "gang_attn_merge_mi300";
+  } else if (t0.name == "paged_attention" || t0.name == "paged_attention_split_kv_mi300") {
+    const bool split = t0.name != "paged_attention";
+    if (t0.ops.size() != (split ? 9u : 8u) || t0.params.size() < (split ? 7u : 6u)) return fail(MK_EINVAL, "%s: wrong number of operands / params", t0.name.c_str());
+    in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
+    out_id = t0.ops.back();
+    nq = t0.params[0];
+    if (split) {
+      chunks = 2;  // the chunked [tokens, chunks * heads * head_dim, kv heads] output always needs the merge task
+      merge = "paged_attention_split_kv_merge_mi300";
+    }
   } else if (t0.name == "kv_cache_update_mi300") {
     if (t0.ops.size() != 8 || t0.params.size() < 7) return fail(MK_EINVAL, "kv_cache_update_mi300 expects 8 operands / 7 params");
     if (i + 1 >= g->tasks.size() || g->tasks[i + 1].name != "paged_attention_ck_fmha_split_kv_mi300")
@@ -335,15 +452,28 @@ int lower_attention(mk_graph *g, size_t &i) {
     if (t1.ops[0] != qws_id || t1.ops[1] != kc_id || t1.ops[2] != vc_id) return fail(MK_EINVAL, "attention does not consume the q workspace / caches of the preceding kv_cache_update");
     out_id = t1.ops[3];
     nq = t0.params[0];
-    if (t1.params[5] != 1) return fail(MK_EUNSUPPORTED, "num_kv_chunks=%d: the kernel splits KV internally; pass 1 and drop the merge layer", t1.params[5]);
+    chunks = t1.params[5];
+    merge = "paged_attention_ck_fmha_merge_mi300";
     consumed = 2;
   } else {
     return fail(MK_EUNSUPPORTED, "attention task '%s' is not supported", t0.name.c_str());
+  }
+  if (chunks < 1) return fail(MK_EINVAL, "%s: num_kv_chunks=%d", t0.name.c_str(), chunks);
+  if (chunks > 1) {
+    const int fin = merge_output_of(g, i + consumed, merge, out_id);
+    if (fin < 0) return fail(MK_EUNSUPPORTED, "%s with num_kv_chunks=%d must be followed by %s over its chunked output", t0.name.c_str(), chunks, merge);
+    out_id = fin;
+    consumed++;
   }
   const Tensor &tin = g->tensors[in_id], &kc = g->tensors[kc_id], &vc = g->tensors[vc_id], &to = g->tensors[out_id];
   if (kc.ndims != 4 || vc.ndims != 4) return fail(MK_EINVAL, "k/v cache must be 4-D [pages, page_size, kv_heads, head_dim]");
   const int nkv = (int)kc.dims[2], D = (int)kc.dims[3];
   if (D != 128) return fail(MK_EUNSUPPORTED, "head_dim %d: only 128 is supported", D);
+  if (kc.dims[0] < g->cfg.max_num_pages || vc.dims[0] < g->cfg.max_num_pages)
+    return fail(MK_EINVAL, "k/v cache holds %lld / %lld pages, fewer than max_num_pages=%d", (long long)kc.dims[0], (long long)vc.dims[0], g->cfg.max_num_pages);
+  for (int d = 1; d < 4; d++)
+    if (kc.dims[d] != vc.dims[d]) return fail(MK_EINVAL, "k and v cache shapes differ");
+  if (kc.dtype != MK_DT_BF16 || vc.dtype != MK_DT_BF16) return fail(MK_EINVAL, "k/v cache must be bf16");
   if (kc.dims[1] != g->cfg.page_size) return fail(MK_EINVAL, "k cache page size %lld != configured %d", (long long)kc.dims[1], g->cfg.page_size);
   if (nkv <= 0 || nq % nkv) return fail(MK_EINVAL, "q heads %d not a multiple of kv heads %d", nq, nkv);
   const int qpk = nq / nkv;
@@ -565,6 +695,7 @@ int lower(mk_graph *g) {
   g->stages.clear();
   g->stage_desc.clear();
   g->weight_bytes = 0;
+  g->last_linear_task = g->last_linear_stage = -1;
   size_t i = 0;
   const int B = g->cfg.max_num_batched_tokens;
   while (i < g->tasks.size()) {
@@ -615,6 +746,9 @@ int lower(mk_graph *g) {
     } else if (linear_kind(t.name, &res, &silu, &extra)) {
       int rc = lower_linear(g, i);
       if (rc) return rc;
+    } else if (t.name == "silu_mul_linear_with_residual") {
+      int rc = lower_silu_mul_linear(g, i);
+      if (rc) return rc;
     } else if (t.name == "silu_mul") {
       if (t.ops.size() != 2) return fail(MK_EINVAL, "silu_mul expects 2 operands");
       const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[t.ops[1]];
@@ -633,7 +767,8 @@ int lower(mk_graph *g) {
       g->stages.push_back(st);
       g->stage_desc.push_back(fmt("SILU_MUL %s -> %s n=%d half=%d", x.name.c_str(), o.name.c_str(), st.n, st.silu_half));
       i++;
-    } else if (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300") {
+    } else if (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300" || t.name == "paged_attention" ||
+               t.name == "paged_attention_split_kv_mi300") {
       int rc = lower_attention(g, i);
       if (rc) return rc;
     } else if (t.name == "moe_topk_softmax_mi300") {
@@ -700,6 +835,9 @@ int lower(mk_graph *g) {
       g->stages.push_back(sr);
       g->stage_desc.push_back(fmt("ARGMAX_REDUCE -> %s", o.name.c_str()));
       i += 2;
+    } else if (t.name == "paged_attention_split_kv_merge_mi300" || t.name == "paged_attention_ck_fmha_merge_mi300" || t.name == "gang_attn_merge_mi300" ||
+               t.name == "splitk_reduce_mi300") {
+      return fail(MK_EUNSUPPORTED, "task '%s' must directly follow the split task whose partial results it combines", t.name.c_str());
     } else {
       return fail(MK_EUNSUPPORTED, "task '%s' has no MI355X lowering", t.name.c_str());
     }
@@ -733,7 +871,10 @@ int task_type_id(const std::string &n) {
       {"gang_linear_silu_mi300", 142}, {"linear_silu_mi300", 182}, {"splitk_linear_mi300", 129}, {"gang_splitk_linear_res_mi300", 144},
       {"gang_linear_n_tiling_mi300", 147}, {"gang_linear_res_n_tiling_mi300", 148}, {"gang_linear_msplit_mi300", 183},
       {"gang_linear_res_msplit_mi300", 184}, {"moe_w13_linear_mi300", 170}, {"moe_w2_linear_mi300", 171}, {"moe_topk_softmax_mi300", 172},
-      {"moe_mul_sum_add_mi300", 173}, {"gang_moe_w13_linear_mi300", 174}, {"gang_moe_w2_linear_mi300", 175}, {"moe_silu_mul", 118}};
+      {"moe_mul_sum_add_mi300", 173}, {"gang_moe_w13_linear_mi300", 174}, {"gang_moe_w2_linear_mi300", 175}, {"moe_silu_mul", 118},
+      {"paged_attention", 116}, {"paged_attention_split_kv_mi300", 130}, {"paged_attention_split_kv_merge_mi300", 131},
+      {"paged_attention_ck_fmha_merge_mi300", 131}, {"gang_attn_merge_mi300", 139}, {"splitk_reduce_mi300", 132},
+      {"silu_mul_linear_with_residual", 105}};
   auto it = ids.find(n);
   return it == ids.end() ? 0 : it->second;
 }
@@ -771,7 +912,7 @@ int build_task_graph_json(mk_graph *g) {
     int po = -1, co = -1;
     for (size_t a = 0; a < c.ops.size() && po < 0; a++)
       for (size_t b = p.ops.size(); b-- > 0;)
-        if (p.ops[b] == c.ops[a]) {
+        if (p.ops[b] == c.ops[a] && c.ops[a] >= 0) {
           po = (int)b;
           co = (int)a;
           break;
@@ -841,10 +982,11 @@ int build_task_graph_json(mk_graph *g) {
       int n_out = 1;
       if (t.name == "argmax_partial") n_out = 2;
       if (t.name == "gang_attn_split_kv_mi300") n_out = 3;
-      if (t.name == "paged_attention_ck_fmha_split_kv_mi300") n_out = 2;
+      if (t.name == "paged_attention_ck_fmha_split_kv_mi300" || t.name == "paged_attention_split_kv_mi300") n_out = 2;
       const int n_in = (int)t.ops.size() - n_out;
       bool first_in = true, first_out = true;
       for (size_t a = 0; a < t.ops.size(); a++) {
+        if (t.ops[a] < 0) continue;  // optional operand that is absent
         const Tensor &tn = g->tensors[t.ops[a]];
         long long off = 0;
         long long dims[4];
@@ -937,10 +1079,21 @@ int mk_graph_create(const mk_config *cfg, mk_graph **out) {
     return fail(MK_EINVAL, "max_num_batched_tokens=%d outside [1, %d]", cfg->max_num_batched_tokens, MK_MAX_TOKENS);
   if (cfg->max_num_batched_requests < 1 || cfg->max_num_batched_requests > MK_MAX_TOKENS)
     return fail(MK_EINVAL, "max_num_batched_requests=%d outside [1, %d]", cfg->max_num_batched_requests, MK_MAX_TOKENS);
+  if (cfg->mode < MK_MODE_OFFLINE || cfg->mode > MK_MODE_ONEPASS) return fail(MK_EINVAL, "mode=%d is not one of enum mk_mode", cfg->mode);
+  if (cfg->max_tokens_per_request < 0 || cfg->max_tokens_per_request > MK_MAX_NEW_PER_REQ)
+    return fail(MK_EINVAL, "max_tokens_per_request=%d outside [0, %d]", cfg->max_tokens_per_request, MK_MAX_NEW_PER_REQ);
   if (cfg->page_size < 1 || cfg->max_num_pages < 1 || cfg->max_seq_length < 2) return fail(MK_EINVAL, "bad page_size / max_num_pages / max_seq_length");
   if ((int64_t)cfg->max_num_pages * cfg->page_size < cfg->max_seq_length)
     return fail(MK_EINVAL, "max_num_pages*page_size=%lld cannot hold one sequence of max_seq_length=%d", (long long)cfg->max_num_pages * cfg->page_size,
                 cfg->max_seq_length);
+  {
+    // Every slot can grow to max_seq_length, and the page ring (like the reference's) hands out pages without checking
+    // that any are free: with fewer pages than that a page would be given to two requests.
+    const int64_t per_req = ((int64_t)cfg->max_seq_length + cfg->page_size - 1) / cfg->page_size;
+    if (per_req * cfg->max_num_batched_requests > cfg->max_num_pages)
+      return fail(MK_EINVAL, "max_num_pages=%d cannot back %d concurrent requests of up to %lld pages each (max_seq_length=%d, page_size=%d)",
+                  cfg->max_num_pages, cfg->max_num_batched_requests, (long long)per_req, cfg->max_seq_length, cfg->page_size);
+  }
   if (cfg->max_num_pages > (MK_LDS_BYTES / 4)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 4);
   if (cfg->device < 0) {
     mk_graph *g = new mk_graph();
@@ -1097,8 +1250,11 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
     if (grid_dim[i] < 1) return fail(MK_EINVAL, "task '%s': grid_dim[%d]=%d", task_name, i, grid_dim[i]);
   }
   for (int i = 0; i < n_operands; i++) {
-    // id -1 = optional operand that is absent (e.g. no q/k norm)
-    if (tensor_ids[i] < -1 || tensor_ids[i] >= (int)g->tensors.size()) return fail(MK_EINVAL, "task '%s': bad tensor id %d", task_name, tensor_ids[i]);
+    // id -1 = optional operand that is absent: only the q/k-norm weights and the cos/sin tables of the attention tasks
+    const bool optional = (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300" || t.name == "paged_attention" ||
+                           t.name == "paged_attention_split_kv_mi300") && i >= 3 && i <= 6;
+    if (tensor_ids[i] >= (int)g->tensors.size() || tensor_ids[i] < (optional ? -1 : 0))
+      return fail(MK_EINVAL, "task '%s': bad tensor id %d for operand %d", task_name, tensor_ids[i], i);
     t.ops.push_back(tensor_ids[i]);
     std::array<int, 3> m = {-1, -1, -1};
     if (input_maps) m = {input_maps[3 * i], input_maps[3 * i + 1], input_maps[3 * i + 2]};
@@ -1111,7 +1267,9 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
   int c;
   static const char *known[] = {"embedding", "rmsnorm", "gang_rmsnorm_mi300", "silu_mul", "gang_attn_split_kv_mi300", "kv_cache_update_mi300",
                                 "paged_attention_ck_fmha_split_kv_mi300", "argmax_partial", "argmax_reduce", "moe_topk_softmax_mi300", "moe_w13_linear_mi300",
-                                "moe_w2_linear_mi300", "gang_moe_w13_linear_mi300", "gang_moe_w2_linear_mi300", "moe_silu_mul", "moe_mul_sum_add_mi300"};
+                                "moe_w2_linear_mi300", "gang_moe_w13_linear_mi300", "gang_moe_w2_linear_mi300", "moe_silu_mul", "moe_mul_sum_add_mi300",
+                                "paged_attention", "paged_attention_split_kv_mi300", "paged_attention_split_kv_merge_mi300",
+                                "paged_attention_ck_fmha_merge_mi300", "gang_attn_merge_mi300", "splitk_reduce_mi300", "silu_mul_linear_with_residual"};
   bool ok = linear_kind(t.name, &a, &b, &c);
   for (auto k : known) ok = ok || t.name == k;
   if (!ok) return fail(MK_EUNSUPPORTED, "Unsupported task name: %s", task_name);
@@ -1154,7 +1312,7 @@ int mk_compile(mk_graph *g) {
   rt.page_size = c.page_size;
   rt.max_pages = c.max_num_pages;
   rt.total_requests = c.total_num_requests;
-  rt.max_new_per_req = MK_MAX_NEW_PER_REQ;
+  rt.max_new_per_req = c.max_tokens_per_request > 0 ? c.max_tokens_per_request : 8;
   rt.eos_token_id = c.eos_token_id;
   rt.step = c.step;
   rt.tokens = (long long *)c.tokens;
@@ -1241,13 +1399,18 @@ int mk_init_requests(mk_graph *g) {
   sc.page_queue_tail = rt.max_pages;
   HIP_TRY(hipMemcpy(g->d_sched, &sc, sizeof(sc), hipMemcpyHostToDevice));
   HIP_TRY(hipMemset(rt.attn_cnt, 0, sizeof(unsigned) * g->attn_cnt_n));
+  HIP_TRY(hipMemset(rt.splitk_cnt, 0, sizeof(unsigned) * 32 * (size_t)g->G));
   return MK_OK;
 }
 
 int mk_enqueue_steps(mk_graph *g, void *stream, int max_iterations) {
   if (!g) return fail(MK_EINVAL, "null argument");
   if (max_iterations < 1) return fail(MK_EINVAL, "max_iterations must be positive");
-  return do_launch(g, (hipStream_t)stream, max_iterations, 1);
+  switch (g->cfg.mode) {
+    case MK_MODE_OFFLINE: return do_launch(g, (hipStream_t)stream, max_iterations, MK_SCHED_OFFLINE);
+    case MK_MODE_ONLINE: return do_launch(g, (hipStream_t)stream, max_iterations, MK_SCHED_ONLINE);
+    default: return do_launch(g, (hipStream_t)stream, 1, MK_SCHED_FROM_META);  // the host's batch is run once
+  }
 }
 
 int mk_wait(mk_graph *g, void *stream, int *finished_out) {
@@ -1265,7 +1428,8 @@ int mk_launch(mk_graph *g, void *stream) {
   int finished = 0;
   int rc = mk_launch_steps(g, stream, 0x7fffffff, &finished);
   if (rc) return rc;
-  if (!finished) return fail(MK_EABORT, "kernel returned before all requests finished");
+  const bool runs_to_completion = g->cfg.mode == MK_MODE_OFFLINE || g->cfg.mode == MK_MODE_ONLINE;
+  if (runs_to_completion && !finished) return fail(MK_EABORT, "kernel returned before all requests finished");
   return MK_OK;
 }
 
@@ -1278,8 +1442,8 @@ int mk_run_once(mk_graph *g, void *stream, int num_tokens, const int32_t *tok_sl
     if (tok_slot[t] < 0 || tok_slot[t] >= rt.max_requests) return fail(MK_EINVAL, "tok_slot[%d]=%d out of range", t, tok_slot[t]);
     if (tok_pos[t] < 0 || tok_pos[t] >= rt.max_seq) return fail(MK_EINVAL, "tok_pos[%d]=%d outside [0, max_seq_length)", t, tok_pos[t]);
     if (tok_first[t] < 0 || tok_first[t] > t || tok_slot[tok_first[t]] != tok_slot[t] || tok_pos[t] - tok_pos[tok_first[t]] != t - tok_first[t] ||
-        t - tok_first[t] >= MK_MAX_NEW_PER_REQ)
-      return fail(MK_EINVAL, "tok_first[%d]=%d is not the first row of a contiguous run of <= %d tokens of the same request", t, tok_first[t], MK_MAX_NEW_PER_REQ);
+        t - tok_first[t] >= rt.max_new_per_req)
+      return fail(MK_EINVAL, "tok_first[%d]=%d is not the first row of a contiguous run of <= %d tokens of the same request", t, tok_first[t], rt.max_new_per_req);
   }
   HIP_TRY(hipSetDevice(g->cfg.device));
   hipStream_t s = (hipStream_t)stream;
@@ -1291,7 +1455,7 @@ int mk_run_once(mk_graph *g, void *stream, int num_tokens, const int32_t *tok_sl
   HIP_TRY(hipMemcpy(&sc, g->d_sched, sizeof(sc), hipMemcpyDeviceToHost));
   sc.num_tokens = num_tokens;
   HIP_TRY(hipMemcpy(g->d_sched, &sc, sizeof(sc), hipMemcpyHostToDevice));
-  int rc = do_launch(g, s, 1, 0);
+  int rc = do_launch(g, s, 1, MK_SCHED_HOST_ARRAYS);
   if (rc) return rc;
   return do_wait(g, s, nullptr);
 }

@@ -256,7 +256,7 @@ __device__ __forceinline__ void barrier_poll(Ctx &c) {
   auto done = [&](const unsigned (&v)[8]) -> bool {
     bool ok = true;
 #pragma unroll
-    for (int x = 0; x < 8; x++) ok = ok && (v[x] >= c.quotas[x] * epoch);
+    for (int x = 0; x < 8; x++) ok = ok && mk_counter_reached(v[x], c.quotas[x] * epoch);
     return ok;
   };
   while (true) {
@@ -388,6 +388,83 @@ __device__ int mk_prepare_next_batch(const MkRuntime &rt, int *scratch_pages) {
   sc->num_tokens = ntok;
   sc->num_reqs = nreq;
   return ntok;
+}
+
+// Batch description for a launch whose batch the HOST prepared (the reference's MODE_ONLINE_NOTOKEN, one pass per launch,
+// persistent_kernel.cuh:570-582, and MODE_ONEPASS): the caller has filled input_tokens, qo_indptr, paged_kv_indptr,
+// paged_kv_indices and paged_kv_last_page_len the way the reference's attention tasks read them -- request slot i owns
+// rows [qo_indptr[i], qo_indptr[i+1]) and its sequence, new tokens included, is (pages - 1) * page_size + last_page_len
+// long, so its rows sit at the last positions of that sequence.  Derives the per-row slot / position / first-row arrays
+// on the device (no host round trip, so a serving loop can enqueue launches back to back).  Runs on one thread.
+__device__ int mk_batch_from_meta(const MkRuntime &rt) {
+  const int R = rt.max_requests, B = rt.max_tokens;
+  int ntok = 0;
+  for (int i = 0; i < R; i++) {
+    const int q0 = rt.qo_indptr[i], n = rt.qo_indptr[i + 1] - q0;
+    if (n <= 0 || q0 < 0 || q0 + n > B) continue;
+    const int pages = rt.kv_indptr[i + 1] - rt.kv_indptr[i];
+    const int len = (pages - 1) * rt.page_size + rt.kv_last_page_len[i];
+    int nn = n > rt.max_new_per_req ? rt.max_new_per_req : n;  // more rows per request than the attention stage holds are not run
+    if (len - nn < 0 || len > rt.max_seq) continue;
+    for (int j = 0; j < nn; j++) {
+      rt.tok_slot[q0 + j] = i;
+      rt.tok_pos[q0 + j] = len - n + j;
+      rt.tok_first[q0 + j] = q0;
+    }
+    if (q0 + nn > ntok) ntok = q0 + nn;
+  }
+  rt.sched->num_tokens = ntok;
+  return ntok;
+}
+
+// The reference's MODE_ONLINE step (persistent_kernel.cuh:538-568): one request (slot 0, request 0) whose tokens the
+// host has written into tokens[0, :]; every pass consumes num_new_tokens[0] of them starting at step[0].  After a pass
+// step[0] advances by what the pass consumed, and the run ends when the position it started from is within two of
+// max_seq_length or the token after it is the EOS id -- the reference's test, on the step value from before the
+// advance.  What the reference leaves to the host and is done here instead: the page table of the one request
+// (identity: page j of the ring is page j of the sequence) and the qo / kv index arrays.  Runs on one thread.
+__device__ int mk_online_next_batch(const MkRuntime &rt) {
+  MkSched *sc = rt.sched;
+  const int PS = rt.page_size;
+  int step = rt.step[0];
+  if (sc->online_started) {
+    const int consumed = sc->num_tokens;
+    rt.step[0] = step + consumed;
+    const bool stop = (step + 2 >= rt.max_seq) || (rt.tokens[step + 1] == rt.eos_token_id);
+    step += consumed;
+    if (stop) {
+      sc->num_tokens = 0;
+      return 0;
+    }
+  }
+  sc->online_started = 1;
+  int n = rt.num_new_tokens ? rt.num_new_tokens[0] : 1;
+  n = n < 1 ? 1 : n;
+  n = min(n, min(rt.max_new_per_req, rt.max_tokens));
+  n = min(n, rt.max_seq - 1 - step);
+  if (n <= 0) {
+    sc->num_tokens = 0;
+    return 0;
+  }
+  for (int j = 0; j < n; j++) {
+    rt.input_tokens[j] = rt.tokens[step + j];
+    rt.tok_slot[j] = 0;
+    rt.tok_pos[j] = step + j;
+    rt.tok_first[j] = 0;
+  }
+  const int need = (step + n + PS - 1) / PS, last = (step + n) % PS;
+  rt.request_ids[0] = 0;
+  rt.kv_last_page_len[0] = last == 0 ? PS : last;
+  for (int j = 0; j < need && j < rt.max_pages; j++) rt.kv_indices[j] = j;
+  rt.qo_indptr[0] = 0;
+  rt.kv_indptr[0] = 0;
+  for (int i = 1; i <= rt.max_requests; i++) {
+    rt.qo_indptr[i] = n;
+    rt.kv_indptr[i] = need;
+  }
+  sc->num_tokens = n;
+  sc->num_reqs = 1;
+  return n;
 }
 
 // ----------------------------------------------------------------------------- weights
@@ -1083,8 +1160,9 @@ __device__ __forceinline__ TilePlan linear_tiles_plan(CStage &st, const Ctx &c) 
   if (st.k % (64 * 2 * MK_TILES_NB) != 0) return p;
   const int tpw = (p.wt + c.G - 1) / c.G;            // tiles per workgroup without a K split
   int S = 1;
-  while (S < MK_TUNE_SPLITK_MAXS && tpw * S < MK_TUNE_TPU && st.k % (S * 2 * 64 * 2 * MK_TILES_NB) == 0) S *= 2;
-  int tpu = (p.wt * S + c.G - 1) / c.G;              // tiles per range
+  while (S < MK_TUNE_SPLITK_MAXS && tpw * S < MK_TUNE_TPU && 2 * S <= c.G && st.k % (S * 2 * 64 * 2 * MK_TILES_NB) == 0) S *= 2;
+  const int gs = c.G / S;                             // ranges the grid can hold: S adjacent workgroups each
+  int tpu = (p.wt + gs - 1) / gs;                     // tiles per range
   tpu = (tpu + unit - 1) / unit * unit;
   if (S > 1 && tpu > 16) return p;                    // a split range is a single sweep
   if (S == 1 && tpw < MK_TUNE_TILES_MIN_TPW) return p;  // a few tiles per workgroup without a K split: the form that splits K inside the workgroup
@@ -2398,11 +2476,14 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int j16 = lane & 15, gg = wave * 4 + (lane >> 4);
   const int nkv = st.num_kv_heads;
-  uint16_t *qs = (uint16_t *)smem;                          // [QPK][128]
-  uint16_t *knew = (uint16_t *)(smem + 2048);               // [8][128]
-  uint16_t *vnew = (uint16_t *)(smem + 2048 + 2048);        // [8][128]
-  int *sflag = (int *)(smem + 6144);
-  float *part = (float *)(smem + 8192);                     // [16][QPK][132]
+  // LDS: q rows, then the K and V rows of this iteration's new positions (a request ingests up to MK_MAX_NEW_PER_REQ prompt
+  // tokens per iteration), then the per-group partial results
+  uint16_t *qs = (uint16_t *)smem;                                        // [QPK][128]
+  int *sflag = (int *)(smem + 2048);
+  uint16_t *knew = (uint16_t *)(smem + 4096);                             // [MK_MAX_NEW_PER_REQ][128]
+  uint16_t *vnew = knew + MK_MAX_NEW_PER_REQ * D;                         // [MK_MAX_NEW_PER_REQ][128]
+  float *part = (float *)(smem + 4096 + 2 * MK_MAX_NEW_PER_REQ * D * 2);  // [16][QPK][132]
+  static_assert(4096 + 2 * MK_MAX_NEW_PER_REQ * 128 * 2 + 16 * QPK * 132 * 4 <= MK_LDS_BYTES, "attention scratch exceeds the LDS window");
   const int n_items = M * nkv;
   int cmax = c.G / n_items;
   cmax = cmax < 1 ? 1 : (cmax > MK_ATTN_MAX_CHUNKS ? MK_ATTN_MAX_CHUNKS : cmax);
@@ -2887,7 +2968,10 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     if (run_scheduler) {
       barrier_wait(c);  // the previous iteration's sampled tokens are complete
       if (c.vid == 0 && threadIdx.x == 0) {
-        const int ntok = mk_prepare_next_batch(*rtp, (int *)smem);
+        int ntok;
+        if (run_scheduler == MK_SCHED_OFFLINE) ntok = mk_prepare_next_batch(*rtp, (int *)smem);
+        else if (run_scheduler == MK_SCHED_ONLINE) ntok = mk_online_next_batch(*rtp);
+        else ntok = mk_batch_from_meta(*rtp);
         if (ntok == 0) rt.sched->finished = 1;
         else rt.sched->iterations++;
         if (rt.timing && rt.sched->iterations <= rt.timing_cap) rt.timing[rt.sched->iterations] = (long long)wall_clock64();

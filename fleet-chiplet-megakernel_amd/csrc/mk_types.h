@@ -17,7 +17,8 @@
 #define MK_MAX_TOKENS 64      // max tokens per iteration supported by the kernels
 #define MK_ATTN_MAX_CHUNKS 32 // split-KV fan-out limit per (token, kv head)
 #define MK_ATTN_PSTRIDE 160   // floats per (work unit, q head) split-KV partial: 128 values + one 128-byte line of (max, sum)
-#define MK_MAX_NEW_PER_REQ 8  // prefill tokens per request per iteration (reference: MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
+#define MK_MAX_NEW_PER_REQ 64 // most prompt tokens one request may ingest per iteration (the attention stage keeps their K/V rows in LDS); the
+                              // configured value defaults to the reference's 8 (MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
 // LDS map of one workgroup (dynamic, > 80 KB pins one workgroup per CU):
 //   [0, 24 KB)      input row(s) of the running stage / attention scratch (attention may run on beyond 32 KB)
 //   [24 KB, 25 KB)  reduction scratch
@@ -124,10 +125,28 @@ struct MkSync {
   unsigned pad3[30];
 };
 
+// Barrier completion test.  Arrival counters and their targets (quota x epoch) are 32-bit and only ever grow during a
+// launch, so on a long launch both wrap; their difference taken as a signed number stays correct as long as the two
+// are less than 2^31 apart, and they are never more than one stage apart.
+#ifdef __HIP__
+#define MK_HOST_DEVICE __host__ __device__
+#else
+#define MK_HOST_DEVICE
+#endif
+MK_HOST_DEVICE inline bool mk_counter_reached(unsigned counter, unsigned target) { return (int)(counter - target) >= 0; }
+
+// Who describes the batch of an iteration (the kernel's `run_scheduler` argument).
+enum MkSchedMode {
+  MK_SCHED_HOST_ARRAYS = 0,  // the host wrote tok_slot / tok_pos / tok_first (mk_run_once)
+  MK_SCHED_OFFLINE = 1,      // on-GPU continuous batching over `tokens` (MODE_OFFLINE)
+  MK_SCHED_FROM_META = 2,    // derived on the GPU from the qo / paged-kv meta tensors the host filled (MODE_ONLINE_NOTOKEN, MODE_ONEPASS)
+  MK_SCHED_ONLINE = 3,       // one request, host-written tokens consumed num_new_tokens[0] at a time (MODE_ONLINE)
+};
+
 // Scheduler state that persists across launches (continuous batching, page ring).
 struct MkSched {
   int page_queue_head, page_queue_tail, next_request_id, num_tokens;
-  int num_reqs, finished, pad0, pad1;
+  int num_reqs, finished, online_started, pad1;
   long long iterations;   // decode iterations executed so far (all launches)
   long long pad2;
 };

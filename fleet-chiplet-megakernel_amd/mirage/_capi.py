@@ -18,6 +18,8 @@ MK_ESTATE = -3
 MK_EABORT = -4
 MK_EUNSUPPORTED = -5
 
+MK_MODES = {"offline": 0, "online": 1, "online_notoken": 2, "onepass": 3}
+
 # symbols include/fleet_mk.h declares; tests check that the library exports every one
 EXPORTED_SYMBOLS = [
     "mk_graph_create", "mk_graph_destroy", "mk_tensor_attach", "mk_tensor_new", "mk_tensor_shuffle",
@@ -39,6 +41,8 @@ class MkConfig(ctypes.Structure):
         ("device", ctypes.c_int),
         ("eos_token_id", ctypes.c_int64),
         ("rms_eps", ctypes.c_float),
+        ("mode", ctypes.c_int),
+        ("max_tokens_per_request", ctypes.c_int),
         ("reserved0", ctypes.c_int),
         ("step", ctypes.c_void_p),
         ("tokens", ctypes.c_void_p),
@@ -128,3 +132,17 @@ def check(rc):
 def int_array(values, ctype=ctypes.c_int):
     values = list(values)
     return (ctype * max(1, len(values)))(*values)
+
+
+def load_address():
+    """Address at which the shared library is mapped in this process (0 if it cannot be determined): lets a crash report
+    that lists program counters be matched against the library."""
+    load()
+    try:
+        with open("/proc/self/maps") as f:
+            for line in f:
+                if line.rstrip().endswith(os.path.basename(LIB_PATH)):
+                    return int(line.split("-", 1)[0], 16)
+    except OSError:
+        pass
+    return 0

@@ -8,7 +8,7 @@ whole generation.  Nothing here computes: without libfleet_mk.so and a gfx950 de
 """
 import ctypes
 import math
-
+import os
 import sys
 
 import torch
@@ -44,12 +44,21 @@ class PersistentKernel:
         spec_decode_config=None,
         use_cutlass_kernel: bool = False,
         eos_token_id: int = -1,
+        max_tokens_per_request: int = None,
     ):
+        """Arguments as the reference constructor (persistent_kernel.py:368-387).  `max_tokens_per_request` is the
+        reference's compile-time MPK_MAX_TOKENS_PER_REQUEST (prompt tokens one request ingests per iteration; 8 on AMD,
+        persistent_kernel.cuh:115-124): None takes the environment variable of that name, else 8; at most 64."""
         self.__finalized__ = False
         self._is_compiled = False
         self._handle = None
         if mode not in valid_persistent_kernel_modes:
             raise ValueError(f"Invalid persistent kernel mode: {mode}")
+        if mode not in _capi.MK_MODES:
+            raise NotImplementedError(f"mode '{mode}' is not supported by the MI355X megakernel (supported: {sorted(_capi.MK_MODES)})")
+        if max_tokens_per_request is None:
+            max_tokens_per_request = int(os.environ.get("MPK_MAX_TOKENS_PER_REQUEST", "8"))
+        self.max_tokens_per_request = int(max_tokens_per_request)
         if world_size != 1 or mpi_rank != 0:
             raise NotImplementedError("the MI355X megakernel runs on one GPU (world_size=1, mpi_rank=0)")
         if spec_decode_config is not None:
@@ -112,6 +121,8 @@ class PersistentKernel:
         cfg.device = -1 if self.host_only else (device.index if device.index is not None else torch.cuda.current_device())
         cfg.eos_token_id = int(eos_token_id)
         cfg.rms_eps = 1e-6
+        cfg.mode = _capi.MK_MODES[mode]
+        cfg.max_tokens_per_request = self.max_tokens_per_request
         cfg.step = mt["step"].data_ptr()
         cfg.tokens = mt["tokens"].data_ptr()
         cfg.input_tokens = mt["input_tokens"].data_ptr()
@@ -256,10 +267,36 @@ class PersistentKernel:
                     (done_counter, (0, -1, -1), -1), (output, (1, -1, -1), -1)], [k_splits])
 
     def splitk_linear_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
-        """persistent_kernel.py:1437.  Lowered like linear_layer: the MI355X stage never splits K across workgroups."""
+        """persistent_kernel.py:1437.  grid_dim = (N blocks, K splits, 1).  With a bf16 [tokens, N] output it is lowered
+        like linear_layer (the stage decides by itself whether to split K over workgroups, and sums the slices in a fixed
+        order); with the reference's fp32 [k_splits * tokens, N] workspace as output it must be followed by
+        splitk_reduce_layer over that workspace, and the pair becomes one linear stage."""
         assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
         self._task("splitk_linear_mi300", grid_dim, block_dim,
                    [(input, (-1, 1, -1), 1), (weight, (0, 1, -1), 1), (output, (1, 0, -1), -1)])
+
+    def splitk_reduce_layer(self, workspace: DTensor, residual: DTensor, output: DTensor, k_splits: int, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1901: output = bf16(sum of the k_splits slices of `workspace` + residual).  Closes a
+        splitk_linear_layer whose output is that workspace; no partial sums are ever written to it."""
+        assert workspace.num_dims == 2  # (k_splits * batch_size, hidden_size)
+        assert residual.num_dims == 2   # (batch_size, hidden_size)
+        assert output.num_dims == 2     # (batch_size, hidden_size)
+        self._task("splitk_reduce_mi300", grid_dim, block_dim,
+                   [(workspace, (1, -1, -1), 1), (residual, (1, -1, -1), 1), (output, (1, -1, -1), -1)], [k_splits])
+
+    def silu_mul_linear_with_residual_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, grid_dim: tuple,
+                                            block_dim: tuple):
+        """persistent_kernel.py:2174: output = bf16(silu_mul(input) @ weight^T + residual) with input = the gate/up linear's
+        [tokens, 2 * intermediate] result.  The activation is folded into the gate/up linear that produced `input` (whose
+        weight view says which columns are gate and which are up) and the product becomes a linear-with-residual stage; an
+        `input` of unknown origin is read as [gate | up] halves, the layout the reference task kernel reads
+        (tasks/ampere/silu_mul_linear.cuh:78-80)."""
+        assert input.num_dims == 2  # (batch_size, 2*intermediate_size)
+        assert weight.num_dims == 2  # (hidden_size, intermediate_size)
+        assert residual.num_dims == 2  # (batch_size, hidden_size)
+        assert input.dim(1) == 2 * weight.dim(1)
+        self._task("silu_mul_linear_with_residual", grid_dim, block_dim,
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), 1), (output, (1, -1, -1), 1)])
 
     # ------------------------------------------------------------------ mixture-of-experts layers
     def moe_topk_softmax_routing_layer(self, input: DTensor, output: tuple, grid_dim: tuple, block_dim: tuple):
@@ -462,7 +499,8 @@ class PersistentKernel:
 
     def paged_attention_ck_fmha_layer(self, q_workspace: DTensor, k_cache: DTensor, v_cache: DTensor, o_acc: DTensor, lse_acc: DTensor,
                                       attention_params: tuple, grid_dim: tuple, block_dim: tuple):
-        """persistent_kernel.py:981.  With num_kv_chunks == 1 `o_acc` is the final bf16 attention output."""
+        """persistent_kernel.py:981.  With num_kv_chunks == 1 `o_acc` is the final bf16 attention output; with more chunks it is
+        the reference's fp32 accumulator and paged_attention_ck_fmha_merge_layer must follow."""
         assert q_workspace.num_dims == 2
         assert k_cache.num_dims == 4 and v_cache.num_dims == 4
         assert o_acc.num_dims == 2 and lse_acc.num_dims == 2
@@ -528,11 +566,91 @@ class PersistentKernel:
     def verify_layer_dispatcher(self, *args, **kwargs):
         raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
 
-    def paged_attention_ck_fmha_merge_layer(self, *args, **kwargs):
-        raise NotImplementedError("split-KV merge layers are not needed: the attention stage splits and merges KV chunks internally; "
-                                  "build the attention layer with num_kv_chunks=1")
+    def single_batch_extend_attention_layer(self, *args, **kwargs):
+        raise NotImplementedError("single_batch_extend_attention_layer belongs to speculative decoding, which the MI355X megakernel does not support")
 
-    gang_paged_attention_split_kv_merge_layer = paged_attention_ck_fmha_merge_layer
+    # ------------------------------------------------------------------ attention variants that lower to the same stage
+    def _attn_flags(self, q_norm, k_norm, cos_pos_embed, sin_pos_embed, head_dim):
+        rotary_embed = 0
+        if cos_pos_embed is not None or sin_pos_embed is not None:
+            assert cos_pos_embed.num_dims == 2 and sin_pos_embed.num_dims == 2  # (seq_len, head_dim)
+            assert cos_pos_embed.dim(1) == head_dim and sin_pos_embed.dim(1) == head_dim
+            rotary_embed = 1
+        qk_norm = 0
+        if q_norm is not None or k_norm is not None:
+            assert q_norm.num_dims == 1 and k_norm.num_dims == 1  # (head_dim)
+            assert q_norm.dim(0) == head_dim and k_norm.dim(0) == head_dim
+            qk_norm = 1
+        return qk_norm, rotary_embed
+
+    def paged_attention_layer(self, input: DTensor, k_cache: DTensor, v_cache: DTensor, q_norm: DTensor, k_norm: DTensor, cos_pos_embed: DTensor,
+                              sin_pos_embed: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:724: q/k-norm + RoPE + KV append + paged attention as one task."""
+        assert input.num_dims == 2 and output.num_dims == 2
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4  # (num_pages, page_size, kv_heads, head_dim)
+        assert k_cache.dim(0) == self.max_num_pages and v_cache.dim(0) == self.max_num_pages
+        assert k_cache.dim(1) == self.page_size and v_cache.dim(1) == self.page_size
+        head_dim, num_kv_heads = k_cache.dim(3), k_cache.dim(2)
+        num_q_heads = output.dim(1) // head_dim
+        qk_norm, rotary_embed = self._attn_flags(q_norm, k_norm, cos_pos_embed, sin_pos_embed, head_dim)
+        assert grid_dim[0] == self.max_num_batched_requests
+        assert grid_dim[1] == num_kv_heads
+        self._task("paged_attention", grid_dim, block_dim,
+                   [(input, (-1, 1, -1), -1), (k_cache, (-1, 2, -1), 1), (v_cache, (-1, 2, -1), 1), (q_norm, _REPL, -1), (k_norm, _REPL, -1),
+                    (cos_pos_embed, _REPL, -1), (sin_pos_embed, _REPL, -1), (output, (-1, 1, -1), -1)],
+                   [num_q_heads, num_kv_heads, qk_norm, rotary_embed, self.max_seq_length, self.page_size])
+
+    def paged_attention_split_kv_layer(self, input: DTensor, k_cache: DTensor, v_cache: DTensor, q_norm: DTensor, k_norm: DTensor,
+                                       cos_pos_embed: DTensor, sin_pos_embed: DTensor, lse: DTensor, output: DTensor, attention_params: tuple,
+                                       grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:804.  Must be followed by paged_attention_split_kv_merge_layer over the same lse / output
+        tensors: the pair becomes ONE attention stage, which chooses its own KV split (at least 64 positions per chunk, as
+        many chunks as there are idle workgroups) and merges the chunks with the same rule (merge_splitkv.cuh:191-219).
+        `lse` and the chunked `output` are never written."""
+        assert input.num_dims == 2
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4
+        assert k_cache.dim(0) == self.max_num_pages and v_cache.dim(0) == self.max_num_pages
+        assert k_cache.dim(1) == self.page_size and v_cache.dim(1) == self.page_size
+        assert output.num_dims == 3 and lse.num_dims == 3
+        head_dim, num_kv_heads = k_cache.dim(3), k_cache.dim(2)
+        num_q_heads, num_kv_chunks = attention_params[0], attention_params[1]
+        qk_norm, rotary_embed = self._attn_flags(q_norm, k_norm, cos_pos_embed, sin_pos_embed, head_dim)
+        assert grid_dim[0] == self.max_num_batched_requests
+        assert grid_dim[1] == num_kv_heads
+        self._task("paged_attention_split_kv_mi300", grid_dim, block_dim,
+                   [(input, (-1, 1, -1), -1), (k_cache, (-1, 2, -1), 1), (v_cache, (-1, 2, -1), 1), (q_norm, _REPL, -1), (k_norm, _REPL, -1),
+                    (cos_pos_embed, _REPL, -1), (sin_pos_embed, _REPL, -1), (lse, (-1, 2, 1), -1), (output, (-1, 2, 1), -1)],
+                   [num_q_heads, num_kv_heads, qk_norm, rotary_embed, self.max_seq_length, self.page_size, num_kv_chunks])
+
+    def paged_attention_split_kv_merge_layer(self, lse: DTensor, output_tmp: DTensor, output: DTensor, attention_params: tuple, grid_dim: tuple,
+                                             block_dim: tuple):
+        """persistent_kernel.py:894 (see paged_attention_split_kv_layer)."""
+        assert lse.num_dims == 3 and output_tmp.num_dims == 3 and output.num_dims == 2
+        num_q_heads, head_dim = attention_params[0], attention_params[1]
+        num_kv_heads = grid_dim[1]
+        self._task("paged_attention_split_kv_merge_mi300", grid_dim, block_dim,
+                   [(lse, (-1, 2, -1), -1), (output_tmp, (-1, 2, -1), -1), (output, (-1, 1, -1), -1)],
+                   [num_q_heads // num_kv_heads, head_dim, self.max_seq_length, self.page_size, num_kv_heads])
+
+    def paged_attention_ck_fmha_merge_layer(self, lse: DTensor, output_tmp: DTensor, output: DTensor, attention_params: tuple, grid_dim: tuple,
+                                            block_dim: tuple):
+        """persistent_kernel.py:1028: closes a paged_attention_ck_fmha_layer built with num_kv_chunks > 1 whose o_acc / lse_acc
+        are `output_tmp` / `lse`; the pair (after kv_cache_update_layer) becomes one attention stage writing `output`."""
+        assert lse.num_dims == 2 and output_tmp.num_dims == 2 and output.num_dims == 2
+        num_q_heads, head_dim, num_kv_chunks, num_kv_heads = attention_params[0], attention_params[1], attention_params[2], attention_params[3]
+        self._task("paged_attention_ck_fmha_merge_mi300", grid_dim, block_dim,
+                   [(lse, _REPL, -1), (output_tmp, _REPL, -1), (output, _REPL, -1)],
+                   [num_q_heads // num_kv_heads, head_dim, self.max_seq_length, self.page_size, num_kv_heads, num_kv_chunks])
+
+    def gang_paged_attention_split_kv_merge_layer(self, lse: DTensor, output_tmp: DTensor, output: DTensor, attention_params: tuple,
+                                                  block_dim: tuple = (256, 1, 1)):
+        """persistent_kernel.py:1141: closes a gang_paged_attention_split_kv_layer built with num_kv_chunks > 1."""
+        assert lse.num_dims == 2 and output_tmp.num_dims == 2 and output.num_dims == 2
+        num_q_heads, head_dim, num_kv_heads, num_kv_chunks = attention_params[0], attention_params[1], attention_params[2], attention_params[3]
+        total = self.max_num_batched_requests * num_kv_heads
+        self._task("gang_attn_merge_mi300", (8, 1, 1), block_dim,
+                   [(lse, _REPL, -1), (output_tmp, _REPL, -1), (output, _REPL, -1)],
+                   [num_q_heads // num_kv_heads, head_dim, self.max_seq_length, self.page_size, num_kv_heads, math.ceil(total / 8), total, num_kv_chunks])
 
     # ------------------------------------------------------------------ compile / run
     def describe_program(self) -> str:

@@ -43,6 +43,15 @@ enum mk_dtype {
 
 enum mk_io_category { MK_IO_DEVICE = 0 /* "cuda_tensor" */, MK_IO_SYMMETRIC = 1 /* "nvshmem_tensor": single GPU => same */ };
 
+/* PersistentKernel's `mode` (persistent_kernel.py:204-214: -DMODE_OFFLINE / MODE_ONLINE / MODE_ONLINE_NOTOKEN / MODE_ONEPASS).
+ *  MK_MODE_OFFLINE         the on-GPU scheduler batches every request of `tokens` to completion (persistent_kernel.cuh:380-536);
+ *  MK_MODE_ONLINE          one request whose tokens the host wrote into tokens[0,:]: every pass consumes num_new_tokens[0] of
+ *                          them from step[0] on, until max_seq_length or the EOS id is reached (persistent_kernel.cuh:538-568);
+ *  MK_MODE_ONLINE_NOTOKEN  one pass per launch over the batch the host described in input_tokens, qo_indptr, paged_kv_indptr,
+ *                          paged_kv_indices and paged_kv_last_page_len (persistent_kernel.cuh:570-582): the serving-loop mode;
+ *  MK_MODE_ONEPASS         the same single pass (the reference compiles its test graphs in this mode). */
+enum mk_mode { MK_MODE_OFFLINE = 0, MK_MODE_ONLINE = 1, MK_MODE_ONLINE_NOTOKEN = 2, MK_MODE_ONEPASS = 3 };
+
 /* Constructor arguments of PersistentKernel (persistent_kernel.py:368-387) plus the
  * ten meta tensors in the order the reference hands them to init_func
  * (persistent_kernel.py:2590-2600).  All meta pointers are device pointers. */
@@ -58,6 +67,9 @@ typedef struct mk_config {
                                    graph without a GPU; mk_compile and the launch calls then fail with MK_ESTATE) */
   int64_t eos_token_id;
   float rms_eps;                /* 0 => 1e-6, the constant baked into the reference kernels */
+  int mode;                     /* enum mk_mode: who prepares the batch of an iteration */
+  int max_tokens_per_request;   /* prompt tokens one request may ingest per iteration; 0 => 8, the reference's default for
+                                   AMD (MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124); at most 64 */
   int reserved0;
   int32_t *step;                /* [total_num_requests] */
   int64_t *tokens;              /* [total_num_requests, max_seq_length] */
@@ -83,7 +95,7 @@ int mk_graph_destroy(mk_graph *g);
 int mk_tensor_attach(mk_graph *g, void *device_ptr, int ndims, const int64_t *dims, const int64_t *strides, int dtype,
                      const char *name);
 /* Replaces new_input + attach_cuda_tensor / attach_nvshmem_tensor (core.pyx:951-965): the library allocates
- * (zero-filled) device memory at mk_compile. */
+ * zero-filled device memory right away (later tasks capture its address) and frees it in mk_graph_destroy. */
 int mk_tensor_new(mk_graph *g, int ndims, const int64_t *dims, const int64_t *strides, int dtype, const char *name,
                   int io_category);
 /* Replaces Graph::shuffle_tensors / fuse_tensors (src/kernel/graph.cc:398-437).  The result is a *view*:
@@ -116,7 +128,8 @@ int mk_compile(mk_graph *g);
  * same handle can serve `tokens` again. */
 int mk_init_requests(mk_graph *g);
 /* Replaces launch_persistent_kernel (persistent_kernel.cuh:2260-2329): one cooperative launch that runs until all
- * requests are finished.  Blocks until the kernel has drained, like the reference. `stream` is a hipStream_t (may be 0). */
+ * requests are finished (offline / online modes) or over the one batch the host described (online_notoken / onepass).
+ * Blocks until the kernel has drained, like the reference. `stream` is a hipStream_t (may be 0). */
 int mk_launch(mk_graph *g, void *stream);
 /* Same kernel, but returns after at most `max_iterations` decode iterations; scheduler state persists in HBM so the
  * next call continues where this one stopped (the reference has no counterpart: its TPOT is an average over one whole

@@ -3,7 +3,8 @@
 Nothing in the product (fleet-chiplet-megakernel_amd/) may import this module; only tests/,
 __graft_entry__.smoke() and bench.py's cpu_baseline leg do, as the checker.
 
-Two restatements of the reference's decode mathematics, written against plain torch CPU ops:
+Two restatements of the reference's decode mathematics, written against plain torch CPU ops (plus order="f64", the
+same model definition evaluated in float64 without intermediate rounding: the yardstick the two are measured against):
 
 * order="torch"  -- the reference's PyTorch model (demo/qwen3/models/modeling_qwen3.py), which is what
   its greedy loop runs (demo/qwen3/demo.py:1193-1230): every op on bf16 tensors with a bf16 rounding
@@ -292,14 +293,14 @@ def rope_t(x, cos_row, sin_row):
 class KVCache:
     """Contiguous per-request cache [layers, max_seq, nkv, D] (the reference's torch path uses one page)."""
 
-    def __init__(self, cfg: Qwen3Config, max_seq: int):
-        self.k = torch.zeros(cfg.num_layers, max_seq, cfg.num_kv_heads, cfg.head_dim, dtype=BF16)
+    def __init__(self, cfg: Qwen3Config, max_seq: int, dtype=BF16):
+        self.k = torch.zeros(cfg.num_layers, max_seq, cfg.num_kv_heads, cfg.head_dim, dtype=dtype)
         self.v = torch.zeros_like(self.k)
 
 
 class Qwen3Oracle:
     def __init__(self, cfg: Qwen3Config, weights: dict, order: str = "kernel"):
-        assert order in ("kernel", "torch")
+        assert order in ("kernel", "torch", "f64")
         self.cfg, self.w, self.order = cfg, weights, order
         self.cos, self.sin = rope_tables(cfg)
         self.route_margins = []  # mixture of experts: smallest routing gap of every layer call since the last forward()
@@ -328,6 +329,8 @@ class Qwen3Oracle:
                 return moe_mlp_k(h, x, W["gate_up_proj"], W["down_proj"], wts, exp)[0]
             m = linear_silu_k(h, W["gate_proj"], W["up_proj"])
             return linear_k(m, W["down_proj"], res=x)
+        if self.order == "f64":
+            return self._layer_f64(li, x, cache, pos0)
         # torch order
         h = rmsnorm_t(x, W["input_norm"])
         q, k, v = F.linear(h, W["q_proj"]), F.linear(h, W["k_proj"]), F.linear(h, W["v_proj"])
@@ -352,34 +355,47 @@ class Qwen3Oracle:
         m = F.silu(F.linear(h, W["gate_proj"])) * F.linear(h, W["up_proj"])
         return x + F.linear(m, W["down_proj"])
 
+    def _layer_f64(self, li: int, x, cache, pos0: int):
+        """The dense layer's definition evaluated in float64 with no intermediate rounding (the same bf16 weights and
+        cos/sin tables, eps as the kernels): the yardstick both rounding orders are measured against.  `cache` must be a
+        KVCache created with dtype=torch.float64."""
+        cfg, W = self.cfg, {k: v.double() for k, v in self.w["layers"][li].items()}
+        assert cfg.num_experts == 0
+        T, D, nq, nkv = x.shape[0], cfg.head_dim, cfg.num_q_heads, cfg.num_kv_heads
+        pos = torch.arange(pos0, pos0 + T)
+        cos, sin = self.cos[pos][:, None, :].double(), self.sin[pos][:, None, :].double()
+        norm = lambda v, w: v * torch.rsqrt(v.pow(2).mean(-1, keepdim=True) + cfg.rms_eps) * w
+        h = norm(x, W["input_norm"])
+        q, k, v = h @ W["q_proj"].t(), h @ W["k_proj"].t(), h @ W["v_proj"].t()
+        q = rope_t(norm(q.view(T, nq, D), W["q_norm"]), cos, sin)
+        k = rope_t(norm(k.view(T, nkv, D), W["k_norm"]), cos, sin)
+        cache.k[li, pos0:pos0 + T] = k
+        cache.v[li, pos0:pos0 + T] = v.view(T, nkv, D)
+        outs = []
+        for t in range(T):
+            L = pos0 + t + 1
+            Kf = cache.k[li, :L].permute(1, 0, 2).repeat_interleave(nq // nkv, 0)  # [nq, L, D]
+            Vf = cache.v[li, :L].permute(1, 0, 2).repeat_interleave(nq // nkv, 0)
+            p = torch.softmax(torch.einsum("hd,hld->hl", q[t], Kf) / math.sqrt(D), -1)
+            outs.append(torch.einsum("hl,hld->hd", p, Vf).reshape(nq * D))
+        x = x + torch.stack(outs) @ W["o_proj"].t()
+        h = norm(x, W["post_norm"])
+        g, u = h @ W["gate_proj"].t(), h @ W["up_proj"].t()
+        return x + (g / (1.0 + torch.exp(-g)) * u) @ W["down_proj"].t()
+
     def forward(self, ids, cache: KVCache, pos0: int):
-        """ids: [T] int64 tokens of one request at positions pos0.. -> logits [T, vocab] bf16."""
+        """ids: [T] int64 tokens of one request at positions pos0.. -> logits [T, vocab] bf16 (float64 for order "f64")."""
         x = self.w["embed"][ids]
         self.route_margins = []
+        if self.order == "f64":
+            x = x.double()
+            for li in range(self.cfg.num_layers):
+                x = self._layer_f64(li, x, cache, pos0)
+            x = x * torch.rsqrt(x.pow(2).mean(-1, keepdim=True) + self.cfg.rms_eps) * self.w["final_norm"].double()
+            return x @ self.w["lm_head"].double().t()
         for li in range(self.cfg.num_layers):
             x = self.layer(li, x, cache, pos0)
         if self.order == "kernel":
             h = rmsnorm_k(x, self.w["final_norm"], self.cfg.rms_eps)
             return linear_k(h, self.w["lm_head"])
         return F.linear(rmsnorm_t(x, self.w["final_norm"]), self.w["lm_head"])
-
-    def greedy(self, prompt, n_new: int, max_seq: int, teacher=None, token_by_token_prefill=False):
-        """Prefill then greedy decode (demo.py:1193-1212).  Returns (tokens [len+n_new], logits per decode step).
-        teacher: optional ids to force-feed instead of the argmax (teacher forcing)."""
-        cache = KVCache(self.cfg, max_seq)
-        P = prompt.shape[0]
-        toks = prompt.tolist()
-        logits_out = []
-        if token_by_token_prefill:
-            for p in range(P):
-                lg = self.forward(prompt[p:p + 1], cache, p)
-        else:
-            lg = self.forward(prompt, cache, 0)[-1:]
-        for i in range(n_new):
-            logits_out.append(lg[0])
-            nxt = int(argmax_k(lg)[0]) if self.order == "kernel" else int(lg[0].argmax(-1))
-            toks.append(nxt)
-            feed = nxt if teacher is None else int(teacher[i])
-            if i + 1 < n_new:
-                lg = self.forward(torch.tensor([feed]), cache, P + i)
-        return torch.tensor(toks), logits_out

@@ -245,3 +245,193 @@ def test_lowering_rejects_bad_moe_graphs():
     mpk.moe_w13_linear_layer(input=n, weight=w, moe_routing_indices=ri, moe_mask=mask, output=y, grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
     with pytest.raises(_capi.MkError, match=r"input must be \[tokens, 264\]"):
         mpk.describe_program()
+
+
+def _attn_tensors(mpk, nq=8, nkv=2, D=128, chunks=1, pages=8):
+    t = dict(qkv=_t(mpk, "qkv", 4, (nq + 2 * nkv) * D), kc=_t(mpk, "kc", pages, 16, nkv, D), vc=_t(mpk, "vc", pages, 16, nkv, D), qn=_t(mpk, "qn", D),
+             kn=_t(mpk, "kn", D), cos=_t(mpk, "cos", 64, D), sin=_t(mpk, "sin", 64, D), out=mpk.new_tensor((4, nq * D), name="attn_out"),
+             qws=mpk.new_tensor((4, nq * D), name="qws"))
+    t["lse"] = mpk.new_tensor((4, nkv * chunks * (nq // nkv)), dtype=mi.float32, name="lse")
+    t["oacc"] = mpk.new_tensor((4, nkv * chunks * (nq // nkv) * D), dtype=mi.float32, name="o_acc")
+    return t
+
+
+def test_every_attention_flavour_lowers_to_one_stage():
+    """The reference API has five ways to say "attention" (persistent_kernel.py:724-1180); with or without a KV split in
+    the graph each becomes ONE stage that writes the final bf16 output (the merge task's output when chunks > 1)."""
+    nq, nkv, D = 8, 2, 128
+    kw = dict(q_norm=None, k_norm=None, cos_pos_embed=None, sin_pos_embed=None)
+
+    def program(build):
+        mpk = _host_mpk(B=4, R=2)
+        build(mpk)
+        return [l.split(None, 1)[1] for l in mpk.describe_program().splitlines()]
+
+    def fused(mpk):
+        t = _attn_tensors(mpk)
+        mpk.paged_attention_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], q_norm=t["qn"], k_norm=t["kn"], cos_pos_embed=t["cos"],
+                                  sin_pos_embed=t["sin"], output=t["out"], grid_dim=(2, nkv, 1), block_dim=(128, 1, 1))
+    p = program(fused)
+    assert len(p) == 1 and p[0].startswith("ATTN qkv -> attn_out") and "norm=1 rope=1" in p[0]
+
+    def split(mpk):
+        t = _attn_tensors(mpk)
+        lse3 = mpk.new_tensor((4, 3 * (nq // nkv), nkv), dtype=mi.float32, name="lse3")
+        tmp3 = mpk.new_tensor((4, 3 * (nq // nkv) * D, nkv), name="tmp3")
+        mpk.paged_attention_split_kv_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], lse=lse3, output=tmp3, attention_params=(nq, 3),
+                                           grid_dim=(2, nkv, 3), block_dim=(128, 1, 1), **kw)
+        mpk.paged_attention_split_kv_merge_layer(lse=lse3, output_tmp=tmp3, output=t["out"], attention_params=(nq, D), grid_dim=(2, nkv, 1),
+                                                 block_dim=(128, 1, 1))
+    p = program(split)
+    assert len(p) == 1 and p[0].startswith("ATTN qkv -> attn_out") and "norm=0 rope=0" in p[0]
+
+    def ck_chunks(mpk):
+        t = _attn_tensors(mpk, chunks=4)
+        mpk.kv_cache_update_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], q_norm=t["qn"], k_norm=t["kn"], cos_pos_embed=t["cos"],
+                                  sin_pos_embed=t["sin"], q_workspace=t["qws"], grid_dim=(2, nkv, 1), block_dim=(256, 1, 1))
+        mpk.paged_attention_ck_fmha_layer(q_workspace=t["qws"], k_cache=t["kc"], v_cache=t["vc"], o_acc=t["oacc"], lse_acc=t["lse"],
+                                          attention_params=(nq, 4, 2), grid_dim=(2, nkv, 4), block_dim=(256, 1, 1))
+        mpk.paged_attention_ck_fmha_merge_layer(lse=t["lse"], output_tmp=t["oacc"], output=t["out"], attention_params=(nq, D, 4, nkv),
+                                                grid_dim=(2, nkv, 1), block_dim=(256, 1, 1))
+    p = program(ck_chunks)
+    assert len(p) == 1 and p[0].startswith("ATTN qkv -> attn_out")
+
+    def gang_chunks(mpk):
+        t = _attn_tensors(mpk, chunks=2)
+        mpk.gang_paged_attention_split_kv_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], q_norm=t["qn"], k_norm=t["kn"],
+                                                cos_pos_embed=t["cos"], sin_pos_embed=t["sin"], lse=t["lse"], output=t["oacc"],
+                                                q_workspace=t["qws"], attention_params=(nq, 2, nq * D))
+        mpk.gang_paged_attention_split_kv_merge_layer(lse=t["lse"], output_tmp=t["oacc"], output=t["out"], attention_params=(nq, D, nkv, 2))
+    p = program(gang_chunks)
+    assert len(p) == 1 and p[0].startswith("ATTN qkv -> attn_out")
+
+    def missing_merge(mpk):
+        t = _attn_tensors(mpk, chunks=2)
+        mpk.gang_paged_attention_split_kv_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], q_norm=t["qn"], k_norm=t["kn"],
+                                                cos_pos_embed=t["cos"], sin_pos_embed=t["sin"], lse=t["lse"], output=t["oacc"],
+                                                q_workspace=t["qws"], attention_params=(nq, 2, nq * D))
+    with pytest.raises(_capi.MkError, match="must be followed by gang_attn_merge_mi300"):
+        program(missing_merge)
+
+    def lone_merge(mpk):
+        t = _attn_tensors(mpk, chunks=2)
+        mpk.gang_paged_attention_split_kv_merge_layer(lse=t["lse"], output_tmp=t["oacc"], output=t["out"], attention_params=(nq, D, nkv, 2))
+    with pytest.raises(_capi.MkError, match="must directly follow"):
+        program(lone_merge)
+
+    def small_cache(mpk):
+        t = _attn_tensors(mpk, pages=4)  # the configuration has 8 pages
+        mpk.gang_paged_attention_split_kv_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], q_norm=t["qn"], k_norm=t["kn"],
+                                                cos_pos_embed=t["cos"], sin_pos_embed=t["sin"], lse=t["lse"], output=t["out"],
+                                                q_workspace=t["qws"], attention_params=(nq, 1, nq * D))
+    with pytest.raises(_capi.MkError, match="fewer than max_num_pages"):
+        program(small_cache)
+    m = _host_mpk()
+    with pytest.raises(NotImplementedError, match="speculative"):
+        m.single_batch_extend_attention_layer()
+
+
+def test_split_k_pair_and_fused_activation_lower_to_linear_stages():
+    """The reference's model builder for this GPU family (mpk/models/qwen3/builder.py:395-420,560-585,700-712) writes QKV
+    and o_proj as splitk_linear into an fp32 workspace + splitk_reduce, and the MLP tail as silu_mul_linear_with_residual."""
+    mpk = _host_mpk(B=4, R=2)
+    H, I = 1024, 1536
+    x, n, nw = mpk.new_tensor((4, H), name="x"), mpk.new_tensor((4, H), name="n"), _t(mpk, "nw", H)
+    W, ws = _t(mpk, "W", H, H), mpk.attach_input(torch.zeros(4 * 4, H, dtype=torch.float32), "splitk_ws")
+    y = mpk.new_tensor((4, H), name="y")
+    mpk.rmsnorm_layer(input=x, weight=nw, output=n, grid_dim=(4, 1, 1), block_dim=(128, 1, 1))
+    mpk.splitk_linear_layer(input=n, weight=W, output=ws, grid_dim=(H // 128, 4, 1), block_dim=(256, 1, 1))
+    mpk.splitk_reduce_layer(workspace=ws, residual=x, output=y, k_splits=4, grid_dim=(H // 128, 1, 1), block_dim=(256, 1, 1))
+    wg, wu = _t(mpk, "wg", I, H), _t(mpk, "wu", I, H)
+    gu = mpk.shuffle_tensors([wg, wu], 0, 6, "gu")  # groups of [gate256 ; up256]
+    mid = mpk.attach_input(torch.zeros(4, 2 * I, dtype=torch.bfloat16), "mlp_mid")
+    wd, out = _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="out")
+    mpk.rmsnorm_layer(input=y, weight=nw, output=n, grid_dim=(4, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_layer(input=n, weight=gu, output=mid, grid_dim=(12, 1, 1), block_dim=(128, 1, 1))
+    mpk.silu_mul_linear_with_residual_layer(input=mid, weight=wd, residual=y, output=out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1))
+    prog = [l.split(None, 1)[1] for l in mpk.describe_program().splitlines()]
+    kinds = [l.split()[0] for l in prog]
+    assert kinds == ["NORM[multi-token", "LINEAR+norm+res", "NORM[multi-token", "LINEAR+norm", "LINEAR+res"]
+    assert "-> y" in prog[1] and "+silu half=256 folded in" in prog[3] and "silu_mul(mlp_mid) x wd -> out" in prog[4] and "k=1536" in prog[4]
+    # a physically interleaved gate/up weight: the producer's grid (one block per half-group) says where gate ends
+    mpk = _host_mpk(B=4, R=2)
+    n, guw = mpk.new_tensor((4, H), name="n"), _t(mpk, "gu", 2 * I, H)
+    mid, wd, y, out = mpk.new_tensor((4, 2 * I), name="mid"), _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="out")
+    mpk.linear_layer(input=n, weight=guw, output=mid, grid_dim=(24, 1, 1), block_dim=(128, 1, 1))
+    mpk.silu_mul_linear_with_residual_layer(input=mid, weight=wd, residual=y, output=out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1))
+    prog = mpk.describe_program()
+    assert "+silu half=128 folded in" in prog
+    # an input of unknown origin is read as [gate | up] halves by a standalone activation stage
+    mpk = _host_mpk(B=4, R=2)
+    mid, wd, y, out = _t(mpk, "mid", 4, 2 * I), _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="out")
+    mpk.silu_mul_linear_with_residual_layer(input=mid, weight=wd, residual=y, output=out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1))
+    kinds = [l.split()[1] for l in mpk.describe_program().splitlines()]
+    assert kinds == ["SILU_MUL", "LINEAR+res"]
+    # a lone split-K linear into a workspace, or a lone reduce, is an error
+    mpk = _host_mpk(B=4, R=2)
+    mpk.splitk_linear_layer(input=mpk.new_tensor((4, H), name="n"), weight=_t(mpk, "W", H, H),
+                            output=mpk.attach_input(torch.zeros(16, H, dtype=torch.float32), "ws"), grid_dim=(8, 4, 1), block_dim=(256, 1, 1))
+    with pytest.raises(_capi.MkError, match="must be followed by splitk_reduce_mi300"):
+        mpk.describe_program()
+
+
+def test_modes_and_configuration_limits():
+    meta = make_meta(2, 64, 4, 2, 8, device="cpu")
+    kw = dict(world_size=1, mpi_rank=0, num_workers=256, num_local_schedulers=0, num_remote_schedulers=0, max_seq_length=64,
+              max_num_batched_requests=2, max_num_batched_tokens=4, max_num_pages=8, page_size=16, meta_tensors=meta, profiler_tensor=None,
+              trace_name=None, spec_decode_config=None, use_cutlass_kernel=False)
+    for mode in ("offline", "online", "online_notoken", "onepass"):
+        assert mi.PersistentKernel(mode=mode, **kw).mode == mode
+    with pytest.raises(NotImplementedError, match="multi_turn"):
+        mi.PersistentKernel(mode="multi_turn", **kw)
+    assert mi.PersistentKernel(mode="offline", **kw).max_tokens_per_request == 8  # the reference's default on AMD
+    assert mi.PersistentKernel(mode="offline", max_tokens_per_request=64, **kw).max_tokens_per_request == 64
+    with pytest.raises(_capi.MkError, match="max_tokens_per_request"):
+        mi.PersistentKernel(mode="offline", max_tokens_per_request=65, **kw)
+    # two requests of up to 4 pages each need 8 pages: the page ring hands pages out without checking
+    with pytest.raises(_capi.MkError, match="cannot back 2 concurrent requests"):
+        mi.PersistentKernel(mode="offline", **{**kw, "max_num_pages": 7, "meta_tensors": make_meta(2, 64, 4, 2, 7, device="cpu")})
+    # tensor id -1 is accepted only for the optional operands of the attention tasks
+    mpk = _host_mpk()
+    x, W = _t(mpk, "x", 4, 1024), _t(mpk, "W", 512, 1024)
+    with pytest.raises(_capi.MkError, match="bad tensor id -1"):
+        mpk._task("linear", (8, 1, 1), (128, 1, 1), [(x, (-1, -1, -1), 1), (W, (0, -1, -1), 1), (None, (1, -1, -1), -1)])
+
+
+def test_barrier_counter_comparison_survives_wraparound(tmp_path):
+    """The grid barrier compares a 32-bit arrival counter with quota x epoch; both wrap after 2^32 arrivals (about half
+    an hour of single-token decode in one launch).  The comparison must stay correct across the wrap."""
+    import subprocess
+    src = tmp_path / "wrap.cpp"
+    src.write_text(r'''
+#include <cstdio>
+#include <initializer_list>
+#include "mk_types.h"
+int main() {
+  const unsigned quota = 32;
+  int bad = 0;
+  // epochs around the wrap of quota * epoch (2^27 epochs), and far beyond it
+  for (unsigned long long e0 : {1ull, (1ull << 27) - 3, (1ull << 27), (1ull << 28) + 5, (1ull << 32) - 2, (1ull << 33) + 7}) {
+    for (unsigned long long e = e0; e < e0 + 6; e++) {
+      const unsigned target = quota * (unsigned)e;              // what the kernel computes (wraps)
+      const unsigned long long arrived_full = 32ull * e;         // every workgroup has arrived
+      for (int missing = 0; missing <= 32; missing += 8) {
+        const unsigned counter = (unsigned)(arrived_full - missing);
+        const bool expect = missing == 0;
+        if (mk_counter_reached(counter, target) != expect) bad++;
+      }
+      // a die that is already one stage ahead must also read as "reached"
+      if (!mk_counter_reached((unsigned)(arrived_full + 32), target)) bad++;
+    }
+  }
+  // the plain comparison is what fails: counter just below 2^32, target wrapped to a small number
+  if ((0xFFFFFFE0u >= 0x00000020u) == mk_counter_reached(0xFFFFFFE0u, 0x00000020u)) bad++;
+  printf("%d\n", bad);
+  return bad != 0;
+}
+''')
+    exe = tmp_path / "wrap"
+    inc = os.path.join(os.path.dirname(os.path.dirname(os.path.abspath(__file__))), "fleet-chiplet-megakernel_amd", "csrc")
+    subprocess.run(["g++", "-std=c++17", "-O1", "-I", inc, str(src), "-o", str(exe)], check=True)
+    res = subprocess.run([str(exe)], capture_output=True, text=True)
+    assert res.returncode == 0 and res.stdout.strip() == "0", res.stdout

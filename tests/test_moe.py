@@ -222,13 +222,14 @@ def test_moe_bs1_greedy_matches_oracle_teacher_forced(mode):
     dec.mpk.finalize()
 
 
-def test_moe_batched_decode_continuous_batching():
-    """BS=4 with six requests of different prompt lengths (chunked prompt ingestion, slot reuse): every generated token must be
-    the oracle's argmax wherever the oracle's margin exceeds 0.05."""
+@pytest.mark.parametrize("B,R_total", [(4, 6), (32, 40)])
+def test_moe_batched_decode_continuous_batching(B, R_total):
+    """BS=4 with six / BS=32 with forty requests of different prompt lengths (chunked prompt ingestion, slot reuse): every
+    generated token must be the oracle's argmax wherever the oracle's margin exceeds 0.05."""
     from oracle.qwen3_ref import KVCache, Qwen3Oracle, argmax_k, make_model_weights, make_prompt
     cfg = _moe_cfg()
     w = make_model_weights(cfg, seed=12)
-    max_seq, R_total, B = 30, 6, 4
+    max_seq = 30
     prompts = [make_prompt(cfg, 3 + (4 * r) % 11, 50 + r) for r in range(R_total)]
     dec = _decoder(cfg, w, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=16, total_requests=R_total)
     toks, steps = dec.generate(prompts)
@@ -248,6 +249,6 @@ def test_moe_batched_decode_continuous_batching():
                 hits += 1
             if p + 1 < max_seq:
                 lg = orc.forward(torch.tensor([tk[p]]), cache, p)
-    assert hits >= 5
+    assert hits >= 5 * (R_total // 6)
     assert dec.mpk.stats()["aborted"] == 0
     dec.mpk.finalize()
