@@ -103,7 +103,8 @@ def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
         assert prefill_iters < 10 * P * B, "prompt ingestion did not finish"
     if W > 0:
         dec.mpk.run_steps(W)
-    ctx0 = int(dec.meta["step"].min().item())  # cached positions per request at the first timed step
+    steps0 = dec.meta["step"].cpu().tolist()   # cached positions of every request at the first timed step (requests that
+    ctx0, ctx0_max = min(steps0), max(steps0)  # ingested their prompt earlier are further along: prompts enter 8 requests at a time)
     stream = torch.cuda.current_stream()
     torch.cuda.synchronize()
     t0 = time.perf_counter()
@@ -113,25 +114,25 @@ def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
     t1 = time.perf_counter()
     st = dec.mpk.stats()
     assert not finished, "requests finished inside the timed region; lower --steps"
-    assert int(dec.meta["step"].min().item()) == ctx0 + K and int(dec.meta["step"].max().item()) == ctx0 + K, "timed region did not run exactly K decode steps"
+    assert dec.meta["step"].cpu().tolist() == [s0 + K for s0 in steps0], "timed region did not run exactly K decode steps for every request"
     wall_ms = (t1 - t0) * 1e3
     kernel_ms = st["last_launch_ms"]
     ms_per_step = wall_ms / K
     # algorithmic bytes: weights once per step + K/V rows of every cached position (positions ctx0+1 .. ctx0+K incl. the new one)
-    kv_positions = sum(ctx0 + 1 + i for i in range(K))
+    kv_positions = sum(s0 + 1 + i for s0 in steps0 for i in range(K))  # summed over the requests
     # mixture of experts: a step streams the experts its tokens select; B tokens choosing top-k of E uniformly touch
     # E * (1 - (1 - k/E)^B) distinct experts per layer in expectation (exactly k for one token)
     moe = shape.num_experts > 0
     distinct = None
     if moe and B > 1:
         distinct = shape.num_experts * (1.0 - (1.0 - shape.num_experts_per_tok / shape.num_experts) ** B)
-    bytes_total = int(K * shape.weight_bytes_per_token(distinct) + B * kv_positions * shape.kv_bytes_per_position())
+    bytes_total = int(K * shape.weight_bytes_per_token(distinct) + kv_positions * shape.kv_bytes_per_position())
     achieved = bytes_total / (kernel_ms * 1e-3) / 1e9
     per_step = MEASURED_TRAFFIC_BYTES_PER_STEP.get((model, B))
     return {
         "batch": B, "ms_per_step": round(ms_per_step, 4), "tokens_per_s": round(B * 1e3 / ms_per_step, 1), "steps": K, "warmup": W,
         "workload": f"{'Qwen3-30B-A3B (128 experts, top-8)' if moe else 'Qwen3-8B'} shape, {shape.num_layers} layers, vocab {shape.vocab_size}, BS={B}, prompt {P}, "
-                    f"context {ctx0}..{ctx0 + K}, max_seq_len {max_seq}, page_size 4096, graph mode {mode}",
+                    f"context {ctx0}..{ctx0_max + K}, max_seq_len {max_seq}, page_size 4096, graph mode {mode}",
         "prefill_iterations": prefill_iters,
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": None if per_step is None else int(per_step * K),
@@ -175,7 +176,7 @@ def main():
     shape = Qwen3Shape.qwen3_30b_a3b(min(args.layers, 48) if args.layers != 36 else 48) if moe else Qwen3Shape(num_layers=args.layers)
     K, W, P = args.steps, args.warmup, args.prompt_length
     batches = [args.batch] if args.batch else ([1, 64] if not moe else [1])
-    max_seq = max(1200, P + W + K + 2)
+    max_seq = max(1200, P + W + K + 2 + 16)
     if args.calib_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)

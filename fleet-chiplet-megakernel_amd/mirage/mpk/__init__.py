@@ -1,5 +1,7 @@
 """MPK (persistent kernel) front end."""
 from .persistent_kernel import PersistentKernel
+from .mpk import MPK, MPKMetadata
+from .models import MirageModelConfig
 
 
 def spec_decode_class(method, **kwargs):

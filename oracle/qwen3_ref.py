@@ -30,9 +30,11 @@ pipelines (third-party, absent from the tree); both restatements accumulate in f
 Mixture of experts (Qwen3-30B-A3B shape): moe_route_k / moe_mlp_k restate the reference's MoE task kernels
 (moe_topk_softmax_mi300.cuh, moe_linear_mi300.cuh, moe_mul_sum_add_mi300.cuh) and are pinned against float64
 softmax + torch.topk, planted ties, a dense float64 evaluation of the same experts, and the E=1 special case that
-reduces to the dense SwiGLU MLP.  moe_block_t restates HF transformers' Qwen3MoeSparseMoeBlock (third-party,
-pinned 4.57.1 in the reference's requirements, not importable here at that version): PARITY UNPINNED beyond
-agreeing with moe_mlp_k within bf16 tolerance.
+reduces to the dense SwiGLU MLP.  moe_block_t restates HF transformers' Qwen3MoeSparseMoeBlock (third-party; the
+reference pins 4.57.1, which is not importable here): tests/test_oracle_vs_hf.py checks it against that block of the
+installed transformers 5.x on the same bf16 inputs, and checks the dense model composition (order "f64") against
+transformers' Qwen3ForCausalLM evaluated in float64; what stays unpinned is only that the pinned 4.57.1 block rounds
+at the same points as the 5.x one.
 """
 import math
 from dataclasses import dataclass
@@ -131,10 +133,12 @@ def rmsnorm_k(x, w, eps=1e-6):
     return ((xf * r) * w.float()).to(BF16)
 
 
-def linear_k(x, W, res=None):
-    y = x.float() @ W.float().t()
+def linear_k(x, W, res=None, acc=torch.float32):
+    """bf16(x W^T [+ res]) accumulated in `acc` (fp32: what the kernels do; float64: the same rounding points with exact
+    sums, used to measure how far two legitimate summation orders drift apart through a deep model)."""
+    y = x.to(acc) @ W.to(acc).t()
     if res is not None:
-        y = y + res.float()
+        y = y + res.to(acc)
     return y.to(BF16)
 
 
@@ -142,9 +146,9 @@ def silu_mul_f32(g, u):
     return g / (1.0 + torch.exp(-g)) * u
 
 
-def linear_silu_k(x, Wg, Wu):
-    xf = x.float()
-    return silu_mul_f32(xf @ Wg.float().t(), xf @ Wu.float().t()).to(BF16)
+def linear_silu_k(x, Wg, Wu, acc=torch.float32):
+    xf = x.to(acc)
+    return silu_mul_f32(xf @ Wg.to(acc).t(), xf @ Wu.to(acc).t()).to(BF16)
 
 
 def silu_mul_k(gate_bf16, up_bf16):
@@ -299,10 +303,13 @@ class KVCache:
 
 
 class Qwen3Oracle:
-    def __init__(self, cfg: Qwen3Config, weights: dict, order: str = "kernel"):
+    def __init__(self, cfg: Qwen3Config, weights: dict, order: str = "kernel", rope=None, acc=torch.float32):
+        """rope: optional (cos, sin) tables [positions, head_dim] replacing the bf16 ones (the float64 order can be given
+        unrounded tables to be compared with an independent float64 evaluation).  acc: accumulation type of the
+        kernel-order linears (see linear_k)."""
         assert order in ("kernel", "torch", "f64")
-        self.cfg, self.w, self.order = cfg, weights, order
-        self.cos, self.sin = rope_tables(cfg)
+        self.cfg, self.w, self.order, self.acc = cfg, weights, order, acc
+        self.cos, self.sin = rope if rope is not None else rope_tables(cfg)
         self.route_margins = []  # mixture of experts: smallest routing gap of every layer call since the last forward()
 
     # one decoder layer on T new tokens of ONE request at absolute positions pos0..pos0+T-1
@@ -313,22 +320,23 @@ class Qwen3Oracle:
         pos = torch.arange(pos0, pos0 + T)
         cos, sin = self.cos[pos][:, None, :], self.sin[pos][:, None, :]
         if self.order == "kernel":
+            acc = self.acc
             h = rmsnorm_k(x, W["input_norm"], cfg.rms_eps)
-            q, k, v = linear_k(h, W["q_proj"]), linear_k(h, W["k_proj"]), linear_k(h, W["v_proj"])
+            q, k, v = linear_k(h, W["q_proj"], acc=acc), linear_k(h, W["k_proj"], acc=acc), linear_k(h, W["v_proj"], acc=acc)
             q = head_norm_rope_k(q.view(T, nq, D), W["q_norm"], cos, sin, cfg.rms_eps)
             k = head_norm_rope_k(k.view(T, nkv, D), W["k_norm"], cos, sin, cfg.rms_eps)
             cache.k[li, pos0:pos0 + T] = k
             cache.v[li, pos0:pos0 + T] = v.view(T, nkv, D)
             a = torch.stack([attention_k(q[t], cache.k[li, :pos0 + t + 1], cache.v[li, :pos0 + t + 1]) for t in range(T)])
-            x = linear_k(a.view(T, nq * D), W["o_proj"], res=x)
+            x = linear_k(a.view(T, nq * D), W["o_proj"], res=x, acc=acc)
             h = rmsnorm_k(x, W["post_norm"], cfg.rms_eps)
             if cfg.num_experts > 0:
-                gate = linear_k(h, W["router"])
+                gate = linear_k(h, W["router"], acc=acc)
                 self.route_margins.append(float(moe_route_margin(gate, cfg.num_experts_per_tok).min()))
                 wts, exp = moe_route_k(gate, cfg.num_experts_per_tok)
                 return moe_mlp_k(h, x, W["gate_up_proj"], W["down_proj"], wts, exp)[0]
-            m = linear_silu_k(h, W["gate_proj"], W["up_proj"])
-            return linear_k(m, W["down_proj"], res=x)
+            m = linear_silu_k(h, W["gate_proj"], W["up_proj"], acc=acc)
+            return linear_k(m, W["down_proj"], res=x, acc=acc)
         if self.order == "f64":
             return self._layer_f64(li, x, cache, pos0)
         # torch order
@@ -397,5 +405,6 @@ class Qwen3Oracle:
             x = self.layer(li, x, cache, pos0)
         if self.order == "kernel":
             h = rmsnorm_k(x, self.w["final_norm"], self.cfg.rms_eps)
-            return linear_k(h, self.w["lm_head"])
+            self.last_hidden = h  # the normalised final hidden state of the last forward()
+            return linear_k(h, self.w["lm_head"], acc=self.acc)
         return F.linear(rmsnorm_t(x, self.w["final_norm"]), self.w["lm_head"])
