@@ -109,6 +109,8 @@ struct mk_graph {
   std::string json, program_text;
   hipEvent_t ev0 = nullptr, ev1 = nullptr;
   bool launch_pending = false;
+  MkSync *pending_sync = nullptr;  // barrier state of the pending / last launch (the graph's own or the static scratch)
+  int max_kv_heads = 1, max_qpk = 1;  // over the attention stages
   double last_ms = 0.0;
   int last_nxcd = 0, last_aborted = 0;
   int64_t weight_bytes = 0;
@@ -1031,17 +1033,20 @@ int upload_runtime(mk_graph *g) {
   return MK_OK;
 }
 
-int do_launch(mk_graph *g, hipStream_t stream, int max_iters, int run_scheduler) {
+// `rt` is the runtime block the kernel receives by value; `cleared_by_caller`: its barrier state has been zeroed already
+int do_launch(mk_graph *g, hipStream_t stream, int max_iters, int run_scheduler, const MkRuntime *rt = nullptr, bool cleared_by_caller = false) {
   if (!g->compiled) return fail(MK_ESTATE, "mk_compile has not been called");
   if (g->launch_pending) return fail(MK_ESTATE, "a launch is still pending: call mk_wait first");
   HIP_TRY(hipSetDevice(g->cfg.device));
-  HIP_TRY(hipMemsetAsync(g->d_sync, 0, sizeof(MkSync), stream));
+  if (!rt) rt = &g->h_rt;
+  if (!cleared_by_caller) HIP_TRY(hipMemsetAsync(rt->sync, 0, sizeof(MkSync), stream));
   const MkRuntime *rtp = g->d_rt;
-  void *args[] = {(void *)&g->h_rt, (void *)&rtp, (void *)&max_iters, (void *)&run_scheduler};
+  void *args[] = {(void *)rt, (void *)&rtp, (void *)&max_iters, (void *)&run_scheduler};
   HIP_TRY(hipEventRecord(g->ev0, stream));
   HIP_TRY(hipLaunchCooperativeKernel((const void *)mk_persistent_kernel, dim3(g->G), dim3(MK_THREADS), args, MK_LDS_BYTES, stream));
   HIP_TRY(hipEventRecord(g->ev1, stream));
   g->launch_pending = true;
+  g->pending_sync = rt->sync;
   return MK_OK;
 }
 
@@ -1053,7 +1058,7 @@ int do_wait(mk_graph *g, hipStream_t stream, int *finished_out) {
   HIP_TRY(hipEventElapsedTime(&ms, g->ev0, g->ev1));
   g->last_ms = ms;
   MkSync hs;
-  HIP_TRY(hipMemcpy(&hs, g->d_sync, sizeof(MkSync), hipMemcpyDeviceToHost));
+  HIP_TRY(hipMemcpy(&hs, g->pending_sync ? g->pending_sync : g->d_sync, sizeof(MkSync), hipMemcpyDeviceToHost));
   int nx = 0;
   for (int i = 0; i < MK_MAX_XCD; i++) nx += hs.xcd_count[i] > 0;
   g->last_nxcd = nx;
@@ -1063,6 +1068,50 @@ int do_wait(mk_graph *g, hipStream_t stream, int *finished_out) {
   if (finished_out) *finished_out = sc.finished;
   if (hs.abort_flag) return fail(MK_EABORT, "kernel watchdog fired (barrier epoch %u): a workgroup waited longer than the spin limit", hs.abort_where);
   return MK_OK;
+}
+
+// ---- launch scratch that no call allocates -------------------------------------------------------------------
+// mk_enqueue_steps_static runs a compiled graph with every piece of launch scratch -- the grid barrier's counters, the
+// K-split partial tiles and their arrival counters, the attention stages' split-KV partials and counters, the
+// sampling stages' per-workgroup partials -- taken from this file-scope device array instead of from the buffers
+// mk_compile allocated.  Each GPU the library runs on holds its own copy of the array until the process ends.
+// Sizes are for the largest launch the entry point accepts (256 workgroups, 64 tokens x 8 kv heads, 8 q heads per kv head).
+constexpr size_t align256(size_t n) { return (n + 255) / 256 * 256; }
+constexpr int MK_STATIC_MAX_WG = 256;
+constexpr int MK_STATIC_MAX_ITEMS = MK_MAX_TOKENS * 8;  // (token, kv head) pairs
+constexpr int MK_STATIC_MAX_QPK = 8;
+constexpr size_t SS_SYNC = 0;
+constexpr size_t SS_SPLITK_CNT = SS_SYNC + align256(sizeof(MkSync));
+constexpr size_t SS_ATTN_CNT = SS_SPLITK_CNT + align256((size_t)MK_STATIC_MAX_WG * 32 * sizeof(unsigned));
+constexpr size_t SS_CLEARED_END = SS_ATTN_CNT + align256((size_t)MK_STATIC_MAX_ITEMS * 32 * sizeof(unsigned));  // [0, here) starts every call at zero
+constexpr size_t SS_ARGMAX_PV = SS_CLEARED_END;
+constexpr size_t SS_ARGMAX_PI = SS_ARGMAX_PV + align256((size_t)MK_MAX_TOKENS * MK_STATIC_MAX_WG * sizeof(float));
+constexpr size_t SS_ATTN_PART = SS_ARGMAX_PI + align256((size_t)MK_MAX_TOKENS * MK_STATIC_MAX_WG * sizeof(int));
+constexpr size_t SS_SPLITK_PART = SS_ATTN_PART + align256((size_t)(MK_STATIC_MAX_ITEMS + MK_ATTN_MAX_CHUNKS) * MK_STATIC_MAX_QPK * MK_ATTN_PSTRIDE * sizeof(float));
+constexpr size_t MK_STATIC_SCRATCH_BYTES = SS_SPLITK_PART + (size_t)MK_STATIC_MAX_WG * 4 * 4 * 4 * 64 * 16;  // about 19.7 MB
+
+static __device__ __align__(256) unsigned char scratch[MK_STATIC_SCRATCH_BYTES];
+
+constexpr int MK_MAX_DEVICES = 64;
+unsigned char *g_scratch_ptr[MK_MAX_DEVICES];  // device address of `scratch` on each device, resolved once per device
+
+// `scratch` is a host-side stand-in in host code, not a device address: the address every kernel argument, fill and
+// copy uses is the one hipGetSymbolAddress returns, asked for once per device with that device current.
+int resolve_scratch(int device) {
+  if (device < 0 || device >= MK_MAX_DEVICES) return fail(MK_EINVAL, "device %d outside [0, %d)", device, MK_MAX_DEVICES);
+  if (g_scratch_ptr[device]) return MK_OK;
+  HIP_TRY(hipSetDevice(device));
+  void *p = nullptr;
+  HIP_TRY(hipGetSymbolAddress(&p, HIP_SYMBOL(scratch)));
+  if (!p) return fail(MK_EHIP, "hipGetSymbolAddress returned a null address for the launch scratch");
+  g_scratch_ptr[device] = (unsigned char *)p;
+  return MK_OK;
+}
+
+// zero-fill by kernel (a fill node that a caller's graph capture records safely, unlike a memset node)
+__global__ void mk_fill_zero_kernel(uint4 *p, size_t n16) {
+  const uint4 z = {0u, 0u, 0u, 0u};
+  for (size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (size_t)gridDim.x * blockDim.x) p[i] = z;
 }
 
 }  // namespace
@@ -1344,7 +1393,11 @@ int mk_compile(mk_graph *g) {
   // counters (device scope / die-local), one 128-byte line per (token, kv head)
   int max_kv = 1;
   for (auto &s : g->stages)
-    if (s.op == MK_OP_ATTN && s.num_kv_heads > max_kv) max_kv = s.num_kv_heads;
+    if (s.op == MK_OP_ATTN) {
+      if (s.num_kv_heads > max_kv) max_kv = s.num_kv_heads;
+      g->max_qpk = std::max(g->max_qpk, s.num_q_heads / s.num_kv_heads);
+    }
+  g->max_kv_heads = max_kv;
   g->attn_cnt_n = (size_t)rt.max_tokens * max_kv * 32 * 2;
   if ((rc = dev_alloc(g, &p, sizeof(unsigned) * g->attn_cnt_n))) return rc;
   rt.attn_cnt = (unsigned *)p;
@@ -1376,6 +1429,7 @@ int mk_compile(mk_graph *g) {
   if ((rc = upload_runtime(g))) return rc;
   HIP_TRY(hipEventCreate(&g->ev0));
   HIP_TRY(hipEventCreate(&g->ev1));
+  if ((rc = resolve_scratch(g->cfg.device))) return rc;  // set-up is where the static launch scratch's address is looked up
   g->compiled = true;
   return mk_init_requests(g);
 }
@@ -1411,6 +1465,36 @@ int mk_enqueue_steps(mk_graph *g, void *stream, int max_iterations) {
     case MK_MODE_ONLINE: return do_launch(g, (hipStream_t)stream, max_iterations, MK_SCHED_ONLINE);
     default: return do_launch(g, (hipStream_t)stream, 1, MK_SCHED_FROM_META);  // the host's batch is run once
   }
+}
+
+int mk_enqueue_steps_static(mk_graph *g, void *stream, int max_iterations) {
+  if (!g) return fail(MK_EINVAL, "null argument");
+  if (!g->compiled) return fail(MK_ESTATE, "mk_compile has not been called");
+  if (max_iterations < 1) return fail(MK_EINVAL, "max_iterations must be positive");
+  if (g->G > MK_STATIC_MAX_WG) return fail(MK_EINVAL, "the static launch scratch holds %d workgroups, this graph runs %d", MK_STATIC_MAX_WG, g->G);
+  if (g->h_rt.max_tokens * g->max_kv_heads > MK_STATIC_MAX_ITEMS || g->max_qpk > MK_STATIC_MAX_QPK)
+    return fail(MK_EINVAL, "the static launch scratch holds %d (token, kv head) pairs of up to %d q heads each; this graph needs %d x %d",
+                MK_STATIC_MAX_ITEMS, MK_STATIC_MAX_QPK, g->h_rt.max_tokens * g->max_kv_heads, g->max_qpk);
+  int rc = resolve_scratch(g->cfg.device);  // already resolved by mk_compile on this device; no allocation either way
+  if (rc) return rc;
+  if (g->launch_pending) return fail(MK_ESTATE, "a launch is still pending: call mk_wait first");
+  HIP_TRY(hipSetDevice(g->cfg.device));
+  unsigned char *base = g_scratch_ptr[g->cfg.device];
+  MkRuntime rt = g->h_rt;
+  rt.sync = (MkSync *)(base + SS_SYNC);
+  rt.splitk_cnt = (unsigned *)(base + SS_SPLITK_CNT);
+  rt.attn_cnt = (unsigned *)(base + SS_ATTN_CNT);
+  rt.argmax_pv = (float *)(base + SS_ARGMAX_PV);
+  rt.argmax_pi = (int *)(base + SS_ARGMAX_PI);
+  rt.attn_part = (float *)(base + SS_ATTN_PART);
+  rt.splitk_part = base + SS_SPLITK_PART;
+  rt.stage_prof = nullptr;  // per-stage timing is library-allocated scratch too: not recorded by this entry point
+  rt.timing = nullptr;
+  // the array keeps what the previous call left: barrier state and arrival counters must start at zero
+  hipLaunchKernelGGL(mk_fill_zero_kernel, dim3(16), dim3(256), 0, (hipStream_t)stream, (uint4 *)base, SS_CLEARED_END / 16);
+  HIP_TRY(hipGetLastError());
+  const int sched = g->cfg.mode == MK_MODE_OFFLINE ? MK_SCHED_OFFLINE : (g->cfg.mode == MK_MODE_ONLINE ? MK_SCHED_ONLINE : MK_SCHED_FROM_META);
+  return do_launch(g, (hipStream_t)stream, sched == MK_SCHED_FROM_META ? 1 : max_iterations, sched, &rt, true);
 }
 
 int mk_wait(mk_graph *g, void *stream, int *finished_out) {

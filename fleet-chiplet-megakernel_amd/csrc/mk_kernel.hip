@@ -2713,8 +2713,12 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     // die's L2: workgroup-scope atomic, ordinary stores and loads (each stage has its own partial buffer and the L1 is
     // invalidated once per iteration, so a partial is never read from a stale line).  Otherwise device scope.
     const int item = u / cmax;
-    const bool local = c.even_xcds && (item * cmax) / c.quota == (item * cmax + C - 1) / c.quota;
-    float *gpart = (float *)st.aux0 + (size_t)u * QPK * MK_ATTN_PSTRIDE;
+    // (a launch whose attention stages all share one partial buffer -- rt.attn_part -- always takes the device-scope
+    // path: a buffer that is rewritten several times per iteration must not be read through lines an earlier stage left
+    // in the L1)
+    const bool local = !rt.attn_part && c.even_xcds && (item * cmax) / c.quota == (item * cmax + C - 1) / c.quota;
+    float *part_base = rt.attn_part ? rt.attn_part : (float *)st.aux0;
+    float *gpart = part_base + (size_t)u * QPK * MK_ATTN_PSTRIDE;
     uint16_t *orow = (uint16_t *)st.out + (size_t)t * st.ld_out + (size_t)h * QPK * D;
     const int mh = tid / TPH, md = (tid - mh * TPH) * DPT;  // this thread merges dims [md, md+DPT) of head mh
     {
@@ -2764,7 +2768,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       __syncthreads();
       if (*sflag) {
         // every chunk partial is read with independent loads (8 bytes each), sixteen chunks in flight per thread
-        const float *ip = (const float *)st.aux0 + (size_t)item * cmax * QPK * MK_ATTN_PSTRIDE;
+        const float *ip = part_base + (size_t)item * cmax * QPK * MK_ATTN_PSTRIDE;
         float mx = -INFINITY, ls = 0.f, os[DPT];
 #pragma unroll
         for (int d = 0; d < DPT; d++) os[d] = 0.f;
@@ -2816,14 +2820,14 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
 
 // Greedy sampling, stage 1: every workgroup scans a contiguous slice of each token's logits and keeps
 // (max, lowest index attaining it).  Reference task: tasks/mi300/argmax_mi300.cuh:78-127.
-__device__ __forceinline__ void stage_argmax_partial(CStage &st, Ctx &c, int M, char *smem) {
+__device__ __forceinline__ void stage_argmax_partial(CStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
   barrier_wait(c);
   const int n = st.n;
   int per = (n + c.G - 1) / c.G;
   per = (per + 1) & ~1;  // even, so slices start on a dword
   const int c0 = c.vid * per, c1 = min(n, c0 + per);
-  float *pv = (float *)st.aux0;
-  int *pi = (int *)st.aux1;
+  float *pv = rt.argmax_pv ? rt.argmax_pv : (float *)st.aux0;
+  int *pi = rt.argmax_pv ? rt.argmax_pi : (int *)st.aux1;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   constexpr int NDW = 5, TB = 4;  // dwords per lane per token, tokens in flight per wavefront
   const int nd = (c1 - c0 + 1) / 2;
@@ -2867,10 +2871,10 @@ __device__ __forceinline__ void stage_argmax_partial(CStage &st, Ctx &c, int M, 
 
 // Greedy sampling, stage 2: one wavefront per token reduces the per-workgroup partials.
 // Reference task: tasks/mi300/argmax_mi300.cuh:129-158.
-__device__ __forceinline__ void stage_argmax_reduce(CStage &st, Ctx &c, int M) {
+__device__ __forceinline__ void stage_argmax_reduce(CStage &st, Ctx &c, const MkRuntime &rt, int M) {
   barrier_wait(c);
-  const float *pv = (const float *)st.aux0;
-  const int *pi = (const int *)st.aux1;
+  const float *pv = rt.argmax_pv ? rt.argmax_pv : (const float *)st.aux0;
+  const int *pi = rt.argmax_pv ? rt.argmax_pi : (const int *)st.aux1;
   long long *out = (long long *)st.out;
   const int lane = threadIdx.x & 63, wave = __builtin_amdgcn_readfirstlane(threadIdx.x >> 6);
   for (int t = c.vid * MK_WAVES + wave; t < M; t += c.G * MK_WAVES) {
@@ -3048,8 +3052,8 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
         case MK_OP_MOE_TOPK: stage_moe_topk(st, c, M); break;
         case MK_OP_MOE_LINEAR: stage_moe_linear(st, c, M, smem); break;
         case MK_OP_MOE_COMBINE: stage_moe_combine(st, c, M); break;
-        case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, M, smem); break;
-        case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, M); break;
+        case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, rt, M, smem); break;
+        case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, rt, M); break;
         default: barrier_wait(c); break;
       }
       const long long t_out = (long long)wall_clock64();

@@ -176,7 +176,10 @@ struct MkRuntime {
   const MkStage *stages;
   MkSync *sync;
   // attention split-KV workspace
-  float *attn_part;     // [units][qpk][head_dim + 2]
+  float *attn_part;     // null: every attention stage has a partial buffer of its own (its descriptor's aux0).  Non-null: ONE buffer
+                        // [units][q/kv][MK_ATTN_PSTRIDE] shared by all attention stages, handed off at device scope only
+  float *argmax_pv;     // non-null: the sampling stages' per-workgroup partials live here ([tokens][workgroups] values / indices)
+  int *argmax_pi;       // instead of in the buffers their descriptors name
   unsigned *attn_cnt;   // [max_tokens * num_kv_heads][32]: one 128-byte line per counter
   void *splitk_part;    // [workgroups][4 wavefronts][4 weight tiles][4 token tiles][64 lanes] f32x4: K-slice partials of the split-K linear
   unsigned *splitk_cnt; // [workgroups][32]: arrival counter per split-K group (one 128-byte line each)

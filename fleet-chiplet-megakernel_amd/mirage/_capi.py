@@ -24,7 +24,7 @@ MK_MODES = {"offline": 0, "online": 1, "online_notoken": 2, "onepass": 3}
 EXPORTED_SYMBOLS = [
     "mk_graph_create", "mk_graph_destroy", "mk_tensor_attach", "mk_tensor_new", "mk_tensor_shuffle",
     "mk_tensor_num_dims", "mk_tensor_dim", "mk_tensor_ptr", "mk_add_task", "mk_generate_task_graph",
-    "mk_compile", "mk_init_requests", "mk_launch", "mk_launch_steps", "mk_enqueue_steps", "mk_wait",
+    "mk_compile", "mk_init_requests", "mk_launch", "mk_launch_steps", "mk_enqueue_steps", "mk_enqueue_steps_static", "mk_wait",
     "mk_run_once", "mk_get_stats", "mk_get_stage_profile", "mk_describe_program", "mk_last_error", "mk_version",
 ]
 
@@ -110,6 +110,7 @@ def load():
     lib.mk_launch.argtypes = [vp, vp]
     lib.mk_launch_steps.argtypes = [vp, vp, ci, cip]
     lib.mk_enqueue_steps.argtypes = [vp, vp, ci]
+    lib.mk_enqueue_steps_static.argtypes = [vp, vp, ci]
     lib.mk_wait.argtypes = [vp, vp, cip]
     i32p = ctypes.POINTER(ctypes.c_int32)
     lib.mk_run_once.argtypes = [vp, vp, ci, i32p, i32p, i32p]

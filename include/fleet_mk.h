@@ -139,6 +139,15 @@ int mk_launch_steps(mk_graph *g, void *stream, int max_iterations, int *finished
  * launch and returns; mk_wait() synchronises and reports watchdog aborts. */
 int mk_enqueue_steps(mk_graph *g, void *stream, int max_iterations);
 int mk_wait(mk_graph *g, void *stream, int *finished_out);
+/* mk_enqueue_steps for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
+ * forbid hipMalloc); it has no counterpart in the reference.  The call allocates and frees nothing, and every piece
+ * of scratch its launch uses -- barrier counters, K-split partial tiles and counters, attention split-KV partials and
+ * counters, sampling partials -- lives in one file-scope device array of about 19.7 MB per GPU (held until the process
+ * ends) instead of in the buffers mk_compile allocated; it is cleared by a fill kernel on `stream`, not by a memset.
+ * Limits (MK_EINVAL beyond them): at most 256 workgroups, max_num_batched_tokens x kv heads <= 512, at most 8 q heads
+ * per kv head.  All calls on one GPU share that array: calls that overlap on one GPU race, whatever their handles or
+ * streams.  Results are bit-identical to mk_enqueue_steps; per-stage timing is not recorded.  Pair with mk_wait. */
+int mk_enqueue_steps_static(mk_graph *g, void *stream, int max_iterations);
 /* Host-driven single pass (the reference's MODE_ONEPASS / online modes, persistent_kernel.cuh:538-582): the caller
  * supplies the batch -- for each of `num_tokens` rows its batch slot, absolute position and the index of the first
  * row of the same request -- and has filled input_tokens / paged_kv_* itself.  Runs the stage program once. */
