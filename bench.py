@@ -114,7 +114,8 @@ def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
     t1 = time.perf_counter()
     st = dec.mpk.stats()
     assert not finished, "requests finished inside the timed region; lower --steps"
-    assert dec.meta["step"].cpu().tolist() == [s0 + K for s0 in steps0], "timed region did not run exactly K decode steps for every request"
+    steps1 = dec.meta["step"].cpu().tolist()
+    assert steps1 == [s0 + K for s0 in steps0], f"timed region did not run exactly K={K} decode steps for every request: {steps0} -> {steps1}"
     wall_ms = (t1 - t0) * 1e3
     kernel_ms = st["last_launch_ms"]
     ms_per_step = wall_ms / K
@@ -176,7 +177,6 @@ def main():
     shape = Qwen3Shape.qwen3_30b_a3b(min(args.layers, 48) if args.layers != 36 else 48) if moe else Qwen3Shape(num_layers=args.layers)
     K, W, P = args.steps, args.warmup, args.prompt_length
     batches = [args.batch] if args.batch else ([1, 64] if not moe else [1])
-    max_seq = max(1200, P + W + K + 2 + 16)
     if args.calib_copy:
         src = torch.ones(1 << 28, dtype=torch.float32, device="cuda")
         dst = torch.empty_like(src)
@@ -186,6 +186,12 @@ def main():
     weights = random_weights(shape, seed=0)
     legs = []
     for B in batches:
+        # The on-GPU scheduler shares B token slots per iteration between decoding requests (one each) and prompt ingestion
+        # (8 tokens per request), exactly as the reference's does: at B = 64 the first requests have decoded some 360 tokens
+        # by the time the last one has ingested its prompt.  The timed K steps start once ALL B requests decode, so the
+        # requests sit at different contexts (the range is in `workload`; the KV bytes of the roofline are the real ones);
+        # max_seq_len is the configuration's 1200 unless the earliest request's K timed steps would not fit.
+        max_seq = max(1200, P + W + K + 2 + (0 if B == 1 else 6 * P))
         dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
         legs.append(run_leg(torch, dec, shape, args.model, B, K, W, P, max_seq, args.mode))
         dec.mpk.finalize()
