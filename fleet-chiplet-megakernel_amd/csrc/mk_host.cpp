@@ -114,6 +114,7 @@ struct mk_graph {
   double last_ms = 0.0;
   int last_nxcd = 0, last_aborted = 0;
   int64_t weight_bytes = 0;
+  int64_t packed_bytes = 0;  // matrix-core copies of the weights held by the handle
   size_t attn_cnt_n = 0;
   int num_ref_tasks = 0, num_ref_events = 0;
   int last_linear_task = -1, last_linear_stage = -1;  // lowering: the most recent linear task and the stage it became
@@ -312,6 +313,14 @@ int lower_linear(mk_graph *g, size_t &i) {
     ns.norm_w = nw.ptr;
     ns.out = no.ptr;
     ns.ld_out = (int)no.strides[0];
+    if (!g->stages.empty()) {
+      // a plain or residual linear whose whole output this norm reads may leave its split-K sum to the norm stage
+      MkStage &pl = g->stages.back();
+      const bool rows_ok = (ns.k & 15) == 0 && ns.k / 8 <= 6 * MK_THREADS && (ns.ld_in & 7) == 0 && (ns.ld_out & 7) == 0 && ((uintptr_t)ns.in & 15) == 0;
+      const bool res_ok = !(pl.flags & MK_F_RES) || ((pl.ld_res & 7) == 0 && ((uintptr_t)pl.res & 15) == 0);
+      if (pl.op == MK_OP_LINEAR && !(pl.flags & MK_F_SILU) && pl.out == ns.in && pl.ld_out == ns.ld_in && pl.n == ns.k && rows_ok && res_ok)
+        pl.flags |= MK_F_DEFER_SUM;
+    }
     g->stages.push_back(ns);
     g->stage_desc.push_back(fmt("NORM[multi-token only] %s -> %s k=%d", nx.name.c_str(), no.name.c_str(), st.k));
     st.flags |= MK_F_NORM;
@@ -1335,6 +1344,46 @@ int mk_generate_task_graph(mk_graph *g, int num_gpus, int my_gpu_id, const char 
   return MK_OK;
 }
 
+// Matrix-core copies of the linear weights (MkStage::wpack).  A graph that can run more than eight tokens per iteration
+// streams its weights through the matrix cores in 16-row tiles; read from a row-major matrix that is 64 bytes from each
+// of 16 rows per request, which HBM serves at about three quarters of the rate of one contiguous stream.  So every such
+// weight is re-laid once, tile by tile, in a buffer the handle owns (this doubles the weight footprint; single-token
+// iterations keep reading the caller's row-major tensors).  FLEET_MK_PACK_WEIGHTS=0 turns the copies off.
+// allocate = false re-runs the copy kernels into the existing buffers (the caller changed weights after compiling).
+static int pack_weights(mk_graph *g, bool allocate) {
+  const char *env = getenv("FLEET_MK_PACK_WEIGHTS");
+  if (g->cfg.max_num_batched_tokens <= 8 || (env && atoi(env) == 0)) return 0;
+  for (auto &st : g->stages) {
+    if (st.op != MK_OP_LINEAR || (st.k & 63) || st.k < 64) continue;
+    const bool silu = st.flags & MK_F_SILU;
+    const int n_out = silu ? st.n / 2 : st.n;
+    const long long tiles = (long long)((n_out + 15) / 16) * (silu ? 2 : 1);
+    const long long total = tiles * (st.k >> 6) * 128;  // 16-byte operands
+    if (allocate) {
+      void *p = nullptr;
+      if (hipMalloc(&p, (size_t)total * 16) != hipSuccess) {
+        (void)hipGetLastError();
+        return fail(MK_EHIP, "no device memory for the %.1f MB matrix-core copy of a weight (FLEET_MK_PACK_WEIGHTS=0 runs without the copies)", total * 16 / 1e6);
+      }
+      g->allocs.push_back(p);
+      st.wpack = p;
+      g->packed_bytes += total * 16;
+    }
+    if (!st.wpack) continue;
+    hipLaunchKernelGGL(mk_pack_weights_kernel, dim3(2048), dim3(256), 0, 0, st.w, st.n, st.k, silu ? 1 : 0, st.silu_half, (u32x4 *)st.wpack, total);
+    HIP_TRY(hipGetLastError());
+  }
+  HIP_TRY(hipDeviceSynchronize());
+  return 0;
+}
+
+int mk_repack_weights(mk_graph *g) {
+  if (!g) return fail(MK_EINVAL, "null argument");
+  if (!g->compiled) return fail(MK_ESTATE, "graph not compiled");
+  HIP_TRY(hipSetDevice(g->cfg.device));
+  return pack_weights(g, false);
+}
+
 int mk_compile(mk_graph *g) {
   if (!g) return fail(MK_EINVAL, "null argument");
   if (g->compiled) return fail(MK_ESTATE, "graph already compiled");
@@ -1410,6 +1459,7 @@ int mk_compile(mk_graph *g) {
       s.aux0 = p;
       s.aux1 = rt.attn_cnt + g->attn_cnt_n / 2;
     }
+  if ((rc = pack_weights(g, true))) return rc;
   if ((rc = dev_alloc(g, &p, sizeof(MkStage) * (g->stages.size() + 1)))) return rc;
   g->d_stages = (MkStage *)p;
   rt.stages = g->d_stages;
@@ -1422,7 +1472,7 @@ int mk_compile(mk_graph *g) {
   if ((rc = dev_alloc(g, &p, sizeof(long long) * (g->timing_cap + 2)))) return rc;
   rt.timing = g->d_timing = (long long *)p;
   rt.timing_cap = g->timing_cap;
-  if ((rc = dev_alloc(g, &p, sizeof(long long) * 4 * (g->stages.size() + 1) * g->G))) return rc;
+  if ((rc = dev_alloc(g, &p, sizeof(long long) * MK_PROF_TICKS * (g->stages.size() + 1) * g->G))) return rc;
   rt.stage_prof = (long long *)p;
   if ((rc = dev_alloc(g, &p, sizeof(MkRuntime)))) return rc;
   g->d_rt = (MkRuntime *)p;
@@ -1554,6 +1604,7 @@ int mk_get_stats(mk_graph *g, mk_stats *out) {
   out->num_xcds = g->last_nxcd;
   out->aborted = g->last_aborted;
   out->weight_bytes = g->weight_bytes;
+  out->packed_weight_bytes = g->packed_bytes;
   out->last_launch_ms = g->last_ms;
   if (g->compiled && !g->launch_pending) {
     MkSched sc;
@@ -1563,15 +1614,24 @@ int mk_get_stats(mk_graph *g, mk_stats *out) {
   return MK_OK;
 }
 
-int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages) {
+// ticks [first, first + 4) of the stage records of one workgroup, scheduler record last
+static int copy_stage_ticks(mk_graph *g, int workgroup, int first, int64_t *ticks_out, int max_stages) {
   if (!g || !ticks_out) return fail(MK_EINVAL, "null argument");
   if (!g->compiled || g->launch_pending) return fail(MK_ESTATE, "no finished launch to report");
   if (workgroup < 0 || workgroup >= g->G) return fail(MK_EINVAL, "workgroup %d outside [0, %d)", workgroup, g->G);
-  const int n = std::min<int>(max_stages, (int)g->stages.size());
-  if (n > 0)
-    HIP_TRY(hipMemcpy(ticks_out, g->h_rt.stage_prof + (size_t)4 * workgroup * g->stages.size(), sizeof(int64_t) * 4 * n, hipMemcpyDeviceToHost));
+  const int recs = (int)g->stages.size() + 1;
+  const int n = std::min<int>(max_stages, recs);
+  if (n <= 0) return 0;
+  std::vector<long long> buf((size_t)MK_PROF_TICKS * recs);
+  HIP_TRY(hipMemcpy(buf.data(), g->h_rt.stage_prof + (size_t)MK_PROF_TICKS * workgroup * recs, sizeof(long long) * buf.size(), hipMemcpyDeviceToHost));
+  for (int s = 0; s < n; s++)
+    for (int k = 0; k < 4; k++) ticks_out[4 * s + k] = buf[(size_t)MK_PROF_TICKS * s + first + k];
   return n;
 }
+
+int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages) { return copy_stage_ticks(g, workgroup, 0, ticks_out, max_stages); }
+
+int mk_get_stage_marks(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages) { return copy_stage_ticks(g, workgroup, 4, ticks_out, max_stages); }
 
 int mk_describe_program(mk_graph *g, const char **text_out) {
   if (!g || !text_out) return fail(MK_EINVAL, "null argument");

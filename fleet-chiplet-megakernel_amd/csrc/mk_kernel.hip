@@ -70,7 +70,22 @@ struct Ctx {
                       // MoE stage that last filled the workgroup's expert list (kept outside the stages' scratch LDS)
   int seq;            // stages executed so far by this workgroup
   bool wrote_through; // the stage that just ran wrote all its outputs with write-through stores: no L2 write-back at its barrier
+  // A split-K linear whose consumer is a full-row norm leaves its K-slice partials unsummed: the norm stage, which reads
+  // every row anyway, sums them (slice order, then the residual, then one rounding: the same arithmetic).
+  int defer_S;            // slices left unsummed by the stage that just ran (0: none)
+  int defer_rows;         // token rows per slice in the partial buffer
+  const float *defer_part;  // [slice][row][n] fp32
+  const void *defer_res;  // residual rows of that linear (null: none)
+  int defer_ld_res;
+#ifdef MK_TRACE
+  long long mark[4];  // (tracing builds) wall-clock marks the running stage sets, stored next to its stage timing
+#endif
 };
+#ifdef MK_TRACE
+#define MK_MARK(c, i) ((c).mark[i] = (long long)wall_clock64())
+#else
+#define MK_MARK(c, i) ((void)0)
+#endif
 
 // ----------------------------------------------------------------------------- small helpers
 __device__ __forceinline__ float bf_lo(uint32_t u) { return __uint_as_float(u << 16); }
@@ -484,6 +499,38 @@ __device__ __forceinline__ const u32x4 *weight_row(CWeight &w, int r, int k8) {
   return (const u32x4 *)w.seg[s] + (size_t)(g * w.seg_rows[s] + o) * k8;
 }
 
+// Re-lays the weights of one linear stage in matrix-core tile order (MkStage::wpack); one thread per 16-byte operand.
+// Rows past the last output repeat it (their products are never stored).
+extern "C" __global__ __launch_bounds__(256) void mk_pack_weights_kernel(const MkWeight w, int n, int k, int silu, int half, u32x4 *dst, long long total) {
+  const int k8 = k / 8, nsteps = k >> 6;
+  const int n_out = silu ? n / 2 : n;
+  for (long long idx = (long long)blockIdx.x * 256 + threadIdx.x; idx < total; idx += (long long)gridDim.x * 256) {
+    const int lane = (int)(idx & 63);
+    long long r = idx >> 6;
+    const int h = (int)(r & 1);
+    r >>= 1;
+    const int step = (int)(r % nsteps), ti = (int)(r / nsteps);
+    const int lr = lane & 15, lg = lane >> 4;
+    int vr;
+    if (silu) {
+      const int o = min((ti >> 1) * 16 + lr, n_out - 1), gi = o / half;
+      vr = gi * 2 * half + (o - gi * half) + ((ti & 1) ? half : 0);
+    } else {
+      vr = min(ti * 16 + lr, n_out - 1);
+    }
+    const u32x4 *row;
+    if (w.nseg == 1) {
+      row = (const u32x4 *)w.seg[0] + (size_t)vr * k8;
+    } else {
+      const int g = vr / w.group_rows;
+      int o = vr - g * w.group_rows, sg = 0;
+      while (sg + 1 < w.nseg && o >= w.seg_rows[sg]) o -= w.seg_rows[sg++];
+      row = (const u32x4 *)w.seg[sg] + (size_t)(g * w.seg_rows[sg] + o) * k8;
+    }
+    dst[idx] = row[step * 8 + h * 4 + lg];
+  }
+}
+
 // ----------------------------------------------------------------------------- stages
 // Every stage function posts barrier_wait(c) itself, after any work that does not depend on the previous
 // stage (weight prefetch), and the main loop posts barrier_arrive(c) when the function returns.
@@ -533,15 +580,65 @@ __device__ __forceinline__ void stage_norm(CStage &st, Ctx &c, int M, char *smem
     for (int j = 0; j < NS; j++)
       if (j * MK_THREADS < k8) g[j] = w4[min(tid + j * MK_THREADS, k8 - 1)];
     barrier_wait(c);
-    for (int t = c.vid; t < M; t += c.G) {
+    const int dS = c.defer_S;
+    c.defer_S = 0;
+    // rows are dealt round-robin over the dies, so a handful of rows does not funnel through one die's memory path
+    const int t0 = c.even_xcds ? c.rank * c.nxcd + c.xi : c.vid;
+    for (int t = t0; t < M; t += c.G) {
       const u32x4 *x = (const u32x4 *)((const uint16_t *)st.in + (size_t)t * st.ld_in);
       u32x4 *y = (u32x4 *)((uint16_t *)st.out + (size_t)t * st.ld_out);
       float ss = 0.f;
+      if (dS) {
+        // the rows are still K-slice partials: finish the producing linear (sum, residual, rounding), store its output
+        // row where it belongs, and normalise the rounded values
+        const u32x4 *r4 = (const u32x4 *)((const uint16_t *)c.defer_res + (size_t)t * c.defer_ld_res);
+#pragma unroll
+        for (int j = 0; j < NS; j++)
+          if (j * MK_THREADS < k8) {
+            const int seg = min(tid + j * MK_THREADS, k8 - 1);
+            float a[8];
+#pragma unroll
+            for (int e = 0; e < 8; e++) a[e] = 0.f;
+            const u32x4 rv = ldc_16B(c.defer_res ? r4 + seg : (const u32x4 *)c.defer_part);  // requested ahead of the partials it is added to
+            auto sum_slices = [&](auto ns) {  // all slices requested at once, summed in slice order
+              constexpr int Q = decltype(ns)::value;
+              u32x4 pv[Q][2];
+#pragma unroll
+              for (int q = 0; q < Q; q++) {
+                const u32x4 *p = (const u32x4 *)(c.defer_part + ((size_t)q * c.defer_rows + t) * st.k) + seg * 2;
+                pv[q][0] = ldc_16B(p);
+                pv[q][1] = ldc_16B(p + 1);
+              }
+#pragma unroll
+              for (int q = 0; q < Q; q++)
+#pragma unroll
+                for (int e = 0; e < 4; e++) {
+                  a[e] += __uint_as_float(pv[q][0][e]);
+                  a[4 + e] += __uint_as_float(pv[q][1][e]);
+                }
+            };
+            if (dS == 2) sum_slices(std::integral_constant<int, 2>{});
+            else if (dS == 4) sum_slices(std::integral_constant<int, 4>{});
+            else sum_slices(std::integral_constant<int, 8>{});
+            if (c.defer_res) {
+#pragma unroll
+              for (int e = 0; e < 4; e++) {
+                a[2 * e] += bf_lo(rv[e]);
+                a[2 * e + 1] += bf_hi(rv[e]);
+              }
+            }
+#pragma unroll
+            for (int e = 0; e < 4; e++) v[j][e] = pack2(a[2 * e], a[2 * e + 1]);
+          }
+#pragma unroll
+        for (int j = 0; j < NS; j++)  // stores after all the loads: neither is moved across the other
+          if (tid + j * MK_THREADS < k8) stc_16B((u32x4 *)x + tid + j * MK_THREADS, v[j]);
+      }
 #pragma unroll
       for (int j = 0; j < NS; j++)
         if (j * MK_THREADS < k8) {
           const bool ok = tid + j * MK_THREADS < k8;
-          v[j] = ldc_16B(x + min(tid + j * MK_THREADS, k8 - 1));
+          if (!dS) v[j] = ldc_16B(x + min(tid + j * MK_THREADS, k8 - 1));
 #pragma unroll
           for (int e = 0; e < 4; e++) ss += ok ? bf_lo(v[j][e]) * bf_lo(v[j][e]) + bf_hi(v[j][e]) * bf_hi(v[j][e]) : 0.f;
         }
@@ -1177,6 +1274,7 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
   c.wrote_through = true;  // partial tiles and outputs are all written through: no L2 write-back at this stage's arrival
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   __syncthreads();
+  MK_MARK(c, 0);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const bool silu = st.flags & MK_F_SILU;
@@ -1300,6 +1398,7 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
       else pipeline(std::false_type{}, std::false_type{});
     }
 
+    MK_MARK(c, 1);
     // ---- combine the S slices (a split range is a single sweep, so slots are indexed by wavefront and tile only)
     if (S > 1) {
       if (has_tile) {
@@ -1318,6 +1417,7 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
         *sflag = last;
       }
       __syncthreads();
+      MK_MARK(c, 2);
       if (!*sflag || !has_tile) return;
 #pragma unroll
       for (int t = 0; t < TW; t++) {
@@ -1340,6 +1440,7 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
         }
       }
     }
+    MK_MARK(c, 3);
     if (!has_tile) return;
     // ---- epilogue: lane l holds token m = mt * 16 + (l & 15), output columns tile * 16 + (l >> 4) * 4 .. + 3
     constexpr int OT = TW >= 2 ? TW / 2 : 1;
@@ -1386,6 +1487,311 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
   }
 }
 
+// Matrix-core linear with the token rows staged through LDS by wavefronts of their own.  A workgroup owns a range of 4..6
+// weight tiles and one K slice, which it works off in passes of 8 steps (512 k).  Wavefronts 0 and 1 hold two or three
+// tiles each and do nothing but stream weights (a ring of NB = 8 steps, 32 or 48 KB per wavefront, which runs on across
+// the passes without ever draining) and feed the matrix cores from LDS; wavefronts 2 and 3 stage the token rows of the
+// NEXT pass -- all rows, 64 KB for 64 tokens, in matrix-core operand order, with loads that write LDS directly (no
+// registers) -- into the other half of a double buffer.  Loads return in issue order per wavefront, and a token-row
+// load queues behind the weight stream in the memory system like any other request, so in a wavefront that also
+// streams weights every batch of row loads stalls the weight ring for a full memory latency; on wavefronts of their
+// own they cost the streaming wavefronts nothing.  (One staging wavefront is not enough: with at most 63 requests
+// outstanding it needs two memory latencies for the 128 requests of a pass, and the pass cannot be shorter than that.)
+// One workgroup barrier per pass hands a buffer over.  The first NB weight steps are requested before the previous
+// stage's barrier is awaited; the rows of the first pass are staged by all four wavefronts.  The S workgroups that
+// share a tile range exchange their partial tiles as the streaming form does (write-through buffer, last arriver sums
+// in slice order), or leave the sum to a norm stage that follows.  Used for the QKV, o, gate/up and down projections at
+// 9..64 tokens.  SwiGLU stages number their weight tiles gate, up, gate, up ...; with three tiles per wavefront the
+// middle pair straddles the two streaming wavefronts and is joined through LDS in the epilogue.
+#define MK_XRES_STEPS 8  // steps per pass
+struct XresPlan {
+  int S;       // K slices per tile range (0: this form cannot run the stage)
+  int groups;  // tile ranges
+  int wt;      // weight tiles of the stage
+  int tpu;     // most tiles a range holds (decides tiles per wavefront and prefetch depth for every workgroup alike)
+};
+__device__ __forceinline__ XresPlan linear_xres_plan(CStage &st, const Ctx &c) {
+  XresPlan p;
+  p.S = 0;
+  p.groups = 0;
+  p.tpu = 0;
+  const bool silu = st.flags & MK_F_SILU;
+  const int n_out = silu ? st.n / 2 : st.n, unit = silu ? 2 : 1;
+  p.wt = ((n_out + 15) / 16) * unit;
+  for (int S = 1; S <= 8; S *= 2) {
+    if (c.G % S || st.k % (S * 64 * MK_XRES_STEPS)) break;
+    const int gs = c.G / S;
+    int tpu = (p.wt + gs - 1) / gs;  // tiles per range
+    tpu = (tpu + unit - 1) / unit * unit;
+    if (tpu > 6) break;              // two streaming wavefronts with three tiles each
+    if (tpu < 4) continue;           // too few tiles to occupy them: split K further
+    p.S = S;
+    p.tpu = tpu;
+    p.groups = (p.wt / unit + tpu / unit - 1) / (tpu / unit);
+    return p;
+  }
+  return p;
+}
+
+template <int MT, int TW>
+__device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const MkRuntime &rt, int M, const XresPlan plan, char *smem) {
+  c.wrote_through = true;  // partial tiles and outputs are all written through: no L2 write-back at this stage's arrival
+  constexpr int NSP = MK_XRES_STEPS;
+  const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+  const int lr = lane & 15, lg = lane >> 4;
+  const bool silu = st.flags & MK_F_SILU;
+  const int K = st.k, k8 = K / 8;
+  const int n_out = silu ? st.n / 2 : st.n, unit = silu ? 2 : 1;
+  const int half = st.silu_half;
+  const int S = plan.S;
+  const int g = c.vid / S, sl = c.vid - g * S;
+  const bool active = g < plan.groups;  // workgroups beyond the last range only keep the barriers
+  const int nun = plan.wt / unit;       // balanced ranges of whole units
+  const int tb = active ? (int)(((long long)g * nun) / plan.groups) * unit : 0, te = active ? (int)(((long long)(g + 1) * nun) / plan.groups) * unit : 0;
+  const int kslice = K / S, kbeg = sl * kslice, nsteps = kslice >> 6, npass = nsteps / NSP;
+  const uint16_t *x = (st.flags & MK_F_NORM) ? (const uint16_t *)st.norm_out : (const uint16_t *)st.in;
+  const int ldx = (st.flags & MK_F_NORM) ? st.ld_norm : st.ld_in;
+  u32x4 *xl = (u32x4 *)smem;  // two buffers of [step of the pass][token tile][2][64 lanes] 16-byte operands
+  constexpr int XBUF = NSP * MT * 128;  // 16-byte operands per buffer
+  int *sflag = (int *)(smem + 2 * XBUF * 16);
+  u32x4 *part = (u32x4 *)rt.splitk_part;
+  // hand the K-slice sum to the norm stage that follows, if there is one and the rows fit the partial buffer
+  const bool defer = (st.flags & MK_F_DEFER_SUM) && S > 1 && (size_t)S * (MT * 16) * st.n * 4 <= (size_t)c.G * 65536;
+  if (defer) {
+    c.defer_S = S;
+    c.defer_rows = MT * 16;
+    c.defer_part = (const float *)rt.splitk_part;
+    c.defer_res = (st.flags & MK_F_RES) ? st.res : nullptr;
+    c.defer_ld_res = st.ld_res;
+  }
+  // this lane's first operand of weight tile ti, and the distance (in 16-byte operands) between steps and between the two
+  // halves of a step: the re-laid copy streams contiguously, the row-major original reads 64 bytes of each of 16 rows
+  const bool packed = st.wpack != nullptr;
+  const int step_stride = packed ? 128 : 8, half_stride = packed ? 64 : 4;
+  auto tile_base = [&](int ti) -> const u32x4 * {
+    if (packed) return (const u32x4 *)st.wpack + ((size_t)ti * (K >> 6) + (kbeg >> 6)) * 128 + lane;
+    int o, vr;
+    if (silu) {
+      o = min((ti >> 1) * 16 + lr, n_out - 1);
+      const int gi = o / half;
+      vr = gi * 2 * half + (o - gi * half) + ((ti & 1) ? half : 0);
+    } else {
+      o = min(ti * 16 + lr, n_out - 1);
+      vr = o;
+    }
+    return weight_row(st.w, vr, k8) + (kbeg >> 3) + lg;
+  };
+  // stage the token rows of one pass: item i = (step, token tile), two 1 KB requests each, straight into LDS (lane l's 16
+  // bytes land at l * 16 behind the request's LDS base, which is the operand order).  `nw` wavefronts share the items:
+  // wavefront `w` of them takes items w, w + nw, ...
+  auto stage_pass = [&](int pass, int w, int nw) {
+    const uint16_t *base = x + kbeg + pass * (NSP * 64) + lg * 8;
+    u32x4 *buf = xl + (pass & 1) * XBUF;
+    for (int i = w; i < MT * NSP; i += nw) {
+      const int step = i / MT, mt = i - step * MT;
+      const uint16_t *src = base + (size_t)min(mt * 16 + lr, M - 1) * ldx + (step << 6);
+      __attribute__((address_space(3))) char *dst = (__attribute__((address_space(3))) char *)(buf + (size_t)i * 128);
+      __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)src, (__attribute__((address_space(3))) void *)dst, 16, 0, 0);
+      __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(src + 32), (__attribute__((address_space(3))) void *)(dst + 1024), 16, 0, 0);
+    }
+  };
+
+  {
+    constexpr int NB = 8, NSW = 2;    // ring depth in steps; streaming wavefronts
+    const bool loader = wave >= NSW;  // stages token rows, holds no tiles
+    const int tw0 = tb + wave * TW;   // a streaming wavefront's first tile
+    const bool has_tile = active && !loader && tw0 < te;
+    const u32x4 *wrow[TW];
+#pragma unroll
+    for (int t = 0; t < TW; t++) wrow[t] = tile_base(max(min(tw0 + t, te - 1), 0));
+    bf16x8 a[NB][TW][2];
+    auto w_load = [&](int step, bf16x8 (&aa)[TW][2]) {
+#pragma unroll
+      for (int t = 0; t < TW; t++) {
+        aa[t][0] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + step * step_stride));
+        aa[t][1] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + step * step_stride + half_stride));
+      }
+    };
+    // weights do not depend on the previous stage: the first NB steps are requested before its barrier is awaited, by the
+    // polling wavefront as well (its first poll result then arrives behind them -- loads return in order -- which costs
+    // nothing unless this workgroup is the barrier's last arriver, and spares it a trip to memory after the barrier)
+    if (has_tile) {
+#pragma unroll
+      for (int j = 0; j < NB; j++) w_load(j, a[j]);
+    }
+    if (c.pending && tid == 0) barrier_poll(c);
+    if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // token rows come from other workgroups: one acquire, then cached loads
+    __syncthreads();
+    barrier_done(c);
+    MK_MARK(c, 0);
+    f32x4 acc[TW][MT];
+#pragma unroll
+    for (int t = 0; t < TW; t++)
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+    auto compute = [&](const u32x4 *xb, const bf16x8 (&aa)[TW][2]) {
+      u32x4 b[2][MT];
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) b[h][mt] = xb[(mt * 2 + h) * 64 + lane];
+      __builtin_amdgcn_sched_barrier(0);  // all operand reads in flight before the first matrix instruction waits
+#pragma unroll
+      for (int h = 0; h < 2; h++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+          for (int t = 0; t < TW; t++) acc[t][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(aa[t][h], __builtin_bit_cast(bf16x8, b[h][mt]), acc[t][mt], 0, 0, 0);
+      __builtin_amdgcn_sched_barrier(0);
+    };
+    // Passes [0, n_refill) refill the ring as they go, the last one only consumes it.  Every pass starts with a workgroup
+    // barrier: its rows have landed (whoever requested them has waited for them) and everybody is done with the other
+    // buffer, into which the loader then requests the next pass's rows.
+    const int n_refill = npass - 1;
+    auto do_pass = [&](int pass, auto refill_c) {
+      constexpr bool REFILL = decltype(refill_c)::value;
+      if (pass == 0 || loader) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (pass == 0) MK_MARK(c, 1);
+      if (loader && active && pass + 1 < npass) stage_pass(pass + 1, wave - NSW, MK_WAVES - NSW);
+      __builtin_amdgcn_sched_barrier(0);
+      if (has_tile) {
+        const u32x4 *xb = xl + (pass & 1) * XBUF;
+#pragma unroll
+        for (int j = 0; j < NSP; j++) {
+          compute(xb + j * MT * 128, a[j]);
+          if (REFILL) w_load(pass * NSP + j + NB, a[j]);
+        }
+      }
+    };
+    if (active) stage_pass(0, wave, MK_WAVES);
+    __builtin_amdgcn_sched_barrier(0);
+    int pass = 0;
+    for (; pass < n_refill; pass++) do_pass(pass, std::true_type{});
+    MK_MARK(c, 2);
+    do_pass(pass, std::false_type{});
+    MK_MARK(c, 3);
+    if (defer) {
+      // the consumer sums the slices: leave them as [slice][token][n] fp32 rows
+      if (has_tile) {
+        float *prow = (float *)rt.splitk_part + (size_t)sl * (MT * 16) * st.n;
+#pragma unroll
+        for (int t = 0; t < TW; t++)
+          if (tw0 + t < te) {
+#pragma unroll
+            for (int mt = 0; mt < MT; mt++)
+              stc_16B((u32x4 *)(prow + (size_t)(mt * 16 + lr) * st.n + (tw0 + t) * 16 + lg * 4), __builtin_bit_cast(u32x4, acc[t][mt]));
+          }
+      }
+      return;
+    }
+    // ---- combine the S slices: partial tiles through the write-through buffer, summed by the last workgroup to arrive
+    if (S > 1) {
+      if (has_tile) {
+#pragma unroll
+        for (int t = 0; t < TW; t++)
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++)
+            stc_16B(part + ((((size_t)c.vid * 4 + wave) * 4 + t) * 4 + mt) * 64 + lane, __builtin_bit_cast(u32x4, acc[t][mt]));
+      }
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      __syncthreads();
+      if (tid == 0) {
+        int last = 0;
+        if (active) {
+          unsigned *cnt = rt.splitk_cnt + (size_t)g * 32;
+          last = __hip_atomic_fetch_add(cnt, 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT) == (unsigned)(S - 1);
+          if (last) __hip_atomic_store(cnt, 0u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+        }
+        *sflag = last;
+      }
+      __syncthreads();
+      if (!*sflag) return;  // (the whole workgroup)
+#pragma unroll
+      for (int t = 0; t < TW; t++)
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) acc[t][mt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      for (int q0 = 0; has_tile && q0 < S; q0 += 4) {  // four slices of both tiles requested at once; summed in slice order
+        u32x4 pv[4][TW][MT];
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          if (q0 + q < S) {
+#pragma unroll
+            for (int t = 0; t < TW; t++)
+#pragma unroll
+              for (int mt = 0; mt < MT; mt++) pv[q][t][mt] = ldc_16B(part + ((((size_t)(g * S + q0 + q) * 4 + wave) * 4 + t) * 4 + mt) * 64 + lane);
+          }
+#pragma unroll
+        for (int q = 0; q < 4; q++)
+          if (q0 + q < S) {
+#pragma unroll
+            for (int t = 0; t < TW; t++)
+#pragma unroll
+              for (int mt = 0; mt < MT; mt++) acc[t][mt] += __builtin_bit_cast(f32x4, pv[q][t][mt]);
+          }
+      }
+    }
+    // ---- epilogue: lane l holds token m = mt * 16 + (l & 15), output columns tile * 16 + (l >> 4) * 4 .. + 3
+    if (silu && (TW & 1)) {
+      // an odd tile count per wavefront leaves the middle gate/up pair split: wavefront 1 hands its first tile (an up
+      // tile) to wavefront 0, which holds the gate tile, through LDS
+      __syncthreads();  // everybody is done with the row buffers
+      if (wave == 1 && has_tile) {
+#pragma unroll
+        for (int mt = 0; mt < MT; mt++) xl[mt * 64 + lane] = __builtin_bit_cast(u32x4, acc[0][mt]);
+      }
+      __syncthreads();
+    }
+    if (!has_tile) return;
+    auto store_tile = [&](int otile, const f32x4 (&v)[MT]) {
+#pragma unroll
+      for (int mt = 0; mt < MT; mt++) {
+        const int m = mt * 16 + lr;
+        if (m < M) {
+          uint16_t *orow = (uint16_t *)st.out + (size_t)m * st.ld_out;
+          const uint16_t *rrow = (const uint16_t *)st.res + (size_t)m * st.ld_res;
+          float rr[4];
+#pragma unroll
+          for (int i = 0; i < 4; i++) {
+            const int n = otile * 16 + lg * 4 + i;
+            float r = v[mt][i];
+            if ((st.flags & MK_F_RES) && n < n_out) r += bf2f(rrow[n]);
+            rr[i] = r;
+          }
+          stc_bf16x4(orow, otile * 16 + lg * 4, n_out, rr);
+        }
+      }
+    };
+    if (!silu) {
+#pragma unroll
+      for (int t = 0; t < TW; t++)
+        if (tw0 + t < te) store_tile(tw0 + t, acc[t]);
+    } else {
+      // tile index relative to the range start is even for gate tiles (ranges hold whole pairs)
+#pragma unroll
+      for (int t = 0; t < TW; t++) {
+        const int ti = tw0 + t;
+        if (ti >= te || ((ti - tb) & 1)) continue;  // pairs are stored by the holder of their gate tile
+        f32x4 v[MT];
+        if (t + 1 < TW) {
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++)
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[mt][i] = silu_mul(acc[t][mt][i], acc[(t + 1) % TW][mt][i]);
+        } else {
+#pragma unroll
+          for (int mt = 0; mt < MT; mt++) {
+            const f32x4 up = __builtin_bit_cast(f32x4, xl[mt * 64 + lane]);
+#pragma unroll
+            for (int i = 0; i < 4; i++) v[mt][i] = silu_mul(acc[t][mt][i], up[i]);
+          }
+        }
+        store_tile(ti >> 1, v);
+      }
+    }
+  }
+}
+
 #ifndef MK_TUNE_NBN
 #define MK_TUNE_NBN 4
 #endif
@@ -1407,6 +1813,7 @@ __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, cha
   // are shared through the XCD's L2
   if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   __syncthreads();
+  MK_MARK(c, 0);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
   const bool silu = st.flags & MK_F_SILU;
@@ -1502,12 +1909,14 @@ __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, cha
           }
       }
     }
+    MK_MARK(c, 1);
     __syncthreads();  // previous sweep's epilogue has finished reading LDS
 #pragma unroll
     for (int t = 0; t < TG; t++)
 #pragma unroll
       for (int mt = 0; mt < MT; mt++) red[((wave * TG + t) * MT + mt) * 64 + lane] = acc[t][mt];
     __syncthreads();
+    MK_MARK(c, 2);
     // epilogue: entry (output tile u, token tile mt, lane slot l) -> 4 consecutive output columns of one token row
     const int entries = not_ * MT * 64;
     for (int e = tid; e < entries; e += MK_THREADS) {
@@ -2923,6 +3332,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
   c.sh_tok = &sh_tok[0][0];
   c.sh_ticket = sh_ticket;
   c.seq = 0;
+  c.defer_S = 0;
   c.wrote_through = false;
   if (threadIdx.x == 0) {
     sh_ticket[0] = sh_ticket[1] = 0;
@@ -2969,8 +3379,10 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
 
   for (int it = 0; it < max_iters && !c.dead; it++) {
     // ---- scheduler step on one thread of virtual workgroup 0, published through the barrier
+    long long t_sched0 = 0, t_sched1 = 0;
     if (run_scheduler) {
       barrier_wait(c);  // the previous iteration's sampled tokens are complete
+      t_sched0 = (long long)wall_clock64();
       if (c.vid == 0 && threadIdx.x == 0) {
         int ntok;
         if (run_scheduler == MK_SCHED_OFFLINE) ntok = mk_prepare_next_batch(*rtp, (int *)smem);
@@ -2979,6 +3391,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
         if (ntok == 0) rt.sched->finished = 1;
         else rt.sched->iterations++;
         if (rt.timing && rt.sched->iterations <= rt.timing_cap) rt.timing[rt.sched->iterations] = (long long)wall_clock64();
+        t_sched1 = (long long)wall_clock64();
       }
       barrier_arrive(c);
     }
@@ -3000,6 +3413,12 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       sh_tok[3][t] = ldc_i32(&rt.kv_indptr[slot]);
     }
     __syncthreads();
+    if (threadIdx.x == 0 && rt.stage_prof && run_scheduler) {
+      long long *pr = rt.stage_prof + MK_PROF_TICKS * ((size_t)c.vid * (rt.num_stages + 1) + rt.num_stages);
+      pr[0] = t_sched0;
+      pr[1] = t_sched1;
+      pr[2] = (long long)wall_clock64();
+    }
     if (M == 0 || c.dead) break;
 
     for (int s = 0; s < rt.num_stages && !c.dead; s++) {
@@ -3025,7 +3444,16 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
             const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
             const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
             const TilePlan plan = linear_tiles_plan(st, c);
-            if (plan.S >= 1) {
+            const XresPlan xp = linear_xres_plan(st, c);
+            if (xp.S >= 1 && M > 8) {
+              if (M <= 32) {
+                if (xp.tpu <= 4) stage_linear_mfma_xres<2, 2>(st, c, rt, M, xp, smem);
+                else stage_linear_mfma_xres<2, 3>(st, c, rt, M, xp, smem);
+              } else {
+                if (xp.tpu <= 4) stage_linear_mfma_xres<4, 2>(st, c, rt, M, xp, smem);
+                else stage_linear_mfma_xres<4, 3>(st, c, rt, M, xp, smem);
+              }
+            } else if (plan.S >= 1) {
               if (M <= 16) stage_linear_mfma_tiles<1>(st, c, rt, M, plan, smem);
               else if (M <= 32) stage_linear_mfma_tiles<2>(st, c, rt, M, plan, smem);
               else if (M <= 48) stage_linear_mfma_tiles<3>(st, c, rt, M, plan, smem);
@@ -3059,11 +3487,17 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       const long long t_out = (long long)wall_clock64();
       barrier_arrive(c);
       if (threadIdx.x == 0 && rt.stage_prof) {
-        long long *pr = rt.stage_prof + 4 * ((size_t)c.vid * rt.num_stages + s);
+        long long *pr = rt.stage_prof + MK_PROF_TICKS * ((size_t)c.vid * (rt.num_stages + 1) + s);
         pr[0] = t_in;
         pr[1] = c.t_wait;
         pr[2] = t_out;
         pr[3] = (long long)wall_clock64();
+#ifdef MK_TRACE
+        for (int i = 0; i < 4; i++) {
+          pr[4 + i] = c.mark[i];
+          c.mark[i] = 0;
+        }
+#endif
       }
     }
   }

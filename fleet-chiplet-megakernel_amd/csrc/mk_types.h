@@ -24,11 +24,14 @@
 //   [24 KB, 25 KB)  reduction scratch
 //   [25 KB, 32 KB)  outputs of a single-token linear, collected before they are written out
 //   [32 KB, 128 KB) routing lists of the mixture-of-experts stages, matrix-core reduction scratch
+//   the matrix-core linear that keeps its token rows resident uses [0, 128 KB) for them and the words above for its flags
+// (gfx950 gives a workgroup up to 160 KB; 156 KB dynamic + the kernel's static arrays stay below that)
 #define MK_RED_OFFSET (24 * 1024)
 #define MK_OUT_OFFSET (25 * 1024)   // [25 KB, 32 KB): outputs of a single-token linear collected before they are written out
 #define MK_MOE_OFFSET (32 * 1024)
 #define MK_MOE_X_OFFSET (40 * 1024)  // [40 KB, 128 KB): input rows of a multi-token MoE linear's (token, slot) pairs
-#define MK_LDS_BYTES (128 * 1024)
+#define MK_LDS_BYTES (156 * 1024)
+#define MK_PROF_TICKS 8
 
 enum MkOp {
   MK_OP_NONE = 0,
@@ -54,6 +57,7 @@ enum MkStageFlags {
   MK_F_EMBED_FROM_TOKENS = 64,  // EMBED: ids come from tokens[req, step+j] instead of input_tokens
   MK_F_MOE_INLINE_TOPK = 128,   // MOE_LINEAR: a single-token iteration routes inside this stage (the MOE_TOPK stage before it is multi-token only)
   MK_F_MOE_COMBINE = 256,       // MOE_LINEAR: a single-token iteration also forms res + sum_k w_k * y_k (the MOE_COMBINE stage after it is multi-token only)
+  MK_F_DEFER_SUM = 512,  // LINEAR: the next stage is a full-row NORM over this stage's output, which may be handed the K-slice partials to sum
 };
 
 #define MK_MOE_MAX_EXPERTS 256  // one thread per expert when the routing lists are built
@@ -85,6 +89,11 @@ struct MkStage {
   const void *norm_w;
   void *norm_out;
   MkWeight w;
+  // LINEAR: the same weights re-laid for the matrix cores (null: none), in 16-row tiles -- plain stages tile t = rows
+  // [16 t, 16 t + 16), SwiGLU stages tile 2j = gate rows of outputs [16 j, 16 j + 16) and tile 2j + 1 their up rows --
+  // as [tile][k / 64][2][64 lanes] 16-byte operands: lane l of (tile, step, h) holds k = 64 step + 32 h + 8 (l / 16) ..
+  // + 7 of the tile's row l % 16.  A tile is one contiguous stream of 32 k bytes.
+  const void *wpack;
   // attention
   void *k_cache, *v_cache;
   const void *q_norm_w, *k_norm_w, *cos_tab, *sin_tab;
@@ -185,5 +194,7 @@ struct MkRuntime {
   unsigned *splitk_cnt; // [workgroups][32]: arrival counter per split-K group (one 128-byte line each)
   long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end
   int timing_cap, pad0;
-  long long *stage_prof; // [workgroups][num_stages][4] ticks of the last iteration: entry, wait done, exit, arrived
+  long long *stage_prof; // [workgroups][num_stages + 1][MK_PROF_TICKS] 100 MHz ticks of the last iteration: entry, wait done, exit, arrived, then
+                         // four marks a stage may set in a build with MK_TRACE defined; the extra record holds the scheduler step:
+                         // [0] previous iteration complete, [1] batch prepared, [2] batch published to every workgroup
 };

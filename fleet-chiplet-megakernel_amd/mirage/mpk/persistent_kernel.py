@@ -723,23 +723,32 @@ class PersistentKernel:
         _capi.check(self._lib.mk_run_once(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), n,
                                           _capi.int_array(tok_slot, i32), _capi.int_array(tok_pos, i32), _capi.int_array(tok_first, i32)))
 
+    def repack_weights(self):
+        """Refresh the library's matrix-core copies of the linear weights after attached weight tensors were overwritten
+        (graphs with max_num_batched_tokens > 8 stream a tile-ordered copy made at compile time).  Not in the reference,
+        whose kernels read the attached tensors in place."""
+        _capi.check(self._lib.mk_repack_weights(self._handle))
+
     def stats(self) -> dict:
         st = _capi.MkStats()
         _capi.check(self._lib.mk_get_stats(self._handle, ctypes.byref(st)))
         return {name: getattr(st, name) for name, _ in st._fields_}
 
-    def stage_profile(self, workgroup: int = 0, raw: bool = False):
+    def stage_profile(self, workgroup: int = 0, raw: bool = False, marks: bool = False):
         """Per-stage timing of the last iteration on one virtual workgroup: list of (description, entered,
         barrier_satisfied, work_done, arrived) in microseconds relative to that workgroup's first stage (raw=True:
-        100 MHz ticks, comparable across workgroups; 0 = stage skipped)."""
-        n = self.stats()["num_stages"]
-        buf = (ctypes.c_int64 * (4 * max(1, n)))()
-        got = _capi.check(self._lib.mk_get_stage_profile(self._handle, int(workgroup), buf, n))
-        desc = self.describe_program().splitlines()
+        100 MHz ticks, comparable across workgroups; 0 = stage skipped).  The last entry, "SCHEDULER", times the scheduler
+        step that opened the iteration: (previous iteration complete, batch prepared [workgroup 0], batch published, 0).
+        marks=True returns the four in-stage marks of a library built with -DMK_TRACE instead."""
+        n = self.stats()["num_stages"] + 1
+        buf = (ctypes.c_int64 * (4 * n))()
+        fn = self._lib.mk_get_stage_marks if marks else self._lib.mk_get_stage_profile
+        got = _capi.check(fn(self._handle, int(workgroup), buf, n))
+        desc = self.describe_program().splitlines() + ["SCHEDULER"]
         if raw:
             return [(desc[i], *[int(buf[4 * i + k]) for k in range(4)]) for i in range(got)]
-        t0 = min(buf[4 * i] for i in range(got) if buf[4 * i] > 0) if got else 0
-        return [(desc[i], *[(buf[4 * i + k] - t0) * 0.01 if buf[4 * i] > 0 else -1.0 for k in range(4)]) for i in range(got)]
+        t0 = min(buf[4 * i] for i in range(got - 1) if buf[4 * i] > 0) if got > 1 else 0
+        return [(desc[i], *[(buf[4 * i + k] - t0) * 0.01 if buf[4 * i + k] > 0 else -1.0 for k in range(4)]) for i in range(got)]
 
     def finalize(self):
         assert not self.__finalized__

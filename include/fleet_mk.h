@@ -148,6 +148,13 @@ int mk_wait(mk_graph *g, void *stream, int *finished_out);
  * per kv head.  All calls on one GPU share that array: calls that overlap on one GPU race, whatever their handles or
  * streams.  Results are bit-identical to mk_enqueue_steps; per-stage timing is not recorded.  Pair with mk_wait. */
 int mk_enqueue_steps_static(mk_graph *g, void *stream, int max_iterations);
+/* No counterpart in the reference (its kernels read the attached weights in place, persistent_kernel.cuh:1966-2256).
+ * A graph with max_num_batched_tokens > 8 keeps, from mk_compile on, a second copy of every linear weight laid out in
+ * 16-row matrix-core tiles (iterations of more than eight tokens stream that copy: one contiguous stream per tile is
+ * served by HBM about a third faster than 64-byte pieces of 16 rows; single-token iterations read the attached
+ * tensors).  A caller that overwrites attached weights after mk_compile calls this to refresh the copies.  Blocking.
+ * The environment variable FLEET_MK_PACK_WEIGHTS=0 (read by mk_compile) runs without copies. */
+int mk_repack_weights(mk_graph *g);
 /* Host-driven single pass (the reference's MODE_ONEPASS / online modes, persistent_kernel.cuh:538-582): the caller
  * supplies the batch -- for each of `num_tokens` rows its batch slot, absolute position and the index of the first
  * row of the same request -- and has filled input_tokens / paged_kv_* itself.  Runs the stage program once. */
@@ -165,13 +172,19 @@ typedef struct mk_stats {
   int64_t iterations;      /* decode iterations executed since mk_init_requests */
   int64_t weight_bytes;    /* bytes of weight matrices streamed by one iteration */
   double last_launch_ms;   /* HIP-event time of the last launch's kernel, on the stream it ran on */
+  int64_t packed_weight_bytes; /* device memory the handle holds for matrix-core copies of the weights (0: none) */
 } mk_stats;
 int mk_get_stats(mk_graph *g, mk_stats *out);
 /* Device-side stage timing of the LAST decode iteration, as seen by virtual workgroup `workgroup`: for each stage four
  * 100 MHz wall-clock ticks {entered, previous stage's barrier satisfied, work done, arrival posted}.  Returns the number
- * of stages written (<= max_stages).  Counterpart of the reference's MPK_ENABLE_EVENT_TIMING ring
+ * of stages written (<= max_stages).  One record more than there are stages may be asked for: the last one times the
+ * scheduler step of that iteration {previous iteration complete, batch prepared (workgroup 0 only), batch published to
+ * this workgroup, 0}.  Counterpart of the reference's MPK_ENABLE_EVENT_TIMING ring
  * (persistent_kernel.cuh:1299-1307,2412-2429). */
 int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages);
+/* Same layout, four further ticks per stage: marks that stage code sets inside its work in a library built with
+ * -DMK_TRACE (zero in a regular build).  Used to see where a stage's time goes. */
+int mk_get_stage_marks(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages);
 /* Stage listing (one line per stage) for debugging and tests; owned by the handle. */
 int mk_describe_program(mk_graph *g, const char **text_out);
 
