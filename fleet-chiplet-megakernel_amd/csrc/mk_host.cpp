@@ -523,6 +523,12 @@ int lower_attention(mk_graph *g, size_t &i) {
     st.q_ws = g->tensors[qws_id].ptr;
     st.ld_qws = (int)g->tensors[qws_id].strides[0];
   }
+  if (!g->stages.empty()) {
+    // a plain linear whose whole output is this stage's q/k/v rows may leave its split-K sum to this stage's row fetch
+    MkStage &pl = g->stages.back();
+    if (pl.op == MK_OP_LINEAR && !(pl.flags & (MK_F_SILU | MK_F_RES)) && pl.out == st.in && pl.ld_out == st.ld_in && pl.n == (nq + 2 * nkv) * D)
+      pl.flags |= MK_F_DEFER_SUM;
+  }
   g->stages.push_back(st);
   g->stage_desc.push_back(fmt("ATTN %s -> %s q=%d kv=%d d=%d norm=%d rope=%d", tin.name.c_str(), to.name.c_str(), nq, nkv, D, !!(st.flags & MK_F_QK_NORM),
                               !!(st.flags & MK_F_ROPE)));

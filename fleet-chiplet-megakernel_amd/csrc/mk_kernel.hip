@@ -74,6 +74,7 @@ struct Ctx {
   // every row anyway, sums them (slice order, then the residual, then one rounding: the same arithmetic).
   int defer_S;            // slices left unsummed by the stage that just ran (0: none)
   int defer_rows;         // token rows per slice in the partial buffer
+  int defer_n;            // row length of the partial buffer (the producing linear's outputs)
   const float *defer_part;  // [slice][row][n] fp32
   const void *defer_res;  // residual rows of that linear (null: none)
   int defer_ld_res;
@@ -1560,6 +1561,7 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
   if (defer) {
     c.defer_S = S;
     c.defer_rows = MT * 16;
+    c.defer_n = st.n;
     c.defer_part = (const float *)rt.splitk_part;
     c.defer_res = (st.flags & MK_F_RES) ? st.res : nullptr;
     c.defer_ld_res = st.ld_res;
@@ -1830,9 +1832,15 @@ __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, cha
   const int half = st.silu_half;
   const int otg = silu ? TG / 2 : TG;  // output tiles per sweep
   f32x4 *red = (f32x4 *)smem;           // [waves][TG][MT][64]
+  // With a tile-ordered weight copy the step's two operands hold k = 64 s + 8 lg .. and 64 s + 32 + 8 lg .. (the copy's
+  // order) and a tile streams contiguously; read from the row-major weights they are the 32 contiguous bytes at
+  // k = 64 s + 16 lg.  The token rows follow the same order.
+  const bool packed = pipe && st.wpack != nullptr;
+  const int wstep = packed ? 128 : 8, whalf = packed ? 64 : 1;  // 16-byte operands between steps / between the halves
+  const int xhalf = packed ? 32 : 8;                           // elements between the halves of a token-row step
   const uint16_t *xrow[MT];
 #pragma unroll
-  for (int mt = 0; mt < MT; mt++) xrow[mt] = x + (size_t)min(mt * 16 + lr, M - 1) * ldx + lg * lgw;
+  for (int mt = 0; mt < MT; mt++) xrow[mt] = x + (size_t)min(mt * 16 + lr, M - 1) * ldx + (packed ? lg * 8 : lg * lgw);
 
   for (int ot0 = t_begin; ot0 < t_end; ot0 += otg) {
     const int not_ = min(otg, t_end - ot0);       // output tiles in this sweep
@@ -1847,7 +1855,8 @@ __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, cha
         const int g = o / half;
         vr = g * 2 * half + (o - g * half) + ((t & 1) ? half : 0);
       }
-      wrow[t] = (const uint16_t *)weight_row(st.w, vr, k8) + lg * lgw;
+      wrow[t] = packed ? (const uint16_t *)((const u32x4 *)st.wpack + (size_t)(silu ? 2 * ot + (t & 1) : ot) * (K >> 6) * 128 + lane)
+                       : (const uint16_t *)weight_row(st.w, vr, k8) + lg * lgw;
     }
     f32x4 acc[TG][MT];
 #pragma unroll
@@ -1864,13 +1873,14 @@ __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, cha
 #pragma unroll
         for (int t = 0; t < TG; t++)
           if (t < nt) {
-            aa[t][0] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k));
-            aa[t][1] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + k + 8));
+            const bf16x8 *wp = (const bf16x8 *)wrow[t] + (k >> 6) * wstep;
+            aa[t][0] = __builtin_nontemporal_load(wp);
+            aa[t][1] = __builtin_nontemporal_load(wp + whalf);
           }
 #pragma unroll
         for (int mt = 0; mt < MT; mt++) {
           bb[mt][0] = *(const bf16x8 *)(xrow[mt] + k);
-          bb[mt][1] = *(const bf16x8 *)(xrow[mt] + k + 8);
+          bb[mt][1] = *(const bf16x8 *)(xrow[mt] + k + xhalf);
         }
       };
 #pragma unroll
@@ -2834,6 +2844,25 @@ __device__ __forceinline__ void head_row_load(const uint16_t *src, int lane, flo
   x0 = bf2f(ldc_u16(src + lane));
   x1 = bf2f(ldc_u16(src + lane + 64));
 }
+// The same two elements when the producing linear left its K-slice partials unsummed: sum of the NS slices in slice
+// order, rounded to bf16 (what that linear would have stored).  `p` points at slice 0's element l of the row.
+template <int NS>
+__device__ __forceinline__ void head_row_load_slices(const float *p, size_t slice_stride, int lane, float &x0, float &x1) {
+  float a[NS], b[NS];
+#pragma unroll
+  for (int q = 0; q < NS; q++) {
+    a[q] = ldc_f32(p + q * slice_stride + lane);
+    b[q] = ldc_f32(p + q * slice_stride + lane + 64);
+  }
+  float s0 = 0.f, s1 = 0.f;
+#pragma unroll
+  for (int q = 0; q < NS; q++) {
+    s0 += a[q];
+    s1 += b[q];
+  }
+  x0 = bfround(s0);
+  x1 = bfround(s1);
+}
 __device__ __forceinline__ void head_row_finish(float x0, float x1, uint16_t *dst, const uint16_t *nw, const uint16_t *cos_row, const uint16_t *sin_row,
                                                 int flags, float eps, int lane) {
   if (flags & MK_F_QK_NORM) {
@@ -2947,6 +2976,21 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   if (have0 && wave != 0) prefetch0();
   barrier_wait(c);
   if (have0 && wave == 0) prefetch0();
+  // the q/k/v rows: stored by the producing linear, or -- when it left its K-slice partials to this stage -- summed here
+  const int dS = c.defer_S;
+  c.defer_S = 0;
+  const float *dpart = c.defer_part;
+  const size_t dn = (size_t)c.defer_n, dslice = (size_t)c.defer_rows * dn;
+  auto fetch = [&](int tok, int off, float &y0, float &y1) {
+    if (dS == 0) {
+      head_row_load((const uint16_t *)st.in + (size_t)tok * st.ld_in + off, lane, y0, y1);
+    } else {
+      const float *pp = dpart + (size_t)tok * dn + off;
+      if (dS == 2) head_row_load_slices<2>(pp, dslice, lane, y0, y1);
+      else if (dS == 4) head_row_load_slices<4>(pp, dslice, lane, y0, y1);
+      else head_row_load_slices<8>(pp, dslice, lane, y0, y1);
+    }
+  };
 
   for (int u = c.vid; u < n_units; u += c.G) {
     AttnUnit a;
@@ -2962,21 +3006,17 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     // ---- phase A: prepare q heads and the new K/V rows of this chunk, two rows per wavefront in flight
     const int n_rows = QPK + a.n_new;
     for (int row0 = wave; row0 < n_rows; row0 += 2 * MK_WAVES) {
-      float x0[2], x1[2];
-      const uint16_t *src[2];
+      float x0[2], x1[2], v0[2], v1[2];
+      int tok[2], off[2];
 #pragma unroll
       for (int r = 0; r < 2; r++) {
         const int row = row0 + r * MK_WAVES;
         if (row < n_rows) {
-          if (row < QPK) {
-            src[r] = (const uint16_t *)st.in + (size_t)t * st.ld_in + (size_t)h * (QPK + 2) * D + row * D;
-          } else {
-            const int tt = a.t0 + (a.new_lo + (row - QPK) - a.p0);
-            src[r] = (const uint16_t *)st.in + (size_t)tt * st.ld_in + (size_t)h * (QPK + 2) * D + QPK * D;
-            vnew[(row - QPK) * D + lane] = ldc_u16(src[r] + D + lane);
-            vnew[(row - QPK) * D + lane + 64] = ldc_u16(src[r] + D + lane + 64);
-          }
-          head_row_load(src[r], lane, x0[r], x1[r]);
+          const bool isq = row < QPK;
+          tok[r] = isq ? t : a.t0 + (a.new_lo + (row - QPK) - a.p0);
+          off[r] = h * (QPK + 2) * D + (isq ? row : QPK) * D;
+          fetch(tok[r], off[r], x0[r], x1[r]);
+          if (!isq) fetch(tok[r], off[r] + D, v0[r], v1[r]);  // (a V row is copied as it is)
         }
       }
 #pragma unroll
@@ -2985,6 +3025,21 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         if (row < n_rows) {
           const bool isq = row < QPK;
           const int pos = isq ? p : a.new_lo + (row - QPK);
+          if (!isq) {
+            vnew[(row - QPK) * D + lane] = (uint16_t)f2bf(v0[r]);
+            vnew[(row - QPK) * D + lane + 64] = (uint16_t)f2bf(v1[r]);
+          }
+          if (dS && a.cidx == C - 1 && tok[r] == t) {
+            // the producing linear left these rows unsummed: the chunk that owns the token's newest position also
+            // stores the token's own q/k/v rows where that linear would have
+            uint16_t *dst = (uint16_t *)st.in + (size_t)t * st.ld_in + off[r];
+            dst[lane] = (uint16_t)f2bf(x0[r]);
+            dst[lane + 64] = (uint16_t)f2bf(x1[r]);
+            if (!isq) {
+              dst[D + lane] = (uint16_t)f2bf(v0[r]);
+              dst[D + lane + 64] = (uint16_t)f2bf(v1[r]);
+            }
+          }
           head_row_finish(x0[r], x1[r], isq ? qs + row * D : knew + (row - QPK) * D, (const uint16_t *)(isq ? st.q_norm_w : st.k_norm_w),
                           (const uint16_t *)st.cos_tab + (size_t)pos * st.ld_cos, (const uint16_t *)st.sin_tab + (size_t)pos * st.ld_cos, st.flags, st.eps,
                           lane);
