@@ -206,6 +206,8 @@ class MPK:
     def run(self, prompt):
         """Offline generation of one prompt in every request slot; returns the decoded text (or the token ids when the
         model came without a tokenizer), mpk.py:336-349."""
+        if not self.is_compiled:
+            self.compile()
         self.load_new_request(prompt)
         torch.cuda.synchronize()
         self.init_per_request()

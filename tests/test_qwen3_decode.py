@@ -242,3 +242,25 @@ def test_bs1_against_torch_order_reference_decode():
     assert worst <= 0.1 and within / total >= 0.90
     assert n15 > 0 and agree15 == n15
     dec.mpk.finalize()
+
+
+@pytest.mark.parametrize("per_req,expect_prefill", [(8, 10), (64, 2)])
+def test_prefill_chunk_size_follows_max_tokens_per_request(per_req, expect_prefill):
+    """A request ingests up to max_tokens_per_request prompt tokens per iteration (the reference's MAX_TOKENS_PER_REQUEST,
+    python/mirage/mpk/persistent_kernel.py:553-560; 8 by default): an 80-token prompt takes ten iterations at 8 and two at
+    64 (the attention stage then holds up to 64 new K/V rows of one request), and the generated tokens pass the same
+    oracle check either way."""
+    from oracle.qwen3_ref import make_model_weights, make_prompt
+    cfg = _small_cfg()
+    w = make_model_weights(cfg, seed=33)
+    P, max_seq = 80, 96
+    prompt = make_prompt(cfg, P, 11)
+    dec = _decoder(cfg, w, max_num_batched_tokens=64, max_num_batched_requests=1, max_seq_length=max_seq, page_size=16, max_tokens_per_request=per_req)
+    toks, steps = dec.generate([prompt])
+    st = dec.mpk.stats()
+    assert st["aborted"] == 0
+    # the last prompt chunk's iteration also samples the first new token; the others each commit one token
+    assert st["iterations"] == expect_prefill + (max_seq - 1 - P), f"{st['iterations']} iterations"
+    assert int(steps[0]) == max_seq - 1
+    _teacher_check(cfg, w, [prompt], toks, max_seq, min_margin_hits=3)
+    dec.mpk.finalize()
