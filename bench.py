@@ -85,8 +85,10 @@ def cpu_baseline(shape, n_layers_sample=2, steps=3, context=80):
 # HBM bytes per decode step as the counters saw them (rocprofv3 --pmc FETCH_SIZE x 2.0 + WRITE_SIZE, both scaled by a
 # 1 GiB copy in the same run; the passes and their commands are in profiles/mk_persistent_kernel_qwen3-8b_bs1.md and
 # ..._bs64.md).  Counter passes cannot run inside a timed benchmark, so the bench line carries these per-step figures
-# times the steps of its launch; a batch size without a committed counter pass reports null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): 15.183e9 + 13.5e6}
+# times the steps of its launch (measured on the default 1024-step launches, whose contexts they average over; a launch of
+# another length holds different KV rows and the figure is then approximate); a batch size without a committed counter
+# pass reports null.
+MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): (15.6965e12 + 20.97e9) / 1024, ("qwen3-8b", 64): (25.928e12 + 1.4045e12) / 1024}
 
 
 def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
