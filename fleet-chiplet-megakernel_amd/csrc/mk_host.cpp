@@ -1358,7 +1358,7 @@ int mk_generate_task_graph(mk_graph *g, int num_gpus, int my_gpu_id, const char 
 // allocate = false re-runs the copy kernels into the existing buffers (the caller changed weights after compiling).
 static int pack_weights(mk_graph *g, bool allocate) {
   const char *env = getenv("FLEET_MK_PACK_WEIGHTS");
-  if (g->cfg.max_num_batched_tokens <= 8 || (env && atoi(env) == 0)) return 0;
+  if (g->cfg.max_num_batched_tokens < 2 || (env && atoi(env) == 0)) return 0;
   for (auto &st : g->stages) {
     if (st.op != MK_OP_LINEAR || (st.k & 63) || st.k < 64) continue;
     const bool silu = st.flags & MK_F_SILU;

@@ -1189,8 +1189,11 @@ __device__ __forceinline__ void stage_linear_small(CStage &st, Ctx &c, int M, ch
 
 // Whether the few-token form can run this stage: reduction length with a tuned instantiation, token rows within the
 // LDS window above MK_MOE_X_OFFSET, collected outputs within the window below MK_MOE_OFFSET.
+#ifndef MK_TUNE_SMALL_MAX
+#define MK_TUNE_SMALL_MAX 2
+#endif
 __device__ __forceinline__ bool linear_small_ok(CStage &st, const Ctx &c, int M) {
-  if (M > 8 || (st.k != 4096 && st.k != 2048)) return false;
+  if (M > MK_TUNE_SMALL_MAX || (st.k != 4096 && st.k != 2048)) return false;
   const int n_out = (st.flags & MK_F_SILU) ? st.n / 2 : st.n;
   return (size_t)M * st.k * 2 <= (size_t)(MK_LDS_BYTES - MK_MOE_X_OFFSET) && (size_t)M * (n_out / c.G + 1) * 2 <= (size_t)MK_MOE_OFFSET;
 }
@@ -3500,7 +3503,7 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
             const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
             const TilePlan plan = linear_tiles_plan(st, c);
             const XresPlan xp = linear_xres_plan(st, c);
-            if (xp.S >= 1 && M > 8) {
+            if (xp.S >= 1 && M > MK_TUNE_SMALL_MAX) {
               if (M <= 32) {
                 if (xp.tpu <= 4) stage_linear_mfma_xres<2, 2>(st, c, rt, M, xp, smem);
                 else stage_linear_mfma_xres<2, 3>(st, c, rt, M, xp, smem);
