@@ -140,7 +140,7 @@ def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s", "frac": round(achieved / HBM_PEAK_GBS, 4),
                      "traffic": None if per_step is None else int(per_step * K),
                      "traffic_source": None if per_step is None else "per-step FETCH_SIZE/WRITE_SIZE counter passes in profiles/ x steps of this launch",
-                     "kernel": "mk_persistent_kernel", "kernel_ms_per_launch": round(kernel_ms, 3), "algorithmic_bytes_per_launch": bytes_total},
+                     "kernel": "mk_persistent_kernel_m1" if B == 1 else "mk_persistent_kernel", "kernel_ms_per_launch": round(kernel_ms, 3), "algorithmic_bytes_per_launch": bytes_total},
     }
 
 

@@ -1049,6 +1049,11 @@ int upload_runtime(mk_graph *g) {
 }
 
 // `rt` is the runtime block the kernel receives by value; `cleared_by_caller`: its barrier state has been zeroed already
+// graphs that never run more than one token per iteration use the kernel instantiated for exactly that
+static const void *kernel_of(const mk_graph *g) {
+  return g->cfg.max_num_batched_tokens == 1 ? (const void *)mk_persistent_kernel_m1 : (const void *)mk_persistent_kernel;
+}
+
 int do_launch(mk_graph *g, hipStream_t stream, int max_iters, int run_scheduler, const MkRuntime *rt = nullptr, bool cleared_by_caller = false) {
   if (!g->compiled) return fail(MK_ESTATE, "mk_compile has not been called");
   if (g->launch_pending) return fail(MK_ESTATE, "a launch is still pending: call mk_wait first");
@@ -1058,7 +1063,7 @@ int do_launch(mk_graph *g, hipStream_t stream, int max_iters, int run_scheduler,
   const MkRuntime *rtp = g->d_rt;
   void *args[] = {(void *)rt, (void *)&rtp, (void *)&max_iters, (void *)&run_scheduler};
   HIP_TRY(hipEventRecord(g->ev0, stream));
-  HIP_TRY(hipLaunchCooperativeKernel((const void *)mk_persistent_kernel, dim3(g->G), dim3(MK_THREADS), args, MK_LDS_BYTES, stream));
+  HIP_TRY(hipLaunchCooperativeKernel(kernel_of(g), dim3(g->G), dim3(MK_THREADS), args, MK_LDS_BYTES, stream));
   HIP_TRY(hipEventRecord(g->ev1, stream));
   g->launch_pending = true;
   g->pending_sync = rt->sync;
@@ -1158,7 +1163,7 @@ int mk_graph_create(const mk_config *cfg, mk_graph **out) {
       return fail(MK_EINVAL, "max_num_pages=%d cannot back %d concurrent requests of up to %lld pages each (max_seq_length=%d, page_size=%d)",
                   cfg->max_num_pages, cfg->max_num_batched_requests, (long long)per_req, cfg->max_seq_length, cfg->page_size);
   }
-  if (cfg->max_num_pages > (MK_LDS_BYTES / 4)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 4);
+  if (cfg->max_num_pages > (MK_LDS_BYTES / 8)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 8);
   if (cfg->device < 0) {
     mk_graph *g = new mk_graph();
     g->cfg = *cfg;
@@ -1404,9 +1409,9 @@ int mk_compile(mk_graph *g) {
   rc = build_task_graph_json(g);
   if (rc) return rc;
   // co-residency: every workgroup must be resident for the in-kernel barriers to make progress
-  HIP_TRY(hipFuncSetAttribute((const void *)mk_persistent_kernel, hipFuncAttributeMaxDynamicSharedMemorySize, MK_LDS_BYTES));
+  HIP_TRY(hipFuncSetAttribute(kernel_of(g), hipFuncAttributeMaxDynamicSharedMemorySize, MK_LDS_BYTES));
   int per_cu = 0;
-  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, (const void *)mk_persistent_kernel, MK_THREADS, MK_LDS_BYTES));
+  HIP_TRY(hipOccupancyMaxActiveBlocksPerMultiprocessor(&per_cu, kernel_of(g), MK_THREADS, MK_LDS_BYTES));
   if (per_cu < 1 || g->G > per_cu * g->num_cus) return fail(MK_EINVAL, "grid of %d workgroups cannot be co-resident (%d per CU x %d CUs)", g->G, per_cu, g->num_cus);
   MkRuntime &rt = g->h_rt;
   rt.num_stages = (int)g->stages.size();

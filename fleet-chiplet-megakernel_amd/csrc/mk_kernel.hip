@@ -303,7 +303,7 @@ __device__ __forceinline__ void barrier_wait(Ctx &c) {
 // (running requests first, then new prefills).  Same observable behaviour on the ten meta
 // tensors as the reference's MODE_OFFLINE prepare_next_batch (persistent_kernel.cuh:380-536).
 // Runs on one thread.  Returns the number of tokens scheduled.
-__device__ int mk_prepare_next_batch(const MkRuntime &rt, int *scratch_pages) {
+__device__ __attribute__((noinline)) int mk_prepare_next_batch(const MkRuntime &rt, int *scratch_pages) {
   MkSched *sc = rt.sched;
   const int R = rt.max_requests, B = rt.max_tokens, PS = rt.page_size, NP = rt.max_pages;
   int head = sc->page_queue_head, tail = sc->page_queue_tail;
@@ -406,13 +406,167 @@ __device__ int mk_prepare_next_batch(const MkRuntime &rt, int *scratch_pages) {
   return ntok;
 }
 
+// The same step on one wavefront: lane i owns batch slot i (at most 64 slots) in the phases that walk the old batch, and
+// candidate request next_request_id + i when new requests are admitted.  What the sequential version carries from slot
+// to slot are running sums -- tokens scheduled so far (saturating at the iteration's token budget), pages in the
+// compacted table, pages taken from / returned to the ring -- and those are wavefront prefix sums:
+//   tokens before slot i = min(sum of the earlier slots' wishes, B)   (a saturating sum of non-negative terms)
+// so every lane derives exactly the values the sequential loop would have reached at its slot; the result is identical
+// entry for entry (checked against the C restatement after every iteration by the GPU scheduler tests).
+// Each lane's dependent loads (request id -> step -> token row) then overlap with the other lanes', which is what the
+// sequential version spends its time on (about 1.8 us per occupied slot).  `lds` holds the page-table snapshot
+// ([0, NP)) and the pages retired in this step in ring order ([NP, 2 NP)): a page returned by one lane and handed out
+// again by another in the same step goes through LDS, never through a store and a load of different lanes.
+__device__ __forceinline__ int wave_incl_scan(int v, int lane) {
+#pragma unroll
+  for (int o = 1; o < 64; o <<= 1) {
+    const int u = __builtin_amdgcn_ds_bpermute(((lane - o) & 63) << 2, v);
+    if (lane >= o) v += u;
+  }
+  return v;
+}
+__device__ __forceinline__ int wave_bcast(int v, int src) { return __builtin_amdgcn_readlane(v, src); }
+
+__device__ __attribute__((noinline)) int mk_prepare_next_batch_wave(const MkRuntime &rt, int *lds, int lane) {
+  MkSched *sc = rt.sched;
+  const int R = rt.max_requests, B = rt.max_tokens, PS = rt.page_size, NP = rt.max_pages;
+  int *snap = lds, *freed = lds + NP;
+  const int head0 = sc->page_queue_head, tail0 = sc->page_queue_tail;
+  const int old_pages = rt.kv_indptr[R];
+  // 1. commit the previous iteration's outputs, find the requests that retire
+  const bool slot = lane < R;
+  int req = slot ? rt.request_ids[lane] : -1;
+  int st = 0, plen = 0, k0 = 0, k1 = 0;
+  bool retire = false;
+  if (req >= 0) {
+    st = rt.step[req];
+    const int q0 = rt.qo_indptr[lane];
+    const int n = rt.qo_indptr[lane + 1] - q0;
+    plen = rt.prompt_lengths[req];
+    k0 = rt.kv_indptr[lane];
+    k1 = rt.kv_indptr[lane + 1];
+    for (int j = 0; j < n; j++) {
+      const int pos = st + j + 1;
+      if (pos >= plen && pos < rt.max_seq) rt.tokens[(long long)req * rt.max_seq + pos] = rt.output_tokens[q0 + j];
+    }
+    st += n;
+    rt.step[req] = st;
+    const bool full = st + 1 >= rt.max_seq;
+    const bool eos = st >= plen && rt.tokens[(long long)req * rt.max_seq + st] == rt.eos_token_id;
+    retire = full || eos;
+  }
+  // 2. snapshot the page table; retired pages go back to the ring in slot order
+  for (int i = lane; i < old_pages; i += 64) snap[i] = rt.kv_indices[i];
+  const int rp = retire ? k1 - k0 : 0;
+  const int rp_incl = wave_incl_scan(rp, lane);
+  const int n_freed = wave_bcast(rp_incl, 63);
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  for (int j = 0; j < rp; j++) {
+    const int pg = snap[k0 + j], at = rp_incl - rp + j;
+    freed[at] = pg;
+    rt.page_queue[(tail0 + at) % NP] = pg;
+  }
+  __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup");
+  __builtin_amdgcn_wave_barrier();
+  __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup");
+  const int avail0 = tail0 - head0;  // pages the ring held before this step
+  auto ring_page = [&](int a) -> int {  // the a-th page handed out in this step
+    return a < avail0 ? rt.page_queue[(head0 + a) % NP] : freed[a - avail0];
+  };
+  // 3. running requests keep their slot order, compacted over retired slots
+  const bool alive = req >= 0 && !retire;
+  const unsigned long long alive_mask = __ballot(alive);
+  const int rank = __popcll(alive_mask & ((1ull << lane) - 1ull));
+  const int nrun = __popcll(alive_mask);
+  const int wish = alive ? (plen - st > 0 ? min(plen - st, rt.max_new_per_req) : 1) : 0;
+  const int wish_incl = wave_incl_scan(wish, lane);
+  const int tok0 = min(wish_incl - wish, B), n = min(wish_incl, B) - tok0;
+  const int had = alive ? k1 - k0 : 0;
+  const int need = alive ? (st + n + PS - 1) / PS : 0;
+  const int need_incl = wave_incl_scan(need, lane);
+  const int fresh = need > had ? need - had : 0;
+  const int fresh_incl = wave_incl_scan(fresh, lane);
+  if (alive) {
+    const int page0 = need_incl - need, a0 = fresh_incl - fresh;
+    rt.request_ids[rank] = req;
+    rt.qo_indptr[rank] = tok0;
+    rt.kv_indptr[rank] = page0;
+    for (int j = 0; j < n; j++) {
+      rt.input_tokens[tok0 + j] = rt.tokens[(long long)req * rt.max_seq + st + j];
+      rt.tok_slot[tok0 + j] = rank;
+      rt.tok_pos[tok0 + j] = st + j;
+      rt.tok_first[tok0 + j] = tok0;
+    }
+    const int last = (st + n) % PS;
+    rt.kv_last_page_len[rank] = last == 0 ? PS : last;
+    for (int j = 0; j < had && j < need; j++) rt.kv_indices[page0 + j] = snap[k0 + j];
+    for (int j = had; j < need; j++) rt.kv_indices[page0 + j] = ring_page(a0 + j - had);
+  }
+  int ntok = min(wave_bcast(wish_incl, 63), B);
+  int npage = wave_bcast(need_incl, 63);
+  int taken = wave_bcast(fresh_incl, 63);
+  int nreq = nrun;
+  // 4. admit new requests while there is room: lane k looks at request next_request_id + k
+  {
+    const int next = sc->next_request_id;
+    const int cand = next + lane;
+    const bool valid = nreq + lane < R && cand < rt.total_requests;
+    const int cplen = valid ? rt.prompt_lengths[cand] : 0;
+    const int cwish = valid ? min(cplen, rt.max_new_per_req) : 0;
+    const int cw_incl = wave_incl_scan(cwish, lane);
+    // the sequential loop reaches candidate k only while the budget is not exhausted, and stops at the first request
+    // that does not exist; candidates are valid in a prefix of the lanes, so "admitted" is a prefix too
+    const bool admit = valid && ntok + (cw_incl - cwish) < B;
+    const int cn = admit ? min(cwish, B - (ntok + cw_incl - cwish)) : 0;
+    const int cneed = admit ? (cn + PS - 1) / PS : 0;
+    const int cneed_incl = wave_incl_scan(cneed, lane);
+    const int n_admit = __popcll(__ballot(admit));
+    if (admit) {
+      const int s_ = nreq + lane, tok0c = ntok + cw_incl - cwish, page0 = npage + cneed_incl - cneed, a0 = taken + cneed_incl - cneed;
+      rt.request_ids[s_] = cand;
+      rt.qo_indptr[s_] = tok0c;
+      rt.kv_indptr[s_] = page0;
+      for (int j = 0; j < cn; j++) {
+        rt.input_tokens[tok0c + j] = rt.tokens[(long long)cand * rt.max_seq + j];
+        rt.tok_slot[tok0c + j] = s_;
+        rt.tok_pos[tok0c + j] = j;
+        rt.tok_first[tok0c + j] = tok0c;
+      }
+      const int last = cn % PS;
+      rt.kv_last_page_len[s_] = last == 0 ? PS : last;
+      for (int j = 0; j < cneed; j++) rt.kv_indices[page0 + j] = ring_page(a0 + j);
+    }
+    const int cn_incl = wave_incl_scan(cn, lane);
+    ntok += wave_bcast(cn_incl, 63);
+    npage += wave_bcast(cneed_incl, 63);
+    taken += wave_bcast(cneed_incl, 63);
+    nreq += n_admit;
+    if (lane == 0) sc->next_request_id = next + n_admit;
+  }
+  // 5. clear unused slots
+  for (int i = nreq + lane; i < R; i += 64) rt.request_ids[i] = -1;
+  for (int i = nreq + lane; i <= R; i += 64) {
+    rt.qo_indptr[i] = ntok;
+    rt.kv_indptr[i] = npage;
+  }
+  if (lane == 0) {
+    sc->page_queue_head = head0 + taken;
+    sc->page_queue_tail = tail0 + n_freed;
+    sc->num_tokens = ntok;
+    sc->num_reqs = nreq;
+  }
+  return ntok;
+}
+
 // Batch description for a launch whose batch the HOST prepared (the reference's MODE_ONLINE_NOTOKEN, one pass per launch,
 // persistent_kernel.cuh:570-582, and MODE_ONEPASS): the caller has filled input_tokens, qo_indptr, paged_kv_indptr,
 // paged_kv_indices and paged_kv_last_page_len the way the reference's attention tasks read them -- request slot i owns
 // rows [qo_indptr[i], qo_indptr[i+1]) and its sequence, new tokens included, is (pages - 1) * page_size + last_page_len
 // long, so its rows sit at the last positions of that sequence.  Derives the per-row slot / position / first-row arrays
 // on the device (no host round trip, so a serving loop can enqueue launches back to back).  Runs on one thread.
-__device__ int mk_batch_from_meta(const MkRuntime &rt) {
+__device__ __attribute__((noinline)) int mk_batch_from_meta(const MkRuntime &rt) {
   const int R = rt.max_requests, B = rt.max_tokens;
   int ntok = 0;
   for (int i = 0; i < R; i++) {
@@ -439,7 +593,7 @@ __device__ int mk_batch_from_meta(const MkRuntime &rt) {
 // max_seq_length or the token after it is the EOS id -- the reference's test, on the step value from before the
 // advance.  What the reference leaves to the host and is done here instead: the page table of the one request
 // (identity: page j of the ring is page j of the sequence) and the qo / kv index arrays.  Runs on one thread.
-__device__ int mk_online_next_batch(const MkRuntime &rt) {
+__device__ __attribute__((noinline)) int mk_online_next_batch(const MkRuntime &rt) {
   MkSched *sc = rt.sched;
   const int PS = rt.page_size;
   int step = rt.step[0];
@@ -3369,8 +3523,96 @@ __device__ __forceinline__ void stage_argmax_reduce(CStage &st, Ctx &c, const Mk
 }
 
 // ----------------------------------------------------------------------------- the kernel
-extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel(const MkRuntime rt, const MkRuntime *rtp, int max_iters,
-                                                                                int run_scheduler) {
+// One pass over the stage program for the M tokens of this iteration.
+template <int MAXM>
+__device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, const int M, char *smem) {
+    for (int s = 0; s < rt.num_stages && !c.dead; s++) {
+      CStage &st = ((CStage *)(unsigned long long)rt.stages)[s];
+      const int op = st.op, flags = st.flags;
+      if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
+      if ((flags & MK_F_ONLY_MULTI) && op == MK_OP_NORM && s + 1 < rt.num_stages) {
+        // the few-token linear normalises its rows itself
+        CStage &nx = ((CStage *)(unsigned long long)rt.stages)[s + 1];
+        if (nx.op == MK_OP_LINEAR && (nx.flags & MK_F_NORM) && nx.in == st.in && linear_small_ok(nx, c, M)) continue;
+      }
+      const long long t_in = (long long)wall_clock64();
+      switch (op) {
+        case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
+        case MK_OP_NORM: stage_norm(st, c, M, smem); break;
+        case MK_OP_LINEAR:
+          if constexpr (MAXM == 1) stage_linear_m1(st, c, smem);
+          else if (M == 1) stage_linear_m1(st, c, smem);
+          else if (linear_small_ok(st, c, M)) {
+            if (M <= 2) stage_linear_small_dispatch<2>(st, c, M, smem);
+            else if (M <= 4) stage_linear_small_dispatch<4>(st, c, M, smem);
+            else stage_linear_small_dispatch<8>(st, c, M, smem);
+          } else {
+            const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
+            const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
+            const TilePlan plan = linear_tiles_plan(st, c);
+            const XresPlan xp = linear_xres_plan(st, c);
+            if (xp.S >= 1 && M > MK_TUNE_SMALL_MAX) {
+              if (M <= 32) {
+                if (xp.tpu <= 4) stage_linear_mfma_xres<2, 2>(st, c, rt, M, xp, smem);
+                else stage_linear_mfma_xres<2, 3>(st, c, rt, M, xp, smem);
+              } else {
+                if (xp.tpu <= 4) stage_linear_mfma_xres<4, 2>(st, c, rt, M, xp, smem);
+                else stage_linear_mfma_xres<4, 3>(st, c, rt, M, xp, smem);
+              }
+            } else if (plan.S >= 1) {
+              if (M <= 16) stage_linear_mfma_tiles<1>(st, c, rt, M, plan, smem);
+              else if (M <= 32) stage_linear_mfma_tiles<2>(st, c, rt, M, plan, smem);
+              else if (M <= 48) stage_linear_mfma_tiles<3>(st, c, rt, M, plan, smem);
+              else stage_linear_mfma_tiles<4>(st, c, rt, M, plan, smem);
+            } else if (narrow) {
+              if (M <= 16) stage_linear_mfma<1, 2, 2 * MK_TUNE_NBN>(st, c, M, smem);
+              else if (M <= 32) stage_linear_mfma<2, 2, MK_TUNE_NBN + MK_TUNE_NBN / 2>(st, c, M, smem);
+              else if (M <= 48) stage_linear_mfma<3, 2, MK_TUNE_NBN>(st, c, M, smem);
+              else stage_linear_mfma<4, 2, MK_TUNE_NBN>(st, c, M, smem);
+            } else {
+              if (M <= 16) stage_linear_mfma<1, 6, 2>(st, c, M, smem);
+              else if (M <= 32) stage_linear_mfma<2, 6, 2>(st, c, M, smem);
+              else if (M <= 48) stage_linear_mfma<3, 6, 2>(st, c, M, smem);
+              else stage_linear_mfma<4, 6, 2>(st, c, M, smem);
+            }
+          }
+          break;
+        case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
+        case MK_OP_ATTN:
+          if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4>(st, c, rt, M, smem);
+          else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8>(st, c, rt, M, smem);
+          else barrier_wait(c);
+          break;
+        case MK_OP_MOE_TOPK: stage_moe_topk(st, c, M); break;
+        case MK_OP_MOE_LINEAR: stage_moe_linear(st, c, M, smem); break;
+        case MK_OP_MOE_COMBINE: stage_moe_combine(st, c, M); break;
+        case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, rt, M, smem); break;
+        case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, rt, M); break;
+        default: barrier_wait(c); break;
+      }
+      const long long t_out = (long long)wall_clock64();
+      barrier_arrive(c);
+      if (threadIdx.x == 0 && rt.stage_prof) {
+        long long *pr = rt.stage_prof + MK_PROF_TICKS * ((size_t)c.vid * (rt.num_stages + 1) + s);
+        pr[0] = t_in;
+        pr[1] = c.t_wait;
+        pr[2] = t_out;
+        pr[3] = (long long)wall_clock64();
+#ifdef MK_TRACE
+        for (int i = 0; i < 4; i++) {
+          pr[4 + i] = c.mark[i];
+          c.mark[i] = 0;
+        }
+#endif
+      }
+    }
+}
+
+// The kernel body, instantiated twice: MAXM = 1 for graphs that never run more than one token per iteration (every
+// multi-token stage form is compiled out, so the single-token loops get the register file to themselves), and the
+// general one.
+template <int MAXM>
+__device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRuntime *rtp, int max_iters, int run_scheduler) {
   extern __shared__ __attribute__((aligned(16))) char smem[];
   __shared__ int sh_bcast[4];
   __shared__ int sh_quota[10];
@@ -3441,9 +3683,14 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
     if (run_scheduler) {
       barrier_wait(c);  // the previous iteration's sampled tokens are complete
       t_sched0 = (long long)wall_clock64();
+      // a handful of slots: one thread walks them; more: a wavefront, one lane per slot
+      const bool wave_sched = run_scheduler == MK_SCHED_OFFLINE && rt.max_requests > 2;
+      int ntok_w = 0;
+      if (c.vid == 0 && threadIdx.x < 64 && wave_sched) ntok_w = mk_prepare_next_batch_wave(*rtp, (int *)smem, threadIdx.x);
       if (c.vid == 0 && threadIdx.x == 0) {
         int ntok;
-        if (run_scheduler == MK_SCHED_OFFLINE) ntok = mk_prepare_next_batch(*rtp, (int *)smem);
+        if (wave_sched) ntok = ntok_w;
+        else if (run_scheduler == MK_SCHED_OFFLINE) ntok = mk_prepare_next_batch(*rtp, (int *)smem);
         else if (run_scheduler == MK_SCHED_ONLINE) ntok = mk_online_next_batch(*rtp);
         else ntok = mk_batch_from_meta(*rtp);
         if (ntok == 0) rt.sched->finished = 1;
@@ -3461,7 +3708,8 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       sh_bcast[0] = ldc_i32(&rt.sched->num_tokens);
     }
     __syncthreads();
-    const int M = __builtin_amdgcn_readfirstlane(sh_bcast[0]);
+    const int Mrt = __builtin_amdgcn_readfirstlane(sh_bcast[0]);
+    const int M = MAXM == 1 ? (Mrt > 0 ? 1 : 0) : Mrt;
     // token metadata of this iteration, read once (it is on the critical path of every attention stage otherwise)
     if ((int)threadIdx.x < M) {
       const int t = threadIdx.x, slot = ldc_i32(&rt.tok_slot[t]);
@@ -3478,87 +3726,19 @@ extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel
       pr[2] = (long long)wall_clock64();
     }
     if (M == 0 || c.dead) break;
-
-    for (int s = 0; s < rt.num_stages && !c.dead; s++) {
-      CStage &st = ((CStage *)(unsigned long long)rt.stages)[s];
-      const int op = st.op, flags = st.flags;
-      if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
-      if ((flags & MK_F_ONLY_MULTI) && op == MK_OP_NORM && s + 1 < rt.num_stages) {
-        // the few-token linear normalises its rows itself
-        CStage &nx = ((CStage *)(unsigned long long)rt.stages)[s + 1];
-        if (nx.op == MK_OP_LINEAR && (nx.flags & MK_F_NORM) && nx.in == st.in && linear_small_ok(nx, c, M)) continue;
-      }
-      const long long t_in = (long long)wall_clock64();
-      switch (op) {
-        case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
-        case MK_OP_NORM: stage_norm(st, c, M, smem); break;
-        case MK_OP_LINEAR:
-          if (M == 1) stage_linear_m1(st, c, smem);
-          else if (linear_small_ok(st, c, M)) {
-            if (M <= 2) stage_linear_small_dispatch<2>(st, c, M, smem);
-            else if (M <= 4) stage_linear_small_dispatch<4>(st, c, M, smem);
-            else stage_linear_small_dispatch<8>(st, c, M, smem);
-          } else {
-            const int wt = (((flags & MK_F_SILU) ? st.n / 2 : st.n) + 15) / 16;  // output tiles of the stage
-            const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
-            const TilePlan plan = linear_tiles_plan(st, c);
-            const XresPlan xp = linear_xres_plan(st, c);
-            if (xp.S >= 1 && M > MK_TUNE_SMALL_MAX) {
-              if (M <= 32) {
-                if (xp.tpu <= 4) stage_linear_mfma_xres<2, 2>(st, c, rt, M, xp, smem);
-                else stage_linear_mfma_xres<2, 3>(st, c, rt, M, xp, smem);
-              } else {
-                if (xp.tpu <= 4) stage_linear_mfma_xres<4, 2>(st, c, rt, M, xp, smem);
-                else stage_linear_mfma_xres<4, 3>(st, c, rt, M, xp, smem);
-              }
-            } else if (plan.S >= 1) {
-              if (M <= 16) stage_linear_mfma_tiles<1>(st, c, rt, M, plan, smem);
-              else if (M <= 32) stage_linear_mfma_tiles<2>(st, c, rt, M, plan, smem);
-              else if (M <= 48) stage_linear_mfma_tiles<3>(st, c, rt, M, plan, smem);
-              else stage_linear_mfma_tiles<4>(st, c, rt, M, plan, smem);
-            } else if (narrow) {
-              if (M <= 16) stage_linear_mfma<1, 2, 2 * MK_TUNE_NBN>(st, c, M, smem);
-              else if (M <= 32) stage_linear_mfma<2, 2, MK_TUNE_NBN + MK_TUNE_NBN / 2>(st, c, M, smem);
-              else if (M <= 48) stage_linear_mfma<3, 2, MK_TUNE_NBN>(st, c, M, smem);
-              else stage_linear_mfma<4, 2, MK_TUNE_NBN>(st, c, M, smem);
-            } else {
-              if (M <= 16) stage_linear_mfma<1, 6, 2>(st, c, M, smem);
-              else if (M <= 32) stage_linear_mfma<2, 6, 2>(st, c, M, smem);
-              else if (M <= 48) stage_linear_mfma<3, 6, 2>(st, c, M, smem);
-              else stage_linear_mfma<4, 6, 2>(st, c, M, smem);
-            }
-          }
-          break;
-        case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
-        case MK_OP_ATTN:
-          if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4>(st, c, rt, M, smem);
-          else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8>(st, c, rt, M, smem);
-          else barrier_wait(c);
-          break;
-        case MK_OP_MOE_TOPK: stage_moe_topk(st, c, M); break;
-        case MK_OP_MOE_LINEAR: stage_moe_linear(st, c, M, smem); break;
-        case MK_OP_MOE_COMBINE: stage_moe_combine(st, c, M); break;
-        case MK_OP_ARGMAX_PARTIAL: stage_argmax_partial(st, c, rt, M, smem); break;
-        case MK_OP_ARGMAX_REDUCE: stage_argmax_reduce(st, c, rt, M); break;
-        default: barrier_wait(c); break;
-      }
-      const long long t_out = (long long)wall_clock64();
-      barrier_arrive(c);
-      if (threadIdx.x == 0 && rt.stage_prof) {
-        long long *pr = rt.stage_prof + MK_PROF_TICKS * ((size_t)c.vid * (rt.num_stages + 1) + s);
-        pr[0] = t_in;
-        pr[1] = c.t_wait;
-        pr[2] = t_out;
-        pr[3] = (long long)wall_clock64();
-#ifdef MK_TRACE
-        for (int i = 0; i < 4; i++) {
-          pr[4 + i] = c.mark[i];
-          c.mark[i] = 0;
-        }
-#endif
-      }
-    }
+    run_stage_program<MAXM>(rt, c, MAXM == 1 ? 1 : M, smem);
   }
   barrier_wait(c);  // drain: nobody leaves while another workgroup may still poll
   if (c.vid == 0 && threadIdx.x == 0 && rt.timing) rt.timing[0] = (long long)wall_clock64();
+}
+
+
+extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel(const MkRuntime rt, const MkRuntime *rtp, int max_iters,
+                                                                                int run_scheduler) {
+  mk_kernel_body<MK_MAX_TOKENS>(rt, rtp, max_iters, run_scheduler);
+}
+// the same for graphs with max_num_batched_tokens == 1
+extern "C" __global__ __launch_bounds__(MK_THREADS, 1) void mk_persistent_kernel_m1(const MkRuntime rt, const MkRuntime *rtp, int max_iters,
+                                                                                   int run_scheduler) {
+  mk_kernel_body<1>(rt, rtp, max_iters, run_scheduler);
 }
