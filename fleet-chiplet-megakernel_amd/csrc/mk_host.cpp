@@ -1107,8 +1107,11 @@ constexpr size_t SS_CLEARED_END = SS_ATTN_CNT + align256((size_t)MK_STATIC_MAX_I
 constexpr size_t SS_ARGMAX_PV = SS_CLEARED_END;
 constexpr size_t SS_ARGMAX_PI = SS_ARGMAX_PV + align256((size_t)MK_MAX_TOKENS * MK_STATIC_MAX_WG * sizeof(float));
 constexpr size_t SS_ATTN_PART = SS_ARGMAX_PI + align256((size_t)MK_MAX_TOKENS * MK_STATIC_MAX_WG * sizeof(int));
-constexpr size_t SS_SPLITK_PART = SS_ATTN_PART + align256((size_t)(MK_STATIC_MAX_ITEMS + MK_ATTN_MAX_CHUNKS) * MK_STATIC_MAX_QPK * MK_ATTN_PSTRIDE * sizeof(float));
-constexpr size_t MK_STATIC_SCRATCH_BYTES = SS_SPLITK_PART + (size_t)MK_STATIC_MAX_WG * 4 * 4 * 4 * 64 * 16;  // about 19.7 MB
+// q-head partials of the attention stages: units of one kv head (up to 8 q heads each), or -- iterations of many tokens --
+// one unit per workgroup over all heads of a token (up to 32 q heads)
+constexpr size_t MK_STATIC_ATTN_HEADS = std::max<size_t>((size_t)(MK_STATIC_MAX_ITEMS + MK_ATTN_MAX_CHUNKS) * MK_STATIC_MAX_QPK, (size_t)(MK_STATIC_MAX_WG + MK_ATTN_MAX_CHUNKS) * 32);
+constexpr size_t SS_SPLITK_PART = SS_ATTN_PART + align256(MK_STATIC_ATTN_HEADS * MK_ATTN_PSTRIDE * sizeof(float));
+constexpr size_t MK_STATIC_SCRATCH_BYTES = SS_SPLITK_PART + (size_t)MK_STATIC_MAX_WG * 4 * 4 * 4 * 64 * 16;  // about 22.8 MB
 
 static __device__ __align__(256) unsigned char scratch[MK_STATIC_SCRATCH_BYTES];
 
@@ -1163,6 +1166,9 @@ int mk_graph_create(const mk_config *cfg, mk_graph **out) {
       return fail(MK_EINVAL, "max_num_pages=%d cannot back %d concurrent requests of up to %lld pages each (max_seq_length=%d, page_size=%d)",
                   cfg->max_num_pages, cfg->max_num_batched_requests, (long long)per_req, cfg->max_seq_length, cfg->page_size);
   }
+  if (((int64_t)cfg->max_seq_length + cfg->page_size - 1) / cfg->page_size > MK_ATTN_MAX_REQ_PAGES)
+    return fail(MK_EINVAL, "max_seq_length=%d over page_size=%d is more than %d pages per request (the attention stage keeps a request's page list in LDS)",
+                cfg->max_seq_length, cfg->page_size, MK_ATTN_MAX_REQ_PAGES);
   if (cfg->max_num_pages > (MK_LDS_BYTES / 8)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 8);
   if (cfg->device < 0) {
     mk_graph *g = new mk_graph();
@@ -1464,9 +1470,12 @@ int mk_compile(mk_graph *g) {
   rt.attn_part = nullptr;
   for (auto &s : g->stages)
     if (s.op == MK_OP_ATTN) {
+      // units of one kv head: max(G, tokens * kv heads) of q/kv heads each; units of all heads: G of all q heads each
       const size_t units = (size_t)std::max(g->G, rt.max_tokens * s.num_kv_heads) + MK_ATTN_MAX_CHUNKS;
       const int qpk = s.num_q_heads / s.num_kv_heads;
-      if ((rc = dev_alloc(g, &p, units * qpk * MK_ATTN_PSTRIDE * sizeof(float), false))) return rc;
+      const size_t heads = std::max(units * qpk, (size_t)(g->G + MK_ATTN_MAX_CHUNKS) * s.num_q_heads);
+      rt.attn_part_cap = rt.attn_part_cap ? std::min<int>(rt.attn_part_cap, (int)heads) : (int)heads;
+      if ((rc = dev_alloc(g, &p, heads * MK_ATTN_PSTRIDE * sizeof(float), false))) return rc;
       s.aux0 = p;
       s.aux1 = rt.attn_cnt + g->attn_cnt_n / 2;
     }
@@ -1548,6 +1557,7 @@ int mk_enqueue_steps_static(mk_graph *g, void *stream, int max_iterations) {
   rt.argmax_pv = (float *)(base + SS_ARGMAX_PV);
   rt.argmax_pi = (int *)(base + SS_ARGMAX_PI);
   rt.attn_part = (float *)(base + SS_ATTN_PART);
+  rt.attn_part_cap = (int)MK_STATIC_ATTN_HEADS;
   rt.splitk_part = base + SS_SPLITK_PART;
   rt.stage_prof = nullptr;  // per-stage timing is library-allocated scratch too: not recorded by this entry point
   rt.timing = nullptr;

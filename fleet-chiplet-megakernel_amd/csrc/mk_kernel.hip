@@ -198,6 +198,9 @@ __device__ __forceinline__ u32x4 ldc_16B(const u32x4 *p) {
 __device__ __forceinline__ void stc_u16(uint16_t *p, uint16_t v) {
   __hip_atomic_store((__attribute__((address_space(1))) uint16_t *)(unsigned long long)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void stc_f32(float *p, float v) {
+  __hip_atomic_store((__attribute__((address_space(1))) unsigned *)(unsigned long long)p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ void stc_16B(u32x4 *p, u32x4 v) {
   __attribute__((address_space(1))) unsigned long long *q = (__attribute__((address_space(1))) unsigned long long *)(unsigned long long)p;
   __hip_atomic_store(q, (unsigned long long)v.x | ((unsigned long long)v.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -3039,6 +3042,9 @@ __device__ __forceinline__ void head_row_finish(float x0, float x1, uint16_t *ds
   dst[lane + 64] = (uint16_t)f2bf(x1);
 }
 
+#ifndef MK_TUNE_ATTN_TILES
+#define MK_TUNE_ATTN_TILES 2
+#endif
 #ifndef MK_TUNE_NPRE
 #define MK_TUNE_NPRE 4
 #endif
@@ -3062,7 +3068,7 @@ struct AttnUnit {
 // Reference tasks: kv_cache_update_impl (tasks/mi300/kv_cache_update_mi300.cuh:41-327),
 // paged_attention_minimal_decode (tasks/mi300/paged_attention_decode_minimal_mi300.cuh:100-371),
 // gang_attention_split_kv_kernel (tasks/mi300/gang_attention_mi300.cuh:49-153).
-template <int QPK>
+template <int QPK, bool MF>
 __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &rt, int M, char *smem) {
   constexpr int D = 128;
   constexpr int NPRE = MK_TUNE_NPRE;          // positions per lane group requested ahead
@@ -3077,8 +3083,18 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   int *sflag = (int *)(smem + 2048);
   uint16_t *knew = (uint16_t *)(smem + 4096);                             // [MK_MAX_NEW_PER_REQ][128]
   uint16_t *vnew = knew + MK_MAX_NEW_PER_REQ * D;                         // [MK_MAX_NEW_PER_REQ][128]
-  float *part = (float *)(smem + 4096 + 2 * MK_MAX_NEW_PER_REQ * D * 2);  // [16][QPK][132]
-  static_assert(4096 + 2 * MK_MAX_NEW_PER_REQ * 128 * 2 + 16 * QPK * 132 * 4 <= MK_LDS_BYTES, "attention scratch exceeds the LDS window");
+  // MF (iterations of many tokens): the cached positions go through the matrix cores, one wavefront per 16-position
+  // tile, and leave four more partial results (one per wavefront) next to the sixteen lane groups'; each wavefront has
+  // two private 4 KB buffers for the V tiles it transposes through LDS.  The page list of the running unit aliases the
+  // partial-result area (used before the partials are written).
+  constexpr int NG = MF ? 20 : 16;
+  constexpr int VS = 1056;  // bytes between the four 1 KB request blocks of a V tile in LDS (+32: neighbouring blocks start in other banks)
+  constexpr int PART_OFF = 4096 + 2 * MK_MAX_NEW_PER_REQ * D * 2, VBUF_OFF = PART_OFF + NG * QPK * 132 * 4;
+  float *part = (float *)(smem + PART_OFF);  // [NG][QPK][132]
+  int *spg = (int *)(smem + PART_OFF);
+  constexpr int RB = QPK == 4 ? MK_TUNE_ATTN_TILES : 2;  // (MF) tiles a wavefront keeps in flight, as LDS allows
+  static_assert(VBUF_OFF + (MF ? MK_WAVES * RB * 4 * VS : 0) <= MK_LDS_BYTES, "attention scratch exceeds the LDS window");
+  static_assert(MK_ATTN_MAX_REQ_PAGES * 4 <= NG * QPK * 132 * 4, "page list exceeds the area it aliases");
   const int n_items = M * nkv;
   int cmax = c.G / n_items;
   cmax = cmax < 1 ? 1 : (cmax > MK_ATTN_MAX_CHUNKS ? MK_ATTN_MAX_CHUNKS : cmax);
@@ -3130,9 +3146,9 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   };
   // the polling wavefront keeps its memory queue empty until the barrier is through (its loads would delay the poll
   // results behind them); its rows are requested right after and land while the q rows are being fetched
-  if (have0 && wave != 0) prefetch0();
+  if (!MF && have0 && wave != 0) prefetch0();
   barrier_wait(c);
-  if (have0 && wave == 0) prefetch0();
+  if (!MF && have0 && wave == 0) prefetch0();
   // the q/k/v rows: stored by the producing linear, or -- when it left its K-slice partials to this stage -- summed here
   const int dS = c.defer_S;
   c.defer_S = 0;
@@ -3160,6 +3176,11 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     }
     const int t = a.t, h = a.h, p = a.p, C = a.C;
     __syncthreads();  // LDS reuse across units
+    // (MF) this unit's page-table entries: requested here, stored to LDS after the row requests below are out -- an LDS
+    // store waits for its load, and loads return in order
+    const int pg_lo = a.start / ps;
+    const int npg = (MF && a.cend > a.start) ? (a.cend - 1) / ps - pg_lo + 1 : 0;
+    const int pg_first = tid < npg ? a.pages[pg_lo + tid] : 0;
     // ---- phase A: prepare q heads and the new K/V rows of this chunk, two rows per wavefront in flight
     const int n_rows = QPK + a.n_new;
     for (int row0 = wave; row0 < n_rows; row0 += 2 * MK_WAVES) {
@@ -3175,6 +3196,10 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
           fetch(tok[r], off[r], x0[r], x1[r]);
           if (!isq) fetch(tok[r], off[r] + D, v0[r], v1[r]);  // (a V row is copied as it is)
         }
+      }
+      if (MF && row0 == wave) {
+        if (tid < npg) spg[tid] = pg_first;
+        for (int i = tid + MK_THREADS; i < npg; i += MK_THREADS) spg[i] = a.pages[pg_lo + i];
       }
 #pragma unroll
       for (int r = 0; r < 2; r++) {
@@ -3204,8 +3229,10 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       }
     }
     __syncthreads();
-    // the chunk that owns the newest position appends this token's K/V and publishes q
-    if (a.cidx == C - 1) {
+    // the chunk that owns the newest position appends this token's K/V and publishes q (MF: after the tile loop, whose
+    // request counting must not see other vector-memory traffic)
+    auto append = [&]() {
+      if (a.cidx != C - 1) return;
       const int j = p - a.new_lo;
       const size_t rowi = (size_t)a.pages[p / ps] * ps + (p % ps);
       uint32_t *kd = (uint32_t *)st.k_cache + (rowi * nkv + h) * (D / 2);
@@ -3216,7 +3243,9 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         uint32_t *qd = (uint32_t *)st.q_ws + ((size_t)t * st.ld_qws + (size_t)h * QPK * D) / 2;
         for (int i = tid; i < QPK * D / 2; i += MK_THREADS) qd[i] = ((const uint32_t *)qs)[i];
       }
-    }
+    };
+    if (!MF) append();
+    MK_MARK(c, first ? 0 : 2);
     // ---- phase B: online softmax over the chunk
     u32x4 qv[QPK];
 #pragma unroll
@@ -3287,6 +3316,130 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         }
       }
     };
+    if constexpr (MF) {
+      // ---- cached positions on the matrix cores.  Tile = 16 positions, one wavefront per tile.  Scores: A = the K tile
+      // (lane (i, g): row of position i; request s of a tile reads bytes 64 s + 16 g of the rows -- 64 contiguous bytes
+      // per row and request -- so step s contracts dims 32 s + 8 g ..), B = q (lane (j, g): head j, same dims; heads
+      // past QPK are zero) -> lane (j, g) holds the scores of head j at
+      // positions 4 g .. 4 g + 3.  Those four weights, as bf16 (value and rounding remainder: two operands), are already
+      // the A operand of a 16x16x16 step over positions; its B operand -- four consecutive positions of one dim --
+      // is read out of the V tile that direct-to-LDS loads put into this wavefront's buffer.  The running maximum is
+      // kept per head for the whole wavefront (the products of a step are summed across its lanes, so they must share
+      // their reference), the running sum per lane.
+      typedef short s16x4 __attribute__((ext_vector_type(4)));
+      const int lr = lane & 15, lg = lane >> 4;
+      char *vb0 = smem + VBUF_OFF + wave * (RB * 4 * VS);
+      bf16x8 qb[4];
+#pragma unroll
+      for (int s_ = 0; s_ < 4; s_++) {
+        const u32x4 z = {0u, 0u, 0u, 0u};
+        qb[s_] = __builtin_bit_cast(bf16x8, lr < QPK ? *(const u32x4 *)(qs + lr * D + s_ * 32 + lg * 8) : z);
+      }
+      f32x4 o[8];
+#pragma unroll
+      for (int dt = 0; dt < 8; dt++) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
+      float mrun = -INFINITY, lsum = 0.f;
+      const int nt = a.cend > a.start ? (a.cend - a.start + 15) >> 4 : 0;
+      auto load_tile = [&](int tt, bf16x8 (&kk)[4], char *vbuf) {
+        const int pos = min(a.start + min(tt, nt - 1) * 16 + lr, a.cend - 1), pg = pos / ps;
+        const size_t base = (((size_t)spg[pg - pg_lo] * ps + (pos - pg * ps)) * nkv + h) * (D / 8) + lg;
+#pragma unroll
+        for (int s_ = 0; s_ < 4; s_++) kk[s_] = __builtin_nontemporal_load((const bf16x8 *)(kc + base + s_ * 4));
+#pragma unroll
+        for (int s_ = 0; s_ < 4; s_++)
+          __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(vc + base + s_ * 4),
+                                           (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + s_ * VS), 16, 0, 0);
+      };
+      const int vlane = (lr >> 3) * 256 + lg * 64 + (lr & 7) * 2;
+      auto compute_tile = [&](int t_, const bf16x8 (&kk)[4], const char *vbuf) {
+        f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+        for (int s_ = 0; s_ < 4; s_++) s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[s_], qb[s_], s4, 0, 0, 0);
+        const int pbase = a.start + t_ * 16 + lg * 4;
+        float sc[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) sc[r] = pbase + r < a.cend ? s4[r] * st.sm_scale_log2 : -INFINITY;
+        float mx = fmaxf(fmaxf(sc[0], sc[1]), fmaxf(sc[2], sc[3]));
+        mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, mx))));
+        mx = fmaxf(mx, __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, mx))));
+        const float mn = fmaxf(mrun, mx);
+        const float alpha = __builtin_amdgcn_exp2f(mrun - mn);
+        float pw[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) pw[r] = __builtin_amdgcn_exp2f(sc[r] - mn);
+        lsum = lsum * alpha + ((pw[0] + pw[1]) + (pw[2] + pw[3]));
+        mrun = mn;
+        if (__ballot(lr < QPK && alpha != 1.f)) {  // (uniform) some head's maximum moved: rescale what has been summed
+          float ar[4];
+#pragma unroll
+          for (int r = 0; r < 4; r++) ar[r] = __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lg * 4 + r) << 2, __builtin_bit_cast(int, alpha)));
+#pragma unroll
+          for (int dt = 0; dt < 8; dt++)
+#pragma unroll
+            for (int r = 0; r < 4; r++) o[dt][r] *= ar[r];
+        }
+        float ph[4];
+#pragma unroll
+        for (int r = 0; r < 4; r++) ph[r] = bfround(pw[r]);
+        const unsigned h01 = pack2(ph[0], ph[1]), h23 = pack2(ph[2], ph[3]);
+        const unsigned l01 = pack2(pw[0] - ph[0], pw[1] - ph[1]), l23 = pack2(pw[2] - ph[2], pw[3] - ph[3]);
+        const s16x4 a_hi = __builtin_bit_cast(s16x4, (unsigned long long)h01 | ((unsigned long long)h23 << 32));
+        const s16x4 a_lo = __builtin_bit_cast(s16x4, (unsigned long long)l01 | ((unsigned long long)l23 << 32));
+        const char *vb = vbuf + vlane;
+#pragma unroll
+        for (int dt = 0; dt < 8; dt++) {
+          const char *q_ = vb + (dt >> 1) * VS + (dt & 1) * 512;
+          const unsigned v0 = *(const uint16_t *)(q_), v1 = *(const uint16_t *)(q_ + 16), v2 = *(const uint16_t *)(q_ + 32), v3 = *(const uint16_t *)(q_ + 48);
+          const s16x4 bv = __builtin_bit_cast(s16x4, (unsigned long long)(v0 | (v1 << 16)) | ((unsigned long long)(v2 | (v3 << 16)) << 32));
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_hi, bv, o[dt], 0, 0, 0);
+          o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_lo, bv, o[dt], 0, 0, 0);
+        }
+      };
+      // RB tiles in flight per wavefront: every request is issued unconditionally (a tile index past the end re-reads the
+      // last tile; it is never computed), and the wait before a tile counts the 8 (RB - 1) requests of the tiles after it
+      int t_ = wave;
+      if (t_ < nt) {
+        bf16x8 kr[RB][4];
+#pragma unroll
+        for (int b_ = 0; b_ < RB - 1; b_++) load_tile(t_ + b_ * MK_WAVES, kr[b_], vb0 + b_ * 4 * VS);
+        bool more = true;
+        while (more) {
+#pragma unroll
+          for (int b_ = 0; b_ < RB; b_++) {
+            // slot (b_ + RB - 1) % RB was computed in the previous round: refill it with the tile RB - 1 ahead
+            load_tile(t_ + (RB - 1) * MK_WAVES, kr[(b_ + RB - 1) % RB], vb0 + ((b_ + RB - 1) % RB) * 4 * VS);
+            if (RB == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
+            else if (RB == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
+            else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
+            if (more) {
+              compute_tile(t_, kr[b_], vb0 + b_ * 4 * VS);
+              t_ += MK_WAVES;
+              more = t_ < nt;
+            }
+          }
+        }
+      }
+      MK_MARK(c, first ? 1 : 3);
+      asm volatile("s_waitcnt vmcnt(0)" ::: "memory");  // (the direct-to-LDS requests of the tile that was not computed)
+      append();
+      __syncthreads();  // every wavefront is done with the page list: the partial results may overwrite it
+      float lt = lsum;
+      lt += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 16) << 2, __builtin_bit_cast(int, lt)));
+      lt += __builtin_bit_cast(float, __builtin_amdgcn_ds_bpermute((lane ^ 32) << 2, __builtin_bit_cast(int, lt)));
+      const int gm = 16 + wave;
+      if (lg == 0 && lr < QPK) {
+        part[(gm * QPK + lr) * 132 + 128] = mrun;
+        part[(gm * QPK + lr) * 132 + 129] = lt;
+      }
+#pragma unroll
+      for (int r = 0; r < 4; r++) {
+        const int head = lg * 4 + r;
+        if (head < QPK) {
+#pragma unroll
+          for (int dt = 0; dt < 8; dt++) part[(gm * QPK + head) * 132 + dt * 16 + lr] = o[dt][r];
+        }
+      }
+    } else {
     int pos = a.start + gg;
     if (first) {
       if (pos < a.cend) process_block(pk, pv, pos);
@@ -3317,6 +3470,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         if (pos >= a.cend) break;
       }
     }
+    }
     for (int j = gg; j < a.n_new; j += 16) process(((const u32x4 *)(knew + j * D))[j16], ((const u32x4 *)(vnew + j * D))[j16]);
     // ---- phase C: merge the 16 groups through LDS
 #pragma unroll
@@ -3345,12 +3499,12 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     {
       float mx = -INFINITY;
 #pragma unroll
-      for (int g = 0; g < 16; g++) mx = fmaxf(mx, part[(g * QPK + mh) * 132 + 128]);
+      for (int g = 0; g < NG; g++) mx = fmaxf(mx, part[(g * QPK + mh) * 132 + 128]);
       float ls = 0.f, os[DPT];
 #pragma unroll
       for (int d = 0; d < DPT; d++) os[d] = 0.f;
 #pragma unroll
-      for (int g = 0; g < 16; g++) {
+      for (int g = 0; g < NG; g++) {
         const float *pp = part + (g * QPK + mh) * 132;
         const float wgt = __builtin_amdgcn_exp2f(pp[128] - mx);
         ls += pp[129] * wgt;
@@ -3579,9 +3733,23 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
           break;
         case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
         case MK_OP_ATTN:
-          if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4>(st, c, rt, M, smem);
-          else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8>(st, c, rt, M, smem);
-          else barrier_wait(c);
+          if constexpr (MAXM == 1) {
+            if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4, false>(st, c, rt, M, smem);
+            else if (st.num_q_heads == 8 * st.num_kv_heads) stage_attn<8, false>(st, c, rt, M, smem);
+            else barrier_wait(c);
+          } else {
+            // many (token, kv head) pairs per workgroup-chunk: cached positions on the matrix cores
+            const bool mf = 2 * M * st.num_kv_heads >= c.G;
+            if (st.num_q_heads == 4 * st.num_kv_heads) {
+              if (mf) stage_attn<4, true>(st, c, rt, M, smem);
+              else stage_attn<4, false>(st, c, rt, M, smem);
+            } else if (st.num_q_heads == 8 * st.num_kv_heads) {
+              if (mf) stage_attn<8, true>(st, c, rt, M, smem);
+              else stage_attn<8, false>(st, c, rt, M, smem);
+            } else {
+              barrier_wait(c);
+            }
+          }
           break;
         case MK_OP_MOE_TOPK: stage_moe_topk(st, c, M); break;
         case MK_OP_MOE_LINEAR: stage_moe_linear(st, c, M, smem); break;

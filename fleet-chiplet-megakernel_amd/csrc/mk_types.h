@@ -18,6 +18,7 @@
 #define MK_ATTN_MAX_CHUNKS 32 // split-KV fan-out limit per (token, kv head)
 #define MK_ATTN_PSTRIDE 160   // floats per (work unit, q head) split-KV partial: 128 values + one 128-byte line of (max, sum)
 #define MK_MAX_NEW_PER_REQ 64 // most prompt tokens one request may ingest per iteration (the attention stage keeps their K/V rows in LDS); the
+#define MK_ATTN_MAX_REQ_PAGES 8192  // page-table entries of one request the attention stage keeps in LDS: max_seq_length / page_size may not exceed it
                               // configured value defaults to the reference's 8 (MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124)
 // LDS map of one workgroup (dynamic, > 80 KB pins one workgroup per CU):
 //   [0, 24 KB)      input row(s) of the running stage / attention scratch (attention may run on beyond 32 KB)
@@ -190,6 +191,8 @@ struct MkRuntime {
   float *argmax_pv;     // non-null: the sampling stages' per-workgroup partials live here ([tokens][workgroups] values / indices)
   int *argmax_pi;       // instead of in the buffers their descriptors name
   unsigned *attn_cnt;   // [max_tokens * num_kv_heads][32]: one 128-byte line per counter
+  int attn_part_cap;    // q-head partials each attention stage's split-KV workspace (or the shared one) holds
+  int pad_apc;
   void *splitk_part;    // [workgroups][4 wavefronts][4 weight tiles][4 token tiles][64 lanes] f32x4: K-slice partials of the split-K linear
   unsigned *splitk_cnt; // [workgroups][32]: arrival counter per split-K group (one 128-byte line each)
   long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end

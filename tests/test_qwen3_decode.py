@@ -264,3 +264,22 @@ def test_prefill_chunk_size_follows_max_tokens_per_request(per_req, expect_prefi
     assert int(steps[0]) == max_seq - 1
     _teacher_check(cfg, w, [prompt], toks, max_seq, min_margin_hits=3)
     dec.mpk.finalize()
+
+
+@pytest.mark.parametrize("B", [32, 64])
+def test_batched_decode_matrix_core_attention_full_head_layout(B):
+    """32 q / 8 kv heads (the full-size head layout) and at least 16 tokens per iteration: the attention stage works the
+    cached positions off on the matrix cores, 16-position tiles per wavefront.  Prompts of 130..250 tokens, prompt
+    ingestion running next to decoding requests; the generated tokens must pass the oracle check."""
+    from oracle.qwen3_ref import Qwen3Config, make_model_weights, make_prompt
+    cfg = Qwen3Config(hidden_size=1024, num_q_heads=32, num_kv_heads=8, head_dim=128, intermediate_size=1536, num_layers=2, vocab_size=2048)
+    w = make_model_weights(cfg, seed=27)
+    max_seq = 272
+    prompts = [make_prompt(cfg, 130 + (17 * i) % 120, 900 + i) for i in range(B)]
+    dec = _decoder(cfg, w, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=64, total_requests=B)
+    toks, steps = dec.generate(prompts)
+    assert dec.mpk.stats()["aborted"] == 0
+    assert all(int(s) == max_seq - 1 for s in steps)
+    pick = [0, 1, B // 2, B - 1]
+    _teacher_check(cfg, w, [prompts[i] for i in pick], toks[pick], max_seq, min_margin_hits=20)
+    dec.mpk.finalize()
