@@ -688,6 +688,21 @@ class PersistentKernel:
         assert self._is_compiled, "call compile() first"
         sp = self._stream_ptr(kwargs.get("default_stream", None))
         _capi.check(self._lib.mk_launch(self._handle, ctypes.c_void_p(sp)))
+        if self.profiler_tensor is not None:
+            self.export_profile()
+
+    def export_profile(self, trace_name: str = None):
+        """With a profiler tensor (reference: persistent_kernel.py:2644-2658): the per-stage device timeline of the last
+        iteration goes into the tensor in the reference's (tag, timestamp) format and out as `<trace_name>.perfetto-trace`
+        (default mirage_<rank>), the raw tensor beside it as `.pt`.  Returns the trace's path."""
+        from .profiler_persistent import export_to_perfetto_trace, fill_profiler_tensor
+        assert self.profiler_tensor is not None, "no profiler tensor was passed to the constructor"
+        n_wg = self.stats()["num_workgroups"]
+        fill_profiler_tensor(self.profiler_tensor, [self.stage_profile(w, raw=True) for w in range(n_wg)])
+        name = (trace_name or self.trace_name or f"mirage_{self.mpi_rank}") + ".perfetto-trace"
+        export_to_perfetto_trace(self.profiler_tensor, name)
+        torch.save(self.profiler_tensor.cpu(), name.replace(".perfetto-trace", ".pt"))
+        return name
 
     def init_request_resources(self):
         """Reset step[], batch slots and the page ring (reference: init_request_func, persistent_kernel.py:63-68)."""
