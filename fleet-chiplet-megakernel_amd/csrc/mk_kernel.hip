@@ -1781,8 +1781,12 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
 #pragma unroll
       for (int j = 0; j < NB; j++) w_load(j, a[j]);
     }
+    // Token rows come from other workgroups and are read with cached loads, so what this die's caches hold of them must
+    // go first.  The invalidate is issued BEFORE the barrier is awaited: nothing on this die reads the stage's input
+    // buffers between the stage that last consumed them (barriers ago) and this barrier, so no stale line can come
+    // back in between, and the invalidate's latency is off the path from the last arrival to the first row request.
+    if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
     if (c.pending && tid == 0) barrier_poll(c);
-    if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");  // token rows come from other workgroups: one acquire, then cached loads
     __syncthreads();
     barrier_done(c);
     MK_MARK(c, 0);
@@ -1969,12 +1973,12 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
 // on 256 workgroups) spend the registers on depth instead: <2, MK_TUNE_NBN>.
 template <int MT, int TG, int NB>
 __device__ __forceinline__ void stage_linear_mfma(CStage &st, Ctx &c, int M, char *smem) {
+  // activations were produced by other workgroups: drop what this die's caches hold of them once, then use cached loads
+  // so the rows are shared through the die's L2.  (Issued before the barrier is awaited: nothing on this die reads
+  // the stage's input buffers between their previous consumer and this barrier.)
+  if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
   barrier_wait(c);
   c.wrote_through = true;  // outputs are written through: no L2 write-back at this stage's arrival
-  // activations were produced by other workgroups: invalidate this CU's L1 once, then use cached loads so the rows
-  // are shared through the XCD's L2
-  if (threadIdx.x == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-  __syncthreads();
   MK_MARK(c, 0);
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   const int lr = lane & 15, lg = lane >> 4;
