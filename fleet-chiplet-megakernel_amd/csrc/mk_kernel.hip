@@ -3092,12 +3092,18 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
   // two private 4 KB buffers for the V tiles it transposes through LDS.  The page list of the running unit aliases the
   // partial-result area (used before the partials are written).
   constexpr int NG = MF ? 20 : 16;
-  constexpr int VS = 1056;  // bytes between the four 1 KB request blocks of a V tile in LDS (+32: neighbouring blocks start in other banks)
+  // A K or V tile in LDS: 16 rows of 256 bytes as four groups of four rows, one direct-to-LDS request per group (each
+  // lane 16 bytes: four whole rows, 1 KB contiguous in LDS), the groups GS bytes apart (+64: the transposed V reads of
+  // the four groups then fall into different banks).  With four q heads per kv head there is room to stage K this way
+  // as well (whole rows per request instead of 64 bytes of each of 16 rows); otherwise K goes to registers.
+  constexpr int GS = 1088, TS = 4 * GS;
+  constexpr bool KLDS = QPK == 4;
+  constexpr int SLOT = KLDS ? 2 * TS : TS;  // bytes per tile in flight
   constexpr int PART_OFF = 4096 + 2 * MK_MAX_NEW_PER_REQ * D * 2, VBUF_OFF = PART_OFF + NG * QPK * 132 * 4;
   float *part = (float *)(smem + PART_OFF);  // [NG][QPK][132]
   int *spg = (int *)(smem + PART_OFF);
   constexpr int RB = QPK == 4 ? MK_TUNE_ATTN_TILES : 2;  // (MF) tiles a wavefront keeps in flight, as LDS allows
-  static_assert(VBUF_OFF + (MF ? MK_WAVES * RB * 4 * VS : 0) <= MK_LDS_BYTES, "attention scratch exceeds the LDS window");
+  static_assert(VBUF_OFF + (MF ? MK_WAVES * RB * SLOT : 0) <= MK_LDS_BYTES, "attention scratch exceeds the LDS window");
   static_assert(MK_ATTN_MAX_REQ_PAGES * 4 <= NG * QPK * 132 * 4, "page list exceeds the area it aliases");
   const int n_items = M * nkv;
   int cmax = c.G / n_items;
@@ -3322,9 +3328,9 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     };
     if constexpr (MF) {
       // ---- cached positions on the matrix cores.  Tile = 16 positions, one wavefront per tile.  Scores: A = the K tile
-      // (lane (i, g): row of position i; request s of a tile reads bytes 64 s + 16 g of the rows -- 64 contiguous bytes
-      // per row and request -- so step s contracts dims 32 s + 8 g ..), B = q (lane (j, g): head j, same dims; heads
-      // past QPK are zero) -> lane (j, g) holds the scores of head j at
+      // (lane (i, g): row of position i; step s contracts dims 32 s + 8 g ..; read from the K tile in LDS, or -- eight q
+      // heads per kv head -- requested straight into registers, 64 bytes of each of 16 rows per request), B = q (lane
+      // (j, g): head j, same dims; heads past QPK are zero) -> lane (j, g) holds the scores of head j at
       // positions 4 g .. 4 g + 3.  Those four weights, as bf16 (value and rounding remainder: two operands), are already
       // the A operand of a 16x16x16 step over positions; its B operand -- four consecutive positions of one dim --
       // is read out of the V tile that direct-to-LDS loads put into this wavefront's buffer.  The running maximum is
@@ -3332,7 +3338,7 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       // their reference), the running sum per lane.
       typedef short s16x4 __attribute__((ext_vector_type(4)));
       const int lr = lane & 15, lg = lane >> 4;
-      char *vb0 = smem + VBUF_OFF + wave * (RB * 4 * VS);
+      char *vb0 = smem + VBUF_OFF + wave * (RB * SLOT);
       bf16x8 qb[4];
 #pragma unroll
       for (int s_ = 0; s_ < 4; s_++) {
@@ -3344,21 +3350,41 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       for (int dt = 0; dt < 8; dt++) o[dt] = (f32x4){0.f, 0.f, 0.f, 0.f};
       float mrun = -INFINITY, lsum = 0.f;
       const int nt = a.cend > a.start ? (a.cend - a.start + 15) >> 4 : 0;
+      auto row_base = [&](int pos) -> size_t {  // first 16-byte operand of the (position, head) row
+        const int pc = min(pos, a.cend - 1), pg = pc / ps;
+        return (((size_t)spg[pg - pg_lo] * ps + (pc - pg * ps)) * nkv + h) * (D / 8);
+      };
       auto load_tile = [&](int tt, bf16x8 (&kk)[4], char *vbuf) {
-        const int pos = min(a.start + min(tt, nt - 1) * 16 + lr, a.cend - 1), pg = pos / ps;
-        const size_t base = (((size_t)spg[pg - pg_lo] * ps + (pos - pg * ps)) * nkv + h) * (D / 8) + lg;
+        const int p0 = a.start + min(tt, nt - 1) * 16;
+        if (!KLDS) {  // K to registers: lane (row, g), request s reads bytes 64 s + 16 g of its row
+          const size_t base = row_base(p0 + lr) + lg;
 #pragma unroll
-        for (int s_ = 0; s_ < 4; s_++) kk[s_] = __builtin_nontemporal_load((const bf16x8 *)(kc + base + s_ * 4));
+          for (int s_ = 0; s_ < 4; s_++) kk[s_] = __builtin_nontemporal_load((const bf16x8 *)(kc + base + s_ * 4));
+        }
+        // to LDS: request s brings rows 4 s .. 4 s + 3 whole (lane (row in group, 16-byte piece))
+        size_t gb[4];
+#pragma unroll
+        for (int s_ = 0; s_ < 4; s_++) gb[s_] = row_base(p0 + 4 * s_ + lg) + lr;
+        if (KLDS) {
+#pragma unroll
+          for (int s_ = 0; s_ < 4; s_++)
+            __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(kc + gb[s_]),
+                                             (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + TS + s_ * GS), 16, 0, 0);
+        }
 #pragma unroll
         for (int s_ = 0; s_ < 4; s_++)
-          __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(vc + base + s_ * 4),
-                                           (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + s_ * VS), 16, 0, 0);
+          __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(vc + gb[s_]),
+                                           (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + s_ * GS), 16, 0, 0);
       };
-      const int vlane = (lr >> 3) * 256 + lg * 64 + (lr & 7) * 2;
+      const int vlane = lg * GS + lr * 2;
+      const int klane = (lr >> 2) * GS + (lr & 3) * 256 + lg * 16;
       auto compute_tile = [&](int t_, const bf16x8 (&kk)[4], const char *vbuf) {
         f32x4 s4 = {0.f, 0.f, 0.f, 0.f};
 #pragma unroll
-        for (int s_ = 0; s_ < 4; s_++) s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kk[s_], qb[s_], s4, 0, 0, 0);
+        for (int s_ = 0; s_ < 4; s_++) {
+          const bf16x8 ko = KLDS ? __builtin_bit_cast(bf16x8, *(const u32x4 *)(vbuf + TS + klane + s_ * 64)) : kk[s_];
+          s4 = __builtin_amdgcn_mfma_f32_16x16x32_bf16(ko, qb[s_], s4, 0, 0, 0);
+        }
         const int pbase = a.start + t_ * 16 + lg * 4;
         float sc[4];
 #pragma unroll
@@ -3392,8 +3418,8 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
         const char *vb = vbuf + vlane;
 #pragma unroll
         for (int dt = 0; dt < 8; dt++) {
-          const char *q_ = vb + (dt >> 1) * VS + (dt & 1) * 512;
-          const unsigned v0 = *(const uint16_t *)(q_), v1 = *(const uint16_t *)(q_ + 16), v2 = *(const uint16_t *)(q_ + 32), v3 = *(const uint16_t *)(q_ + 48);
+          const char *q_ = vb + dt * 32;
+          const unsigned v0 = *(const uint16_t *)(q_), v1 = *(const uint16_t *)(q_ + 256), v2 = *(const uint16_t *)(q_ + 512), v3 = *(const uint16_t *)(q_ + 768);
           const s16x4 bv = __builtin_bit_cast(s16x4, (unsigned long long)(v0 | (v1 << 16)) | ((unsigned long long)(v2 | (v3 << 16)) << 32));
           o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_hi, bv, o[dt], 0, 0, 0);
           o[dt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(a_lo, bv, o[dt], 0, 0, 0);
@@ -3405,18 +3431,18 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
       if (t_ < nt) {
         bf16x8 kr[RB][4];
 #pragma unroll
-        for (int b_ = 0; b_ < RB - 1; b_++) load_tile(t_ + b_ * MK_WAVES, kr[b_], vb0 + b_ * 4 * VS);
+        for (int b_ = 0; b_ < RB - 1; b_++) load_tile(t_ + b_ * MK_WAVES, kr[b_], vb0 + b_ * SLOT);
         bool more = true;
         while (more) {
 #pragma unroll
           for (int b_ = 0; b_ < RB; b_++) {
             // slot (b_ + RB - 1) % RB was computed in the previous round: refill it with the tile RB - 1 ahead
-            load_tile(t_ + (RB - 1) * MK_WAVES, kr[(b_ + RB - 1) % RB], vb0 + ((b_ + RB - 1) % RB) * 4 * VS);
+            load_tile(t_ + (RB - 1) * MK_WAVES, kr[(b_ + RB - 1) % RB], vb0 + ((b_ + RB - 1) % RB) * SLOT);
             if (RB == 2) asm volatile("s_waitcnt vmcnt(8)" ::: "memory");
             else if (RB == 3) asm volatile("s_waitcnt vmcnt(16)" ::: "memory");
             else asm volatile("s_waitcnt vmcnt(24)" ::: "memory");
             if (more) {
-              compute_tile(t_, kr[b_], vb0 + b_ * 4 * VS);
+              compute_tile(t_, kr[b_], vb0 + b_ * SLOT);
               t_ += MK_WAVES;
               more = t_ < nt;
             }
