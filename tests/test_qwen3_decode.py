@@ -266,13 +266,15 @@ def test_prefill_chunk_size_follows_max_tokens_per_request(per_req, expect_prefi
     dec.mpk.finalize()
 
 
-@pytest.mark.parametrize("B", [32, 64])
-def test_batched_decode_matrix_core_attention_full_head_layout(B):
+@pytest.mark.parametrize("B,nkv", [(32, 8), (64, 8), (64, 4)])
+def test_batched_decode_matrix_core_attention_full_head_layout(B, nkv):
     """32 q / 8 kv heads (the full-size head layout) and at least 16 tokens per iteration: the attention stage works the
     cached positions off on the matrix cores, 16-position tiles per wavefront.  Prompts of 130..250 tokens, prompt
     ingestion running next to decoding requests; the generated tokens must pass the oracle check."""
     from oracle.qwen3_ref import Qwen3Config, make_model_weights, make_prompt
-    cfg = Qwen3Config(hidden_size=1024, num_q_heads=32, num_kv_heads=8, head_dim=128, intermediate_size=1536, num_layers=2, vocab_size=2048)
+    # 8 kv heads: four q heads each, K and V tiles both staged through LDS; 4 kv heads: eight q heads each (the
+    # Qwen3-30B-A3B head layout), K tiles in registers
+    cfg = Qwen3Config(hidden_size=1024, num_q_heads=32, num_kv_heads=nkv, head_dim=128, intermediate_size=1536, num_layers=2, vocab_size=2048)
     w = make_model_weights(cfg, seed=27)
     max_seq = 272
     prompts = [make_prompt(cfg, 130 + (17 * i) % 120, 900 + i) for i in range(B)]
