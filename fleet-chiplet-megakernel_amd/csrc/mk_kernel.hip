@@ -1774,9 +1774,7 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
         aa[t][1] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + step * step_stride + half_stride));
       }
     };
-    // weights do not depend on the previous stage: the first NB steps are requested before its barrier is awaited, by the
-    // polling wavefront as well (its first poll result then arrives behind them -- loads return in order -- which costs
-    // nothing unless this workgroup is the barrier's last arriver, and spares it a trip to memory after the barrier)
+    // weights do not depend on the previous stage: the first NB steps are requested before its barrier is awaited
     if (has_tile) {
 #pragma unroll
       for (int j = 0; j < NB; j++) w_load(j, a[j]);
@@ -1785,8 +1783,13 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
     // go first.  The invalidate is issued BEFORE the barrier is awaited: nothing on this die reads the stage's input
     // buffers between the stage that last consumed them (barriers ago) and this barrier, so no stale line can come
     // back in between, and the invalidate's latency is off the path from the last arrival to the first row request.
-    if (tid == 0) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
-    if (c.pending && tid == 0) barrier_poll(c);
+    // The poll runs on the first row-staging wavefront, which has no weight loads in flight: loads return in order, so
+    // on a streaming wavefront the poll's answer would wait behind the NB steps just requested -- two to four
+    // microseconds for exactly the workgroups that enter last (those that did the norm stage's rows, or everybody after
+    // an attention stage), which are the ones the stage then waits for.
+    constexpr int POLL_TID = NSW * 64;
+    if (tid == POLL_TID) __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "agent");
+    if (c.pending && tid == POLL_TID) barrier_poll(c);
     __syncthreads();
     barrier_done(c);
     MK_MARK(c, 0);
