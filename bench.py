@@ -88,10 +88,27 @@ def cpu_baseline(shape, n_layers_sample=2, steps=3, context=80):
 # times the steps of its launch (measured on the default 1024-step launches, whose contexts they average over; a launch of
 # another length holds different KV rows and the figure is then approximate); a batch size without a committed counter
 # pass reports null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): (15.6973e12 + 14.99e9) / 1024, ("qwen3-8b", 64): (25.9588e12 + 1.4023e12) / 1024}
+MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): (15.6965e12 + 14.99e9) / 1024, ("qwen3-8b", 64): (25.8980e12 + 1.4039e12) / 1024}
 
 
-def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
+def print_stage_profile(dec, B, out=sys.stderr):
+    """Where the last iteration of the last launch went: per stage, over all workgroups, when they entered the stage, when
+    they saw the previous stage's barrier complete and when they arrived at the stage's own barrier (microseconds after
+    the first workgroup entered the first stage; device timestamps, 100 MHz)."""
+    import numpy as np
+    G = dec.mpk.stats()["num_workgroups"]
+    prof = [dec.mpk.stage_profile(w, raw=True) for w in range(G)]
+    rows = [i for i in range(len(prof[0]) - 1) if prof[0][i][1] > 0]  # (the last record times the scheduler step)
+    t0 = min(prof[w][rows[0]][1] for w in range(G))
+    print(f"stage profile, BS={B}, last iteration ({G} workgroups; us): entered min..max | barrier seen min..max | arrived min / median / max", file=out)
+    for i in rows:
+        ent, seen, arr = (np.array([prof[w][i][k] for w in range(G)], dtype=np.float64) * 0.01 - t0 * 0.01 for k in (1, 2, 4))
+        print(f"  {prof[0][i][0][:56]:56s} {ent.min():8.1f}..{ent.max():8.1f} | {seen.min():8.1f}..{seen.max():8.1f} | "
+              f"{arr.min():8.1f} / {np.median(arr):8.1f} / {arr.max():8.1f}", file=out)
+    out.flush()
+
+
+def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode, stage_profile=False):
     """Ingest B prompts of P tokens, run W untimed decode steps, then time exactly K decode steps in ONE persistent launch."""
     prompts = [torch.randint(0, shape.vocab_size, (P,), generator=torch.Generator().manual_seed(r)) for r in range(B)]
     dec.load_prompts(prompts)
@@ -118,6 +135,8 @@ def run_leg(torch, dec, shape, model, B, K, W, P, max_seq, mode):
     assert not finished, "requests finished inside the timed region; lower --steps"
     steps1 = dec.meta["step"].cpu().tolist()
     assert steps1 == [s0 + K for s0 in steps0], f"timed region did not run exactly K={K} decode steps for every request: {steps0} -> {steps1}"
+    if stage_profile:
+        print_stage_profile(dec, B)
     wall_ms = (t1 - t0) * 1e3
     kernel_ms = st["last_launch_ms"]
     ms_per_step = wall_ms / K
@@ -158,6 +177,8 @@ def main():
                     help="qwen3-8b: the headline dense shape; qwen3-30b-a3b: the mixture-of-experts shape (128 experts, top-8), reported alongside")
     ap.add_argument("--no-cpu-baseline", action="store_true")
     ap.add_argument("--calib-copy", action="store_true", help="also run one 1 GiB device-to-device copy (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
+    ap.add_argument("--stage-profile", action="store_true",
+                    help="after each timed launch, print its last iteration's per-stage timeline over all workgroups to stderr")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this build runs the decode megakernel on ONE GPU; --gpus must be 1 "
@@ -195,7 +216,7 @@ def main():
         # max_seq_len is the configuration's 1200 unless the earliest request's K timed steps would not fit.
         max_seq = max(1200, P + W + K + 2 + (0 if B == 1 else 6 * P))
         dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
-        legs.append(run_leg(torch, dec, shape, args.model, B, K, W, P, max_seq, args.mode))
+        legs.append(run_leg(torch, dec, shape, args.model, B, K, W, P, max_seq, args.mode, args.stage_profile))
         dec.mpk.finalize()
         del dec
     del weights
