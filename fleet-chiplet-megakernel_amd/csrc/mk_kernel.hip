@@ -969,24 +969,24 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   if (!ctrl) {
     // weights do not depend on the previous stage: the first outputs' rows are requested before its barrier completes
     if (NL > 0) {
-      u32x4 lb[NL > 0 ? NL : 1][NROW][KL];
-      // the register slots draw first, so a short range is held in registers and only the surplus is parked
+      // A rolling window of U outputs: output i goes to register slot i % U; from the U-th on, the slot's previous
+      // output has landed by then and is parked in LDS first.  The first NL outputs end up parked, the last U stay in the
+      // register slots, and never more than U outputs per wavefront are in flight -- a load the control wavefront issues
+      // (the barrier poll, then the input row) queues behind whatever the CU has in flight, so it must not be the whole
+      // prefetch.  Every load is unconditional (an exhausted ticket re-reads a valid row), so the waits count exactly.
 #pragma unroll
-      for (int j = 0; j < U; j++) {
-        uo[j] = take();
-        if (uo[j] >= 0) load_unit(uo[j], buf[j]);
+      for (int i = 0; i < NL + U; i++) {
+        const int sl = i % U;
+        if (i >= U) {
+#pragma unroll
+          for (int h = 0; h < NROW; h++)
+#pragma unroll
+            for (int kc = 0; kc < KL; kc++) lrows[(((i - U) * NROW + h) * KL + kc) * 64 + lane] = buf[sl][h][kc];
+          lo_[i - U] = uo[sl];
+        }
+        uo[sl] = take();
+        load_unit(uo[sl] >= 0 ? uo[sl] : min(o_begin, n_out - 1), buf[sl]);
       }
-#pragma unroll
-      for (int i = 0; i < NL; i++) {
-        lo_[i] = take();
-        load_unit(lo_[i] >= 0 ? lo_[i] : min(o_begin, n_out - 1), lb[i]);  // unconditional (an exhausted ticket re-reads a valid row)
-      }
-#pragma unroll
-      for (int i = 0; i < NL; i++)
-#pragma unroll
-        for (int h = 0; h < NROW; h++)
-#pragma unroll
-          for (int kc = 0; kc < KL; kc++) lrows[((i * NROW + h) * KL + kc) * 64 + lane] = lb[i][h][kc];
     } else {
 #pragma unroll
       for (int j = 0; j < U; j++) {
