@@ -30,20 +30,25 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #endif
 
 // weight rows in flight per wavefront of the single-token linear (K = 4096 with SwiGLU / K = 4096 plain / K = 12288)
+// (a shallow window and more rows parked in LDS across the barrier beat a deep window: whatever a CU has in flight sits in
+// front of the control wavefront's barrier poll and input-row loads)
 #ifndef MK_TUNE_R8
-#define MK_TUNE_R8 4
+#define MK_TUNE_R8 2
 #endif
 #ifndef MK_TUNE_R8N
-#define MK_TUNE_R8N 4
+#define MK_TUNE_R8N 2
+#endif
+#ifndef MK_TUNE_R4
+#define MK_TUNE_R4 2  // K = 2048
 #endif
 #ifndef MK_TUNE_MOE_R13
-#define MK_TUNE_MOE_R13 4
+#define MK_TUNE_MOE_R13 2  // [gate ; up] row pairs in flight per wavefront (K = 2048)
 #endif
 #ifndef MK_TUNE_MOE_R2
-#define MK_TUNE_MOE_R2 16
+#define MK_TUNE_MOE_R2 1   // output rows (x 8 experts) in flight per wavefront
 #endif
 #ifndef MK_TUNE_NL
-#define MK_TUNE_NL 2
+#define MK_TUNE_NL 3
 #endif
 #ifndef MK_TUNE_R24
 #define MK_TUNE_R24 2
@@ -1140,7 +1145,7 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
     stage_linear_m1_t<24, MK_TUNE_R24, false>(st, c, smem);
   } else if (st.k == 2048) {
     if (silu) stage_linear_m1_t<4, 4, true>(st, c, smem);
-    else stage_linear_m1_t<4, 4, false>(st, c, smem);
+    else stage_linear_m1_t<4, MK_TUNE_R4, false>(st, c, smem);
   } else if (st.k == 1024 && !silu) {
     stage_linear_m1_t<2, 4, false>(st, c, smem);
   } else {
@@ -2944,9 +2949,9 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
       // outputs of one workgroup do not fit the LDS collection window: generic form below
     } else if (silu && !st.ld_in_slot && nx <= 768) {
       if (st.k <= 1024) return stage_moe_linear_m1<2, 4, true>(st, c, smem);
-      if (st.k <= 2048) return stage_moe_linear_m1<4, 3, true>(st, c, smem);
+      if (st.k <= 2048) return stage_moe_linear_m1<4, MK_TUNE_MOE_R13, true>(st, c, smem);
     } else if (!silu && (st.flags & MK_F_MOE_COMBINE) && st.ld_in_slot && st.topk == 8 && nx <= 768) {
-      if (st.k <= 1024) return stage_moe_linear_m1<2, 2, false>(st, c, smem);
+      if (st.k <= 1024) return stage_moe_linear_m1<2, MK_TUNE_MOE_R2, false>(st, c, smem);
     }
   }
   if (M > 1) {
