@@ -1670,6 +1670,9 @@ __device__ __forceinline__ void stage_linear_mfma_tiles(CStage &st, Ctx &c, cons
 // 9..64 tokens.  SwiGLU stages number their weight tiles gate, up, gate, up ...; with three tiles per wavefront the
 // middle pair straddles the two streaming wavefronts and is joined through LDS in the epilogue.
 #define MK_XRES_STEPS 8  // steps per pass
+#ifndef MK_TUNE_XRES_PRE
+#define MK_TUNE_XRES_PRE 6  // ring steps requested before the previous stage's barrier is awaited
+#endif
 struct XresPlan {
   int S;       // K slices per tile range (0: this form cannot run the stage)
   int groups;  // tile ranges
@@ -1779,10 +1782,13 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
         aa[t][1] = __builtin_nontemporal_load((const bf16x8 *)(wrow[t] + step * step_stride + half_stride));
       }
     };
-    // weights do not depend on the previous stage: the first NB steps are requested before its barrier is awaited
+    // weights do not depend on the previous stage: the first NBP steps are requested before its barrier is awaited, the
+    // rest of the ring right after the first pass's token rows (what a CU has in flight sits in front of the barrier
+    // poll and of the row requests)
+    constexpr int NBP = MK_TUNE_XRES_PRE < NB ? MK_TUNE_XRES_PRE : NB;
     if (has_tile) {
 #pragma unroll
-      for (int j = 0; j < NB; j++) w_load(j, a[j]);
+      for (int j = 0; j < NBP; j++) w_load(j, a[j]);
     }
     // Token rows come from other workgroups and are read with cached loads, so what this die's caches hold of them must
     // go first.  The invalidate is issued BEFORE the barrier is awaited: nothing on this die reads the stage's input
@@ -1824,7 +1830,13 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
     const int n_refill = npass - 1;
     auto do_pass = [&](int pass, auto refill_c) {
       constexpr bool REFILL = decltype(refill_c)::value;
-      if (pass == 0 || loader) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      if (pass == 0 && has_tile && NBP < NB) {
+        // the token rows of pass 0 have landed once nothing but the ring steps requested after them is outstanding
+        static_assert((NB - NBP) * TW * 2 <= 63, "vmcnt range");
+        asm volatile("s_waitcnt vmcnt(%0)" ::"n"((NB - NBP) * TW * 2) : "memory");
+      } else if (pass == 0 || loader) {
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+      }
       __syncthreads();
       if (pass == 0) MK_MARK(c, 1);
       if (loader && active && pass + 1 < npass) stage_pass(pass + 1, wave - NSW, MK_WAVES - NSW);
@@ -1839,6 +1851,11 @@ __device__ __forceinline__ void stage_linear_mfma_xres(CStage &st, Ctx &c, const
       }
     };
     if (active) stage_pass(0, wave, MK_WAVES);
+    __builtin_amdgcn_sched_barrier(0);
+    if (has_tile) {
+#pragma unroll
+      for (int j = NBP; j < NB; j++) w_load(j, a[j]);
+    }
     __builtin_amdgcn_sched_barrier(0);
     int pass = 0;
     for (; pass < n_refill; pass++) do_pass(pass, std::true_type{});
