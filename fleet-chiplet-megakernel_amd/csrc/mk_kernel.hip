@@ -41,11 +41,18 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_R4
 #define MK_TUNE_R4 2  // K = 2048
 #endif
+#ifndef MK_TUNE_MOE_M1_R13
+#define MK_TUNE_MOE_M1_R13 2  // single-token expert W13: [gate ; up] row pairs in flight per wavefront (K = 2048)
+#endif
+#ifndef MK_TUNE_MOE_M1_R2
+#define MK_TUNE_MOE_M1_R2 1   // single-token expert W2: output rows (x 8 experts) in flight per wavefront
+#endif
+// units per group of the multi-token expert linears (W13 / W2)
 #ifndef MK_TUNE_MOE_R13
-#define MK_TUNE_MOE_R13 2  // [gate ; up] row pairs in flight per wavefront (K = 2048)
+#define MK_TUNE_MOE_R13 4
 #endif
 #ifndef MK_TUNE_MOE_R2
-#define MK_TUNE_MOE_R2 1   // output rows (x 8 experts) in flight per wavefront
+#define MK_TUNE_MOE_R2 16
 #endif
 #ifndef MK_TUNE_NL
 #define MK_TUNE_NL 3
@@ -2966,9 +2973,9 @@ __device__ __forceinline__ void stage_moe_linear(CStage &st, Ctx &c, int M, char
       // outputs of one workgroup do not fit the LDS collection window: generic form below
     } else if (silu && !st.ld_in_slot && nx <= 768) {
       if (st.k <= 1024) return stage_moe_linear_m1<2, 4, true>(st, c, smem);
-      if (st.k <= 2048) return stage_moe_linear_m1<4, MK_TUNE_MOE_R13, true>(st, c, smem);
+      if (st.k <= 2048) return stage_moe_linear_m1<4, MK_TUNE_MOE_M1_R13, true>(st, c, smem);
     } else if (!silu && (st.flags & MK_F_MOE_COMBINE) && st.ld_in_slot && st.topk == 8 && nx <= 768) {
-      if (st.k <= 1024) return stage_moe_linear_m1<2, MK_TUNE_MOE_R2, false>(st, c, smem);
+      if (st.k <= 1024) return stage_moe_linear_m1<2, MK_TUNE_MOE_M1_R2, false>(st, c, smem);
     }
   }
   if (M > 1) {
