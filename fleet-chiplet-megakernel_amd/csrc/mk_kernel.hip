@@ -1038,6 +1038,10 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   float ures[U];
 #pragma unroll
   for (int j = 0; j < U; j++) ures[j] = (has_res && uo[j] >= 0) ? bf2f(ldc_u16(res + uo[j])) : 0.f;
+  // (the residual values of the parked outputs too: requested together here, not one round trip per parked output)
+  float lres[NL > 0 ? NL : 1];
+#pragma unroll
+  for (int i = 0; i < (NL > 0 ? NL : 1); i++) lres[i] = (NL > 0 && has_res && !ctrl && lo_[i] >= 0) ? bf2f(ldc_u16(res + lo_[i])) : 0.f;
   const u32x4 *xs4 = (const u32x4 *)xs;
   u32x4 xr[KL <= 8 ? KL : 1];
   if (KL <= 8) {
@@ -1057,8 +1061,7 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
         }
 #pragma unroll
         for (int h = 0; h < NROW; h++) a[h] = wave_sum(a[h]);
-        const float r = has_res ? bf2f(ldc_u16(res + lo_[i])) : 0.f;
-        const float v = SILU ? silu_mul(a[0], a[NROW - 1]) : a[0] + r;
+        const float v = SILU ? silu_mul(a[0], a[NROW - 1]) : a[0] + lres[i];
         if (lane == 0) so[lo_[i] - o_begin] = (uint16_t)f2bf(v);
       }
     }
