@@ -3155,13 +3155,25 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     a.h = item - a.t * nkv;
     a.p = __builtin_amdgcn_readfirstlane(c.sh_tok[a.t]);
     const int L = a.p + 1;
-    int C = (L + 63) / 64;  // at least 64 positions (4 per lane group) per chunk
-    a.C = C > cmax ? cmax : C;
-    if (a.cidx >= a.C) return false;
-    a.start = (int)(((long long)L * a.cidx) / a.C);
-    a.end = (int)(((long long)L * (a.cidx + 1)) / a.C);
     a.t0 = __builtin_amdgcn_readfirstlane(c.sh_tok[2 * MK_MAX_TOKENS + a.t]);
     a.p0 = __builtin_amdgcn_readfirstlane(c.sh_tok[a.t0]);
+    const int Lc = min(a.p0, L);  // cached positions this token sees
+    // Up to 64 cached positions (4 per lane group: one block) per chunk.  While workgroups are plenty, one more chunk
+    // takes this iteration's new positions and nothing else: that chunk also prepares their K/V rows and appends the
+    // newest one, which would otherwise make it the last to finish.
+    const int Cd = (Lc + 63) / 64 + 1;
+    const bool own_chunk = L > 64 && Cd <= cmax;
+    int C = own_chunk ? Cd : (L + 63) / 64;
+    a.C = C > cmax ? cmax : C;
+    if (a.cidx >= a.C) return false;
+    if (own_chunk) {
+      const int nc = a.C - 1;
+      a.start = a.cidx < nc ? (int)(((long long)Lc * a.cidx) / nc) : Lc;
+      a.end = a.cidx < nc ? (int)(((long long)Lc * (a.cidx + 1)) / nc) : L;
+    } else {
+      a.start = (int)(((long long)L * a.cidx) / a.C);
+      a.end = (int)(((long long)L * (a.cidx + 1)) / a.C);
+    }
     a.pages = rt.kv_indices + __builtin_amdgcn_readfirstlane(c.sh_tok[3 * MK_MAX_TOKENS + a.t]);
     a.new_lo = max(a.start, a.p0);  // new positions handled here: [new_lo, end)
     a.n_new = a.end > a.new_lo ? a.end - a.new_lo : 0;
