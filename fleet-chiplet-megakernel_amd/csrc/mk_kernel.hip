@@ -57,6 +57,9 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_NL
 #define MK_TUNE_NL 3
 #endif
+#ifndef MK_TUNE_W0_KL
+#define MK_TUNE_W0_KL 8  // single-token linears with rows of at least this many KB arrive without a workgroup barrier
+#endif
 #ifndef MK_TUNE_R24
 #define MK_TUNE_R24 2
 #endif
@@ -82,6 +85,8 @@ struct Ctx {
                       // MoE stage that last filled the workgroup's expert list (kept outside the stages' scratch LDS)
   int seq;            // stages executed so far by this workgroup
   bool wrote_through; // the stage that just ran wrote all its outputs with write-through stores: no L2 write-back at its barrier
+  bool arrive_w0;     // ... and all of them from wavefront 0, after a workgroup barrier, having reset the next stage's work
+                      // counter itself: the arrival then needs no workgroup barrier of its own (see barrier_arrive)
   // A split-K linear whose consumer is a full-row norm leaves its K-slice partials unsummed: the norm stage, which reads
   // every row anyway, sums them (slice order, then the residual, then one rounding: the same arithmetic).
   int defer_S;            // slices left unsummed by the stage that just ran (0: none)
@@ -258,6 +263,19 @@ __device__ __forceinline__ bool spin_ok(MkSync *s, unsigned &spins, unsigned whe
 // in that die's L2).  Nothing is returned, so nobody waits on the atomic.
 __device__ __forceinline__ void barrier_arrive(Ctx &c) {
   MkSync *s = c.sync;
+  if (c.arrive_w0) {
+    // Only wavefront 0 has stores outstanding: it waits for them and posts the arrival; the other wavefronts go straight
+    // on to the next stage, whose weight prefetch is then in flight while those stores are still being acknowledged
+    // (about a microsecond per stage in which the CU otherwise requests nothing).
+    c.arrive_w0 = false;
+    if (__builtin_amdgcn_readfirstlane(threadIdx.x >> 6) == 0) asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+    c.seq++;
+    c.epoch++;
+    if (threadIdx.x == 0) __hip_atomic_fetch_add(&s->local_ctr[c.xcd][0], 1u, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+    c.wrote_through = false;
+    c.pending = true;
+    return;
+  }
   asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
   c.seq++;
   if (threadIdx.x == 0) c.sh_ticket[c.seq & 1] = 0;  // the counter of the stage that starts now (last used two stages ago)
@@ -1020,11 +1038,24 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   // Outputs are collected in LDS and written out together once every worker is done: one write-through request per
   // 128-byte line instead of one 2-byte write per output.
   uint16_t *so = (uint16_t *)(smem + MK_OUT_OFFSET);
+  // Rows of 8 KB and more: wavefront 0 alone writes the outputs out, so that the arrival needs no workgroup barrier and
+  // the other wavefronts go straight on to the next stage's prefetch (barrier_arrive).  With shorter rows (stages of a
+  // few microseconds) the earlier prefetch gains less than it costs wavefront 0's arrival and next poll, which then
+  // queue behind it.
+  constexpr bool W0 = KL >= MK_TUNE_W0_KL;
   auto flush = [&]() {
+    if (W0 && tid == 0) c.sh_ticket[(c.seq + 1) & 1] = 0;  // the next stage's work counter (idle since the previous stage)
     __syncthreads();
     uint16_t *dst = (uint16_t *)st.out + o_begin;
-    for (int i = tid; i < o_end - o_begin; i += MK_THREADS) stc_u16(dst + i, so[i]);
+    if (W0) {
+      if (wave == 0) {
+        for (int i = lane; i < o_end - o_begin; i += 64) stc_u16(dst + i, so[i]);
+      }
+    } else {
+      for (int i = tid; i < o_end - o_begin; i += MK_THREADS) stc_u16(dst + i, so[i]);
+    }
     c.wrote_through = true;
+    c.arrive_w0 = W0;
   };
   if (ctrl) {  // the control wavefront has done its part: it now streams rows like the others
 #pragma unroll
@@ -3879,6 +3910,7 @@ __device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRunt
   c.seq = 0;
   c.defer_S = 0;
   c.wrote_through = false;
+  c.arrive_w0 = false;
   if (threadIdx.x == 0) {
     sh_ticket[0] = sh_ticket[1] = 0;
     sh_ticket[2] = -2;
