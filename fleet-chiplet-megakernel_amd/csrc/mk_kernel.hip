@@ -953,7 +953,7 @@ __device__ __forceinline__ void stage_x_m1_wave(CStage &st, const Ctx &c, uint32
 // busy across the grid barrier, and a slot is refilled from the workgroup's ticket counter as soon as it is consumed.
 // Reference tasks: linear_kernel_ck (tasks/mi300/linear_ck_mi300.cuh:289-619), gang_linear_silu_kernel
 // (tasks/mi300/gang_linear_mi300.cuh:359-576).
-template <int KL, int R, bool SILU>
+template <int KL, int R, bool SILU, bool W0OK>
 __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem) {
   const int tid = threadIdx.x, lane = tid & 63, wave = __builtin_amdgcn_readfirstlane(tid >> 6);
   constexpr int K8 = KL * 64;
@@ -1042,7 +1042,8 @@ __device__ __forceinline__ void stage_linear_m1_t(CStage &st, Ctx &c, char *smem
   // the other wavefronts go straight on to the next stage's prefetch (barrier_arrive).  With shorter rows (stages of a
   // few microseconds) the earlier prefetch gains less than it costs wavefront 0's arrival and next poll, which then
   // queue behind it.
-  constexpr bool W0 = KL >= MK_TUNE_W0_KL;
+  // (only in the kernel instantiation for single-token graphs: W0OK)
+  constexpr bool W0 = W0OK && KL >= MK_TUNE_W0_KL;
   auto flush = [&]() {
     if (W0 && tid == 0) c.sh_ticket[(c.seq + 1) & 1] = 0;  // the next stage's work counter (idle since the previous stage)
     __syncthreads();
@@ -1173,6 +1174,7 @@ __device__ __forceinline__ void stage_linear_m1_generic(CStage &st, Ctx &c, char
   }
 }
 
+template <bool W0OK>
 __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) {
   const bool silu = st.flags & MK_F_SILU;
   // the tuned forms collect a workgroup's outputs in the LDS window [MK_OUT_OFFSET, MK_MOE_OFFSET)
@@ -1180,15 +1182,15 @@ __device__ __forceinline__ void stage_linear_m1(CStage &st, Ctx &c, char *smem) 
   if (!fits) {
     stage_linear_m1_generic(st, c, smem);
   } else if (st.k == 4096) {
-    if (silu) stage_linear_m1_t<8, MK_TUNE_R8, true>(st, c, smem);
-    else stage_linear_m1_t<8, MK_TUNE_R8N, false>(st, c, smem);
+    if (silu) stage_linear_m1_t<8, MK_TUNE_R8, true, W0OK>(st, c, smem);
+    else stage_linear_m1_t<8, MK_TUNE_R8N, false, W0OK>(st, c, smem);
   } else if (st.k == 12288 && !silu) {
-    stage_linear_m1_t<24, MK_TUNE_R24, false>(st, c, smem);
+    stage_linear_m1_t<24, MK_TUNE_R24, false, W0OK>(st, c, smem);
   } else if (st.k == 2048) {
-    if (silu) stage_linear_m1_t<4, 4, true>(st, c, smem);
-    else stage_linear_m1_t<4, MK_TUNE_R4, false>(st, c, smem);
+    if (silu) stage_linear_m1_t<4, 4, true, W0OK>(st, c, smem);
+    else stage_linear_m1_t<4, MK_TUNE_R4, false, W0OK>(st, c, smem);
   } else if (st.k == 1024 && !silu) {
-    stage_linear_m1_t<2, 4, false>(st, c, smem);
+    stage_linear_m1_t<2, 4, false, W0OK>(st, c, smem);
   } else {
     stage_linear_m1_generic(st, c, smem);
   }
@@ -3802,8 +3804,8 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
         case MK_OP_EMBED: stage_embed(st, c, rt, M); break;
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
         case MK_OP_LINEAR:
-          if constexpr (MAXM == 1) stage_linear_m1(st, c, smem);
-          else if (M == 1) stage_linear_m1(st, c, smem);
+          if constexpr (MAXM == 1) stage_linear_m1<true>(st, c, smem);
+          else if (M == 1) stage_linear_m1<false>(st, c, smem);
           else if (linear_small_ok(st, c, M)) {
             if (M <= 2) stage_linear_small_dispatch<2>(st, c, M, smem);
             else if (M <= 4) stage_linear_small_dispatch<4>(st, c, M, smem);
