@@ -88,7 +88,7 @@ def cpu_baseline(shape, n_layers_sample=2, steps=3, context=80):
 # times the steps of its launch (measured on the default 1024-step launches, whose contexts they average over; a launch of
 # another length holds different KV rows and the figure is then approximate); a batch size without a committed counter
 # pass reports null.
-MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): (15.6243e12 + 15.73e9) / 1024, ("qwen3-8b", 64): (25.9040e12 + 1.4045e12) / 1024}
+MEASURED_TRAFFIC_BYTES_PER_STEP = {("qwen3-8b", 1): (15.6246e12 + 15.74e9) / 1024, ("qwen3-8b", 64): (25.8955e12 + 1.4045e12) / 1024}
 
 
 def print_stage_profile(dec, B, out=sys.stderr):
