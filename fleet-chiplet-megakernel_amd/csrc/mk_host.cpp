@@ -93,6 +93,7 @@ struct mk_graph {
   int G = 0;
   std::vector<Tensor> tensors;
   std::vector<Task> tasks;
+  std::vector<Task> ltasks;  // what lower() walks: `tasks` with composite tasks expanded
   bool compiled = false;
   bool host_only = false;  // created with device < 0: records, validates, lowers and emits the task graph, never launches
   std::vector<void *> allocs;
@@ -216,15 +217,24 @@ std::string fmt(const char *f, ...) {
   return buf;
 }
 
+// operands are listed inputs first, outputs last: how many of a task's operands are outputs
+int num_outputs(const Task &t) {
+  if (t.name == "argmax_partial") return 2;
+  if (t.name == "gang_attn_split_kv_mi300") return 3;
+  if (t.name == "paged_attention_ck_fmha_split_kv_mi300" || t.name == "paged_attention_split_kv_mi300") return 2;
+  if (t.name == "moe_topk_softmax_mi300") return 3;
+  return 1;
+}
+
 // Lower one linear-type task (optionally preceded by a norm task whose output it consumes, optionally
 // followed by a silu_mul consuming its output) into stages.
 int lower_linear(mk_graph *g, size_t &i) {
   const Task *norm = nullptr;
-  if (is_norm(g->tasks[i].name)) {
-    norm = &g->tasks[i];
+  if (is_norm(g->ltasks[i].name)) {
+    norm = &g->ltasks[i];
     i++;
   }
-  const Task &lt = g->tasks[i];
+  const Task &lt = g->ltasks[i];
   bool res, silu;
   int extra;
   if (!linear_kind(lt.name, &res, &silu, &extra)) return fail(MK_EINVAL, "internal: '%s' is not a linear", lt.name.c_str());
@@ -236,7 +246,7 @@ int lower_linear(mk_graph *g, size_t &i) {
   if (lt.name == "splitk_linear_mi300" && g->tensors[out_id].dtype == MK_DT_F32) {
     // the reference's two-task split-K: partial products into an fp32 workspace, then splitk_reduce [workspace, residual,
     // output] sums the slices and adds the residual.  The pair is one stage here; the workspace is never written.
-    const Task *rd = i + 1 < g->tasks.size() ? &g->tasks[i + 1] : nullptr;
+    const Task *rd = i + 1 < g->ltasks.size() ? &g->ltasks[i + 1] : nullptr;
     if (!rd || rd->name != "splitk_reduce_mi300" || rd->ops.size() != 3 || rd->ops[0] != out_id)
       return fail(MK_EUNSUPPORTED, "splitk_linear_mi300 into an fp32 workspace must be followed by splitk_reduce_mi300 over that workspace");
     res = true;
@@ -262,9 +272,9 @@ int lower_linear(mk_graph *g, size_t &i) {
   st.eps = g->cfg.rms_eps;
   // a following silu_mul over this linear's (library-owned) output is folded into the epilogue
   const Task *act = nullptr;
-  if (!silu && !res && i + 1 < g->tasks.size() && g->tasks[i + 1].name == "silu_mul" && g->tasks[i + 1].ops.size() == 2 &&
-      g->tasks[i + 1].ops[0] == out_id && tout.kind == T_OWNED) {
-    act = &g->tasks[i + 1];
+  if (!silu && !res && i + 1 < g->ltasks.size() && g->ltasks[i + 1].name == "silu_mul" && g->ltasks[i + 1].ops.size() == 2 &&
+      g->ltasks[i + 1].ops[0] == out_id && tout.kind == T_OWNED) {
+    act = &g->ltasks[i + 1];
   }
   int final_out = out_id;
   if (silu || act) {
@@ -342,14 +352,17 @@ int lower_linear(mk_graph *g, size_t &i) {
 }
 
 // silu_mul_linear_with_residual [input [tokens, 2I], weight [H, I], residual, output]: out = silu_mul(input) W^T + residual.
-// When `input` was produced by the linear stage right before it, the activation moves into that stage's epilogue
-// (single rounding, like the fused gate/up task) writing a library-owned [tokens, I] tensor, and the gate/up tensor
-// itself is no longer written; which rows are gate and which are up comes from the producer's weight view (a
-// shuffled [gate ; up] view) or, for a physically interleaved weight, from the producer's grid (one block per
-// half-group, which is how the reference drivers size it).  Otherwise a standalone activation stage reads `input` as
-// [gate | up] halves, the layout the reference task kernel reads (tasks/ampere/silu_mul_linear.cuh:78-80).
+// Which columns of `input` are gate and which are up:
+//   * `input` was produced by the linear stage right before it through a shuffled [gate ; up] weight view: the view says so;
+//   * params[0] > 0 (the builder that interleaved a physical weight passes its group size): groups of
+//     [gate x params[0] ; up x params[0]];
+//   * otherwise [gate | up] halves, the layout the reference task kernel reads (tasks/mi300/silu_mul_linear_mi300.cuh:40-42,
+//     tasks/ampere/silu_mul_linear.cuh:78-80).
+// When the producer is that linear stage and no later task reads `input`, the activation moves into the producer's
+// epilogue (single rounding, like the fused gate/up task) writing a library-owned [tokens, I] tensor and the gate/up tensor
+// itself is no longer written.  Otherwise a standalone activation stage reads `input`.
 int lower_silu_mul_linear(mk_graph *g, size_t &i) {
-  const Task &t = g->tasks[i];
+  const Task &t = g->ltasks[i];
   if (t.ops.size() != 4) return fail(MK_EINVAL, "silu_mul_linear_with_residual expects 4 operands");
   const Tensor &x = g->tensors[t.ops[0]], &w = g->tensors[t.ops[1]], &r = g->tensors[t.ops[2]], &o = g->tensors[t.ops[3]];
   const int B = g->cfg.max_num_batched_tokens;
@@ -364,34 +377,50 @@ int lower_silu_mul_linear(mk_graph *g, size_t &i) {
   if (rc) return rc;
   const bool have_producer = g->last_linear_stage >= 0 && g->last_linear_stage == (int)g->stages.size() - 1;
   MkStage *prev = have_producer ? &g->stages.back() : nullptr;
-  if (prev && prev->op == MK_OP_LINEAR && prev->out == x.ptr && !(prev->flags & (MK_F_SILU | MK_F_RES)) && prev->n == 2 * I) {
-    int half = 0;
-    if (prev->w.nseg == 2 && prev->w.seg_rows[0] == prev->w.seg_rows[1]) {
-      half = prev->w.seg_rows[0];
-    } else if (prev->w.nseg == 1) {
-      const Task &pt = g->tasks[g->last_linear_task];
-      const int blocks = pt.grid[0] * pt.grid[1] * pt.grid[2];
-      half = (blocks >= 2 && (2 * I) % blocks == 0) ? 2 * I / blocks : I;
+  if (prev && !(prev->op == MK_OP_LINEAR && prev->out == x.ptr && !(prev->flags & (MK_F_SILU | MK_F_RES)) && prev->n == 2 * I)) prev = nullptr;
+  int half = I;
+  const char *how = "[gate | up] halves";
+  if (prev && prev->w.nseg == 2 && prev->w.seg_rows[0] == prev->w.seg_rows[1]) {
+    half = prev->w.seg_rows[0];
+    how = "groups of the producer's shuffled weight view";
+  } else if (!t.params.empty() && t.params[0] > 0) {
+    half = t.params[0];
+    how = "groups given by the caller";
+  }
+  if (half <= 0 || I % half) return fail(MK_EINVAL, "silu_mul_linear_with_residual: gate/up groups of %d rows do not divide the intermediate size %d", half, I);
+  // folding stops the gate/up tensor from being written: no later task may read it before some task writes it again
+  // (drivers reuse one gate/up buffer for every layer)
+  bool read_later = false;
+  for (size_t j = i + 1; j < g->ltasks.size() && !read_later; j++) {
+    const Task &lt = g->ltasks[j];
+    const size_t n_in = lt.ops.size() - (size_t)num_outputs(lt);
+    bool rewritten = false;
+    for (size_t a = 0; a < lt.ops.size(); a++) {
+      if (lt.ops[a] != t.ops[0]) continue;
+      if (a < n_in) read_later = true;
+      else rewritten = true;
     }
-    if (half <= 0 || (2 * I) % (2 * half)) return fail(MK_EINVAL, "silu_mul_linear_with_residual: cannot tell gate rows from up rows of '%s'", x.name.c_str());
+    if (rewritten) break;
+  }
+  if (prev && !read_later) {
     prev->flags |= MK_F_SILU;
     prev->silu_half = half;
     prev->out = mid;
     prev->ld_out = I;
-    g->stage_desc.back() += fmt(" [+silu half=%d folded in from silu_mul_linear_with_residual; output is library-owned]", half);
+    g->stage_desc.back() += fmt(" [+silu half=%d (%s) folded in from silu_mul_linear_with_residual; output is library-owned]", half, how);
   } else {
     MkStage a;
     memset(&a, 0, sizeof(a));
     a.op = MK_OP_SILU_MUL;
     a.n = I;
-    a.silu_half = I;
-    a.groups = 1;
+    a.silu_half = half;
+    a.groups = I / half;
     a.in = x.ptr;
     a.ld_in = (int)x.strides[0];
     a.out = mid;
     a.ld_out = I;
     g->stages.push_back(a);
-    g->stage_desc.push_back(fmt("SILU_MUL %s -> (library) n=%d half=%d", x.name.c_str(), I, I));
+    g->stage_desc.push_back(fmt("SILU_MUL %s -> (library) n=%d half=%d (%s)", x.name.c_str(), I, half, how));
   }
   MkStage st;
   memset(&st, 0, sizeof(st));
@@ -420,8 +449,8 @@ int lower_silu_mul_linear(mk_graph *g, size_t &i) {
 // A merge task that closes a split-KV attention task: [lse, chunked output, final output].  Returns the final
 // output's tensor id when task `j` is such a merge over the attention's chunked output, -1 otherwise.
 int merge_output_of(mk_graph *g, size_t j, const char *merge_name, int chunked_out_id) {
-  if (j >= g->tasks.size()) return -1;
-  const Task &m = g->tasks[j];
+  if (j >= g->ltasks.size()) return -1;
+  const Task &m = g->ltasks[j];
   if (m.name != merge_name || m.ops.size() != 3 || m.ops[1] != chunked_out_id) return -1;
   return m.ops[2];
 }
@@ -431,7 +460,7 @@ int merge_output_of(mk_graph *g, size_t j, const char *merge_name, int chunked_o
 // num_kv_chunks > 1 together with the merge task that must follow (the stage writes the merge's output; the chunked
 // accumulator and the log-sum-exp tensor of the reference's two-task form are never touched).
 int lower_attention(mk_graph *g, size_t &i) {
-  const Task &t0 = g->tasks[i];
+  const Task &t0 = g->ltasks[i];
   int in_id, kc_id, vc_id, qn_id, kn_id, cos_id, sin_id, out_id, qws_id = -1, nq = 0, chunks = 1;
   size_t consumed = 1;
   const char *merge = nullptr;
@@ -442,9 +471,12 @@ int lower_attention(mk_graph *g, size_t &i) {
     nq = t0.params[0];
     chunks = t0.params[6];
     merge = "gang_attn_merge_mi300";
-  } else if (t0.name == "paged_attention" || t0.name == "paged_attention_split_kv_mi300") {
-    const bool split = t0.name != "paged_attention";
-    if (t0.ops.size() != (split ? 9u : 8u) || t0.params.size() < (split ? 7u : 6u)) return fail(MK_EINVAL, "%s: wrong number of operands / params", t0.name.c_str());
+  } else if (t0.name == "paged_attention" || t0.name == "paged_attention_split_kv_mi300" || t0.name == "attention") {
+    // "attention" (python/mirage/mpk/persistent_kernel.py:587-650) is the form with one contiguous cache row range per
+    // request, [requests, seq_len, kv heads, head_dim]: a paged cache whose pages are max_seq_length long
+    const bool split = t0.name == "paged_attention_split_kv_mi300";
+    const size_t need_params = t0.name == "attention" ? 4u : (split ? 7u : 6u);
+    if (t0.ops.size() != (split ? 9u : 8u) || t0.params.size() < need_params) return fail(MK_EINVAL, "%s: wrong number of operands / params", t0.name.c_str());
     in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
     out_id = t0.ops.back();
     nq = t0.params[0];
@@ -454,9 +486,9 @@ int lower_attention(mk_graph *g, size_t &i) {
     }
   } else if (t0.name == "kv_cache_update_mi300") {
     if (t0.ops.size() != 8 || t0.params.size() < 7) return fail(MK_EINVAL, "kv_cache_update_mi300 expects 8 operands / 7 params");
-    if (i + 1 >= g->tasks.size() || g->tasks[i + 1].name != "paged_attention_ck_fmha_split_kv_mi300")
+    if (i + 1 >= g->ltasks.size() || g->ltasks[i + 1].name != "paged_attention_ck_fmha_split_kv_mi300")
       return fail(MK_EUNSUPPORTED, "kv_cache_update_mi300 must be followed by paged_attention_ck_fmha_split_kv_mi300");
-    const Task &t1 = g->tasks[i + 1];
+    const Task &t1 = g->ltasks[i + 1];
     if (t1.ops.size() != 5 || t1.params.size() < 9) return fail(MK_EINVAL, "paged_attention_ck_fmha_split_kv_mi300 expects 5 operands / 9 params");
     in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
     qws_id = t0.ops[7];
@@ -548,7 +580,7 @@ bool rows_contiguous_3d(const Tensor &t) { return t.ndims == 3 && t.strides[2] =
 // the routing follows directly, single-token iterations route inside that linear and this stage runs for multi-token
 // iterations only.
 int lower_moe_topk(mk_graph *g, size_t &i, bool *inline_next) {
-  const Task &t = g->tasks[i];
+  const Task &t = g->ltasks[i];
   if (t.ops.size() != 4) return fail(MK_EINVAL, "%s expects 4 operands", t.name.c_str());
   const Tensor &lg = g->tensors[t.ops[0]], &tw = g->tensors[t.ops[1]], &ri = g->tensors[t.ops[2]], &mk = g->tensors[t.ops[3]];
   const int B = g->cfg.max_num_batched_tokens;
@@ -561,10 +593,10 @@ int lower_moe_topk(mk_graph *g, size_t &i, bool *inline_next) {
   if (ri.ndims != 2 || ri.dtype != MK_DT_I32 || ri.dims[0] != E || ri.dims[1] < B || ri.strides[1] != 1)
     return fail(MK_EINVAL, "%s: routing indices must be [experts, tokens] int32", t.name.c_str());
   if (mk.dtype != MK_DT_I32 || mk.elems() < (size_t)E + 1) return fail(MK_EINVAL, "%s: mask must hold experts+1 int32", t.name.c_str());
-  if (i + 1 >= g->tasks.size() || !is_moe_linear(g->tasks[i + 1].name) || g->tasks[i + 1].ops.size() != 5 || g->tasks[i + 1].ops[2] != t.ops[2] ||
-      g->tasks[i + 1].ops[3] != t.ops[3])
+  if (i + 1 >= g->ltasks.size() || !is_moe_linear(g->ltasks[i + 1].name) || g->ltasks[i + 1].ops.size() != 5 || g->ltasks[i + 1].ops[2] != t.ops[2] ||
+      g->ltasks[i + 1].ops[3] != t.ops[3])
     return fail(MK_EUNSUPPORTED, "%s must be followed by the per-expert linear that consumes its routing table (it publishes the active-expert mask)", t.name.c_str());
-  *inline_next = g->tensors[g->tasks[i + 1].ops[0]].ndims == 2;
+  *inline_next = g->tensors[g->ltasks[i + 1].ops[0]].ndims == 2;
   MkStage st;
   memset(&st, 0, sizeof(st));
   st.op = MK_OP_MOE_TOPK;
@@ -588,7 +620,7 @@ int lower_moe_topk(mk_graph *g, size_t &i, bool *inline_next) {
 // slot of a token sees the same row: W13) or [tokens, topk, K] (W2).  A directly following moe_silu_mul / moe_mul_sum_add
 // over its output becomes the epilogue.
 int lower_moe_linear(mk_graph *g, size_t &i, const MkStage *router) {
-  const Task &t = g->tasks[i];
+  const Task &t = g->ltasks[i];
   if (t.ops.size() != 5) return fail(MK_EINVAL, "%s expects 5 operands", t.name.c_str());
   const Tensor &x = g->tensors[t.ops[0]], &w = g->tensors[t.ops[1]], &ri = g->tensors[t.ops[2]], &mk = g->tensors[t.ops[3]], &y = g->tensors[t.ops[4]];
   const int B = g->cfg.max_num_batched_tokens;
@@ -642,7 +674,7 @@ int lower_moe_linear(mk_graph *g, size_t &i, const MkStage *router) {
   }
   size_t consumed = 1;
   std::string extra;
-  const Task *nx = i + 1 < g->tasks.size() ? &g->tasks[i + 1] : nullptr;
+  const Task *nx = i + 1 < g->ltasks.size() ? &g->ltasks[i + 1] : nullptr;
   if (nx && nx->name == "moe_silu_mul" && nx->ops.size() == 2 && nx->ops[0] == t.ops[4] && N % 2 == 0) {
     const Tensor &o = g->tensors[nx->ops[1]];
     if (!rows_contiguous_3d(o) || o.dtype != MK_DT_BF16 || o.dims[0] < B || o.dims[1] != topk || o.dims[2] != N / 2)
@@ -678,7 +710,7 @@ int lower_moe_linear(mk_graph *g, size_t &i, const MkStage *router) {
 
 // moe_mul_sum_add_mi300 [expert outputs [tokens,topk,n], routing weights [tokens,topk], residual, output]
 int lower_moe_combine(mk_graph *g, size_t &i, bool fused_single) {
-  const Task &t = g->tasks[i];
+  const Task &t = g->ltasks[i];
   if (t.ops.size() != 4) return fail(MK_EINVAL, "%s expects 4 operands", t.name.c_str());
   const Tensor &x = g->tensors[t.ops[0]], &tw = g->tensors[t.ops[1]], &r = g->tensors[t.ops[2]], &o = g->tensors[t.ops[3]];
   const int B = g->cfg.max_num_batched_tokens;
@@ -713,10 +745,58 @@ int lower(mk_graph *g) {
   g->stage_desc.clear();
   g->weight_bytes = 0;
   g->last_linear_task = g->last_linear_stage = -1;
-  size_t i = 0;
   const int B = g->cfg.max_num_batched_tokens;
-  while (i < g->tasks.size()) {
-    const Task &t = g->tasks[i];
+  // The list that is lowered: the recorded tasks, with the composite ones spelt out as the tasks they stand for (the
+  // task graph handed back to the caller keeps them as recorded).
+  g->ltasks.clear();
+  for (const Task &t : g->tasks) {
+    if (t.name == "rmsnorm_linear") {
+      // [input, norm weight, linear weight, output] (python/mirage/mpk/persistent_kernel.py:566-585): RMSNorm into a
+      // library-owned row buffer, then a plain linear over it
+      if (t.ops.size() != 4) return fail(MK_EINVAL, "rmsnorm_linear expects 4 operands");
+      const Tensor &x = g->tensors[t.ops[0]];
+      if (x.ndims != 2) return fail(MK_EINVAL, "rmsnorm_linear: input must be 2-D");
+      const std::string nm = "rmsnorm_linear_norm_out_" + std::to_string(g->ltasks.size());
+      int nid = -1;
+      for (size_t k = 0; k < g->tensors.size(); k++)
+        if (g->tensors[k].name == nm) nid = (int)k;
+      if (nid < 0) {
+        Tensor nt;
+        nt.name = nm;
+        nt.ndims = 2;
+        nt.dtype = x.dtype;
+        nt.kind = T_OWNED;
+        nt.dims[0] = x.dims[0];
+        nt.dims[1] = x.dims[1];
+        nt.strides[0] = x.dims[1];
+        nt.strides[1] = 1;
+        void *p = nullptr;
+        int rc = dev_alloc(g, &p, (size_t)x.dims[0] * x.dims[1] * dtype_size(x.dtype));
+        if (rc) return rc;
+        nt.ptr = p;
+        g->tensors.push_back(nt);
+        nid = (int)g->tensors.size() - 1;
+      }
+      Task n = t, l = t;
+      n.name = "rmsnorm";
+      n.ops = {t.ops[0], t.ops[1], nid};
+      n.maps = {t.maps[0], t.maps[1], t.maps[0]};
+      n.forloop = {t.forloop[0], t.forloop[1], t.forloop[0]};
+      n.params.clear();
+      l.name = "linear";
+      l.ops = {nid, t.ops[2], t.ops[3]};
+      l.maps = {t.maps[0], t.maps[2], t.maps[3]};
+      l.forloop = {t.forloop[0], t.forloop[2], t.forloop[3]};
+      l.params.clear();
+      g->ltasks.push_back(n);
+      g->ltasks.push_back(l);
+    } else {
+      g->ltasks.push_back(t);
+    }
+  }
+  size_t i = 0;
+  while (i < g->ltasks.size()) {
+    const Task &t = g->ltasks[i];
     bool res, silu;
     int extra;
     if (t.name == "embedding") {
@@ -739,7 +819,7 @@ int lower(mk_graph *g) {
       i++;
     } else if (is_norm(t.name)) {
       if (t.ops.size() != 3) return fail(MK_EINVAL, "%s expects 3 operands", t.name.c_str());
-      if (i + 1 < g->tasks.size() && linear_kind(g->tasks[i + 1].name, &res, &silu, &extra) && g->tasks[i + 1].ops[0] == t.ops[2]) {
+      if (i + 1 < g->ltasks.size() && linear_kind(g->ltasks[i + 1].name, &res, &silu, &extra) && g->ltasks[i + 1].ops[0] == t.ops[2]) {
         int rc = lower_linear(g, i);
         if (rc) return rc;
       } else {
@@ -785,7 +865,7 @@ int lower(mk_graph *g) {
       g->stage_desc.push_back(fmt("SILU_MUL %s -> %s n=%d half=%d", x.name.c_str(), o.name.c_str(), st.n, st.silu_half));
       i++;
     } else if (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300" || t.name == "paged_attention" ||
-               t.name == "paged_attention_split_kv_mi300") {
+               t.name == "paged_attention_split_kv_mi300" || t.name == "attention") {
       int rc = lower_attention(g, i);
       if (rc) return rc;
     } else if (t.name == "moe_topk_softmax_mi300") {
@@ -822,11 +902,63 @@ int lower(mk_graph *g) {
       g->stages.push_back(st);
       g->stage_desc.push_back(fmt("SILU_MUL(moe) %s -> %s n=%d rows/token=%d", x.name.c_str(), o.name.c_str(), st.n, st.topk));
       i++;
+    } else if (t.name == "identity") {
+      // [input, output], same shape (python/mirage/mpk/persistent_kernel.py:2153-2172; tasks/ampere/identity.cuh:24-37)
+      if (t.ops.size() != 2) return fail(MK_EINVAL, "identity expects 2 operands");
+      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[t.ops[1]];
+      if (x.ndims != o.ndims || x.ndims < 2 || x.dtype != o.dtype || x.kind == T_SHUFFLED || o.kind == T_SHUFFLED) return fail(MK_EINVAL, "identity: input and output must be stored tensors of one shape and dtype");
+      int64_t inner = 1;
+      for (int d = 0; d < x.ndims; d++) {
+        if (x.dims[d] != o.dims[d] || x.strides[d] != o.strides[d]) return fail(MK_EINVAL, "identity: input and output shapes differ");
+        if (d) inner *= x.dims[d];
+      }
+      if (x.strides[0] != inner) return fail(MK_EINVAL, "identity: rows must be contiguous");
+      if (x.dims[0] < B) return fail(MK_EINVAL, "identity: tensors need at least max_num_batched_tokens=%d rows", B);
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_COPY;
+      st.n = (int)(inner * (int64_t)dtype_size(x.dtype) / 2);  // 16-bit units per token row
+      st.in = x.ptr;
+      st.out = o.ptr;
+      st.ld_in = st.ld_out = st.n;
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("COPY %s -> %s units=%d", x.name.c_str(), o.name.c_str(), st.n));
+      i++;
+    } else if (t.name == "argmax") {
+      // [logits, output] in one task (python/mirage/mpk/persistent_kernel.py:2195-2205): the same two stages as the
+      // partial + reduce pair, over library-owned partials
+      if (t.ops.size() != 2) return fail(MK_EINVAL, "argmax expects 2 operands");
+      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[t.ops[1]];
+      if (x.ndims != 2 || x.dtype != MK_DT_BF16 || o.dtype != MK_DT_I64) return fail(MK_EINVAL, "argmax: logits must be 2-D bf16 and the output int64");
+      void *pv = nullptr, *pi = nullptr;
+      int rc = dev_alloc(g, &pv, sizeof(float) * (size_t)B * g->G);
+      if (rc) return rc;
+      rc = dev_alloc(g, &pi, sizeof(int) * (size_t)B * g->G);
+      if (rc) return rc;
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_ARGMAX_PARTIAL;
+      st.n = (int)x.dims[1];
+      st.in = x.ptr;
+      st.ld_in = (int)x.strides[0];
+      st.aux0 = pv;
+      st.aux1 = pi;
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("ARGMAX_PARTIAL %s n=%d", x.name.c_str(), st.n));
+      MkStage sr;
+      memset(&sr, 0, sizeof(sr));
+      sr.op = MK_OP_ARGMAX_REDUCE;
+      sr.aux0 = pv;
+      sr.aux1 = pi;
+      sr.out = o.ptr;
+      g->stages.push_back(sr);
+      g->stage_desc.push_back(fmt("ARGMAX_REDUCE -> %s", o.name.c_str()));
+      i++;
     } else if (t.name == "argmax_partial") {
       if (t.ops.size() != 3) return fail(MK_EINVAL, "argmax_partial expects 3 operands");
-      if (i + 1 >= g->tasks.size() || g->tasks[i + 1].name != "argmax_reduce" || g->tasks[i + 1].ops.size() != 3)
+      if (i + 1 >= g->ltasks.size() || g->ltasks[i + 1].name != "argmax_reduce" || g->ltasks[i + 1].ops.size() != 3)
         return fail(MK_EUNSUPPORTED, "argmax_partial must be followed by argmax_reduce");
-      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[g->tasks[i + 1].ops[2]];
+      const Tensor &x = g->tensors[t.ops[0]], &o = g->tensors[g->ltasks[i + 1].ops[2]];
       if (x.ndims != 2 || x.dtype != MK_DT_BF16 || o.dtype != MK_DT_I64) return fail(MK_EINVAL, "argmax: logits must be 2-D bf16 and the output int64");
       void *pv = nullptr, *pi = nullptr;
       int rc = dev_alloc(g, &pv, sizeof(float) * (size_t)B * g->G);
@@ -865,18 +997,32 @@ int lower(mk_graph *g) {
 }
 
 // ---- reference-shaped task graph (JSON) ------------------------------------------------------
-// One task per grid block of every recorded operator, events between consecutive operators with
-// the gcd partition-matching rule of the reference (src/kernel/runtime.cc:519-557), task 0 =
-// TERMINATE, task 1 = BEGIN_TASK_GRAPH, event 0 = TERMINATION, event 1 = LAUNCH_DEPENDENT_TASKS over
-// [2, N), last event = END_OF_TASK_GRAPH (runtime.cc:176-182,590-595,1662-1665).
+// The task / event graph the reference's Graph::generate_task_graph builds for the recorded operators
+// (src/kernel/runtime.cc:164-612, printed by print_task_graph :948-1437), re-derived:
+//   * task 0 = TERMINATE, task 1 = BEGIN_TASK_GRAPH; event 0 = TERMINATION, event 1 = LAUNCH_DEPENDENT_TASKS over
+//     [2, #tasks); the last event = END_OF_TASK_GRAPH, triggered by every task of the last operator (:176-182,580-595);
+//   * the first operator's tasks follow in (bid.x, bid.y, bid.z) order and are the "first_tasks" (:499-513);
+//   * between operators i and i+1 the dependency is carried by ONE tensor -- the last (consumer input, producer output)
+//     pair naming the same tensor (:519-531); along each of its dims the number of events is gcd(producer partition,
+//     consumer partition) (:533-557); an event holds the consumer blocks whose index along the mapped grid axis falls
+//     into its slice, in bid order, and is triggered by the producer blocks of the matching slice (:53-140).  Consumer
+//     tasks are therefore stored event by event, not in plain bid order;
+//   * every launch event ends as EVENT_EMPTY, its tasks carrying `dependent_event` (:593-611; the LAUNCH_TASKS /
+//     LAUNCH_MASSIVE_TASKS distinction of :102-105 does not survive that rewrite); tasks without a dependency and the
+//     two bookkeeping tasks carry EVENT_INVALID_ID.
+// The six metadata keys are views of one 8-byte union that starts as all ones (runtime_header.h:223-256) and receives
+// the writes of runtime.cc:365-452 in that order -- including the request_id = bid.x every task gets through the
+// always-true term at :380.  Two operators that share no tensor (the reference asserts) get one event from all
+// producer blocks to all consumer blocks.
 struct RefTask {
   int op_index;
   int bid[3];
-  long long trigger_event, dependent_event;
+  unsigned long long trigger_event, dependent_event;
 };
 struct RefEvent {
   int type, num_triggers, first_task, last_task;
 };
+static const unsigned long long REF_EVENT_INVALID = 0x7ffffffffffffffeull;
 
 int task_type_id(const std::string &n) {
   // runtime_header.h:91-188 task ids for the tasks this library lowers
@@ -891,155 +1037,290 @@ int task_type_id(const std::string &n) {
       {"moe_mul_sum_add_mi300", 173}, {"gang_moe_w13_linear_mi300", 174}, {"gang_moe_w2_linear_mi300", 175}, {"moe_silu_mul", 118},
       {"paged_attention", 116}, {"paged_attention_split_kv_mi300", 130}, {"paged_attention_split_kv_merge_mi300", 131},
       {"paged_attention_ck_fmha_merge_mi300", 131}, {"gang_attn_merge_mi300", 139}, {"splitk_reduce_mi300", 132},
-      {"silu_mul_linear_with_residual", 105}};
+      {"silu_mul_linear_with_residual", 105}, {"rmsnorm_linear", 102}, {"identity", 121}, {"argmax", 109}, {"attention", 103},
+      {"find_ngram_partial", 112}, {"find_ngram_global", 113}, {"target_verify_greedy", 114}};
   auto it = ids.find(n);
   return it == ids.end() ? 0 : it->second;
 }
 
-// partition of the tensor shared by producer and consumer along each of its dims
-void partition_of(const Task &t, int operand, int ndims, int part[4]) {
+// which param of a gang task is its tiles-per-XCD count (src/kernel/graph.cc:584-675,825-838); -1: not a gang task
+int gang_tiles_param(const std::string &n) {
+  if (n == "gang_linear_mi300" || n == "gang_linear_n_tiling_mi300" || n == "gang_linear_res_mi300" || n == "gang_linear_res_n_tiling_mi300" ||
+      n == "gang_linear_silu_mi300")
+    return 4;
+  if (n == "gang_linear_msplit_mi300" || n == "gang_linear_res_msplit_mi300") return 3;
+  if (n == "gang_rmsnorm_mi300") return 0;
+  if (n == "gang_attn_split_kv_mi300") return 7;
+  if (n == "gang_attn_merge_mi300") return 5;
+  if (n == "gang_moe_w13_linear_mi300" || n == "gang_moe_w2_linear_mi300") return 2;
+  if (n == "gang_splitk_linear_res_mi300") return -2;  // params[2] * params[3]
+  return -1;
+}
+
+// The 8-byte metadata union of a task (runtime_header.h:238-256), little endian: bytes 0-1 request_id / n_tile_start,
+// bytes 2-3 kv_idx / n_tile_count, bytes 0-3 expert_offset, bytes 4-7 merge_task_offset / _linear_reserved.
+unsigned long long ref_task_metadata(const Task &t, const int bid[3]) {
+  unsigned long long m = ~0ull;
+  auto set16 = [&](int at, unsigned v) { m = (m & ~(0xffffull << (8 * at))) | ((unsigned long long)(v & 0xffffu) << (8 * at)); };
+  auto set32 = [&](int at, unsigned v) { m = (m & ~(0xffffffffull << (8 * at))) | ((unsigned long long)v << (8 * at)); };
+  const int type = task_type_id(t.name);
+  set16(0, (unsigned)bid[0]);  // request_id: written for every task (runtime.cc:380 is a bare enumerator in an || chain)
+  if (type == 170 || type == 171 || type == 182) set32(0, (unsigned)((bid[1] << 16) | (bid[0] & 0xFFFF)));
+  const int gp = gang_tiles_param(t.name);
+  if (gp != -1) {
+    int tiles = 0;
+    if (gp == -2) tiles = t.params.size() > 3 ? t.params[2] * t.params[3] : 0;
+    else tiles = (int)t.params.size() > gp ? t.params[gp] : 0;
+    set16(2, (unsigned)tiles);
+    if (type == 183 || type == 184) {
+      set16(0, 0);
+      set32(4, (unsigned)bid[0]);
+    } else if (type == 138 || type == 139) {
+      set16(0, (unsigned)(bid[0] * tiles));
+    } else {
+      set16(0, 0);
+    }
+  }
+  if (type == 130 || type == 131 || type == 141) {
+    set16(2, (unsigned)bid[2]);
+    set32(4, (unsigned)bid[1]);
+  }
+  return m;
+}
+
+// partition of a tensor along each of its dims by one operand's grid mapping (later axes override earlier ones)
+void partition_of(const Task &t, int operand, int part[4]) {
   for (int d = 0; d < 4; d++) part[d] = 1;
   for (int a = 0; a < 3; a++) {
     const int d = t.maps[operand][a];
-    if (d >= 0 && d < ndims) part[d] = t.grid[a];
+    if (d >= 0 && d < 4) part[d] = t.grid[a];
   }
 }
 
 int build_task_graph_json(mk_graph *g) {
   std::vector<RefTask> tasks;
   std::vector<RefEvent> events;
-  tasks.push_back({-1, {0, 0, 0}, 0, 0});  // TERMINATE
-  tasks.push_back({-1, {0, 0, 0}, 0, 0});  // BEGIN_TASK_GRAPH
-  events.push_back({911 /*EVENT_TERMINATION*/, 0, 0, 0});
+  tasks.push_back({-1, {0, 0, 0}, REF_EVENT_INVALID, REF_EVENT_INVALID});  // TERMINATE
+  tasks.push_back({-1, {0, 0, 0}, 1, REF_EVENT_INVALID});                  // BEGIN_TASK_GRAPH triggers event 1
+  events.push_back({911 /*EVENT_TERMINATION*/, 1, 0, 0});
   events.push_back({903 /*EVENT_LAUNCH_DEPENDENT_TASKS*/, 1, 2, 0});
-  std::vector<std::pair<int, int>> op_range;  // [first, last) task per operator
+  std::vector<int> first_tasks;
+  std::map<std::array<int, 3>, int> pre_map, cur_map;  // bid -> task index, of the previous / current operator
   for (size_t oi = 0; oi < g->tasks.size(); oi++) {
-    const Task &t = g->tasks[oi];
-    const int first = (int)tasks.size();
-    for (int x = 0; x < t.grid[0]; x++)
-      for (int y = 0; y < t.grid[1]; y++)
-        for (int z = 0; z < t.grid[2]; z++) tasks.push_back({(int)oi, {x, y, z}, 0, 0});
-    op_range.push_back({first, (int)tasks.size()});
-  }
-  tasks[1].trigger_event = 1;
-  // events between consecutive operators
-  for (size_t oi = 0; oi + 1 < g->tasks.size(); oi++) {
-    const Task &p = g->tasks[oi], &c = g->tasks[oi + 1];
-    // the shared tensor: an operand of the consumer that the producer also lists
-    int po = -1, co = -1;
-    for (size_t a = 0; a < c.ops.size() && po < 0; a++)
-      for (size_t b = p.ops.size(); b-- > 0;)
-        if (p.ops[b] == c.ops[a] && c.ops[a] >= 0) {
-          po = (int)b;
-          co = (int)a;
-          break;
+    const Task &c = g->tasks[oi];
+    cur_map.clear();
+    if (oi == 0) {
+      for (int x = 0; x < c.grid[0]; x++)
+        for (int y = 0; y < c.grid[1]; y++)
+          for (int z = 0; z < c.grid[2]; z++) {
+            cur_map[{x, y, z}] = (int)tasks.size();
+            first_tasks.push_back((int)tasks.size());
+            tasks.push_back({(int)oi, {x, y, z}, REF_EVENT_INVALID, REF_EVENT_INVALID});
+          }
+      pre_map = cur_map;
+      continue;
+    }
+    const Task &p = g->tasks[oi - 1];
+    // the tensor that carries the dependency: the last (consumer input, producer output) pair naming the same tensor
+    const int c_in = (int)c.ops.size() - num_outputs(c), p_in = (int)p.ops.size() - num_outputs(p);
+    int co = -1, po = -1;
+    for (int a = 0; a < c_in; a++)
+      for (int b = p_in; b < (int)p.ops.size(); b++)
+        if (c.ops[a] >= 0 && c.ops[a] == p.ops[b]) {
+          co = a;
+          po = b;
         }
-    int ev_parts = 1;
-    int pp[4] = {1, 1, 1, 1}, cp[4] = {1, 1, 1, 1};
-    if (po >= 0) {
-      const int nd = g->tensors[p.ops[po]].ndims;
-      partition_of(p, po, nd, pp);
-      partition_of(c, co, nd, cp);
-      for (int d = 0; d < nd; d++) ev_parts *= std::gcd(pp[d], cp[d]);
+    int ev_dims[4] = {1, 1, 1, 1};
+    std::array<int, 3> in_map = {-1, -1, -1}, out_map = {-1, -1, -1};
+    if (co >= 0) {
+      int pp[4], cp[4];
+      in_map = c.maps[co];
+      out_map = p.maps[po];
+      partition_of(c, co, cp);
+      partition_of(p, po, pp);
+      for (int d = 0; d < 4; d++) ev_dims[d] = std::gcd(pp[d], cp[d]);
     }
-    const int np = op_range[oi].second - op_range[oi].first, nc = op_range[oi + 1].second - op_range[oi + 1].first;
-    if (np % ev_parts || nc % ev_parts) ev_parts = 1;
-    for (int e = 0; e < ev_parts; e++) {
-      const int ev = (int)events.size();
-      const int pf = op_range[oi].first + e * (np / ev_parts), cf = op_range[oi + 1].first + e * (nc / ev_parts);
-      events.push_back({900 /*EVENT_EMPTY: consumers carry dependent_event*/, np / ev_parts, cf, cf + nc / ev_parts});
-      for (int k = 0; k < np / ev_parts; k++) tasks[pf + k].trigger_event = ev;
-      for (int k = 0; k < nc / ev_parts; k++) tasks[cf + k].dependent_event = ev;
-    }
+    // depth-first over the tensor's dims: each combination of slices is one event
+    int idx[4];
+    for (idx[0] = 0; idx[0] < ev_dims[0]; idx[0]++)
+      for (idx[1] = 0; idx[1] < ev_dims[1]; idx[1]++)
+        for (idx[2] = 0; idx[2] < ev_dims[2]; idx[2]++)
+          for (idx[3] = 0; idx[3] < ev_dims[3]; idx[3]++) {
+            int clo[3] = {0, 0, 0}, chi[3] = {c.grid[0], c.grid[1], c.grid[2]}, plo[3] = {0, 0, 0}, phi[3] = {p.grid[0], p.grid[1], p.grid[2]};
+            for (int d = 0; d < 4; d++)
+              for (int a = 0; a < 3; a++) {
+                if (in_map[a] == d) {
+                  const int f = c.grid[a] / ev_dims[d];
+                  clo[a] = idx[d] * f;
+                  chi[a] = (idx[d] + 1) * f;
+                }
+                if (out_map[a] == d) {
+                  const int f = p.grid[a] / ev_dims[d];
+                  plo[a] = idx[d] * f;
+                  phi[a] = (idx[d] + 1) * f;
+                }
+              }
+            const int ev = (int)events.size();
+            RefEvent e = {900 /*EVENT_EMPTY: its tasks carry dependent_event*/, 0, (int)tasks.size(), 0};
+            for (int x = clo[0]; x < chi[0]; x++)
+              for (int y = clo[1]; y < chi[1]; y++)
+                for (int z = clo[2]; z < chi[2]; z++) {
+                  cur_map[{x, y, z}] = (int)tasks.size();
+                  tasks.push_back({(int)oi, {x, y, z}, REF_EVENT_INVALID, (unsigned long long)ev});
+                }
+            e.last_task = (int)tasks.size();
+            for (int x = plo[0]; x < phi[0]; x++)
+              for (int y = plo[1]; y < phi[1]; y++)
+                for (int z = plo[2]; z < phi[2]; z++) {
+                  auto it = pre_map.find({x, y, z});
+                  if (it == pre_map.end()) return fail(MK_EINVAL, "task graph: producer block (%d,%d,%d) of '%s' has no task", x, y, z, p.name.c_str());
+                  tasks[it->second].trigger_event = (unsigned long long)ev;
+                  e.num_triggers++;
+                }
+            events.push_back(e);
+          }
+    if ((int)cur_map.size() != c.grid[0] * c.grid[1] * c.grid[2])
+      return fail(MK_EINVAL, "task graph: the partitions of '%s' and '%s' over their shared tensor leave blocks of '%s' without an event", p.name.c_str(),
+                  c.name.c_str(), c.name.c_str());
+    pre_map = cur_map;
   }
-  // last operator triggers END_OF_TASK_GRAPH
+  // the last operator's tasks trigger END_OF_TASK_GRAPH
   const int end_ev = (int)events.size();
-  if (!g->tasks.empty()) {
-    const int lf = op_range.back().first, ll = op_range.back().second;
-    events.push_back({910 /*EVENT_END_OF_TASK_GRAPH*/, ll - lf, 0, 0});
-    for (int k = lf; k < ll; k++) tasks[k].trigger_event = end_ev;
-  }
+  for (auto &kv : pre_map)
+    if (tasks[kv.second].trigger_event == REF_EVENT_INVALID) tasks[kv.second].trigger_event = (unsigned long long)end_ev;
+  events.push_back({910 /*EVENT_END_OF_TASK_GRAPH*/, (int)pre_map.size(), 0, 0});
   events[1].last_task = (int)tasks.size();
   g->num_ref_tasks = (int)tasks.size();
   g->num_ref_events = (int)events.size();
-  // sanity check (reference: runtime.cc:614-674): simulate once; every task runs once, every event fires once
+  // sanity check (reference: runtime.cc:614-674): run the graph once from the first tasks; every task must run exactly
+  // once, every event between operators fire exactly once, and END_OF_TASK_GRAPH be reached
   {
-    std::vector<int> counter(events.size(), 0), fired(events.size(), 0), ran(tasks.size(), 0);
-    std::vector<int> ready;
-    ran[1] = 1;
-    fired[1] = 1;
-    for (int k = 2; k < (int)tasks.size(); k++)
-      if (tasks[k].dependent_event == 0) ready.push_back(k);
+    std::vector<int> left(events.size()), fired(events.size(), 0), ran(tasks.size(), 0);
+    for (size_t e = 0; e < events.size(); e++) left[e] = events[e].num_triggers;
+    std::vector<int> queue(first_tasks.begin(), first_tasks.end());
     size_t head = 0;
-    while (head < ready.size()) {
-      const int k = ready[head++];
+    while (head < queue.size()) {
+      const int k = queue[head++];
       if (ran[k]++) return fail(MK_EINVAL, "task graph sanity check: task %d scheduled twice", k);
-      const long long ev = tasks[k].trigger_event;
-      if (++counter[ev] == events[ev].num_triggers) {
-        if (fired[ev]++) return fail(MK_EINVAL, "task graph sanity check: event %lld fired twice", ev);
-        for (int c2 = events[ev].first_task; c2 < events[ev].last_task && events[ev].type == 900; c2++) ready.push_back(c2);
+      const unsigned long long ev = tasks[k].trigger_event;
+      if (ev == REF_EVENT_INVALID) continue;
+      if (left[ev] <= 0) return fail(MK_EINVAL, "task graph sanity check: event %llu triggered more often than it counts", ev);
+      if (--left[ev] == 0) {
+        if (fired[ev]++) return fail(MK_EINVAL, "task graph sanity check: event %llu fired twice", ev);
+        if (events[ev].type == 900)
+          for (int c2 = events[ev].first_task; c2 < events[ev].last_task; c2++) queue.push_back(c2);
       }
     }
     for (int k = 2; k < (int)tasks.size(); k++)
       if (ran[k] != 1) return fail(MK_EINVAL, "task graph sanity check: task %d ran %d times", k, ran[k]);
+    for (int e = 2; e < end_ev; e++)
+      if (fired[e] != 1) return fail(MK_EINVAL, "task graph sanity check: event %d fired %d times", e, fired[e]);
     if (!g->tasks.empty() && fired[end_ev] != 1) return fail(MK_EINVAL, "task graph sanity check: END_OF_TASK_GRAPH fired %d times", fired[end_ev]);
+  }
+  // variant ids: the reference registers one code variant per distinct instantiation of a task type (task_register.cc:
+  // same constants -> same variant); restated here as: tasks of one type with the same name, per-block operand shapes and
+  // params share a variant, numbered in order of first appearance
+  std::vector<int> variant(g->tasks.size(), 0);
+  {
+    std::map<int, std::vector<std::string>> seen;  // task type -> signatures
+    for (size_t oi = 0; oi < g->tasks.size(); oi++) {
+      const Task &t = g->tasks[oi];
+      std::string sig = t.name;
+      for (size_t a = 0; a < t.ops.size(); a++) {
+        sig += "|";
+        if (t.ops[a] < 0) continue;
+        const Tensor &tn = g->tensors[t.ops[a]];
+        int part[4];
+        partition_of(t, (int)a, part);
+        for (int d = 0; d < tn.ndims; d++) sig += fmt("%lld,", (long long)(tn.dims[d] / std::gcd((long long)tn.dims[d], (long long)part[d])));
+      }
+      for (int v : t.params) sig += fmt(";%d", v);
+      auto &lst = seen[task_type_id(t.name)];
+      size_t k = 0;
+      while (k < lst.size() && lst[k] != sig) k++;
+      if (k == lst.size()) lst.push_back(sig);
+      variant[oi] = (int)k;
+    }
   }
   // JSON
   std::string &j = g->json;
   j.clear();
   j += "{\n \"all_tasks\": [\n";
-  for (size_t k = 0; k < tasks.size(); k++) {
-    const RefTask &rt = tasks[k];
-    int type = k == 0 ? 0 /*TASK_TERMINATE*/ : (k == 1 ? 10 /*TASK_BEGIN_TASK_GRAPH*/ : task_type_id(g->tasks[rt.op_index].name));
-    j += fmt("  {\"task_type\": %d, \"variant_id\": 0, \"inputs\": [", type);
-    std::string outs;
-    if (rt.op_index >= 0) {
-      const Task &t = g->tasks[rt.op_index];
-      // operands: inputs first, outputs last; count outputs by task type
-      int n_out = 1;
-      if (t.name == "argmax_partial") n_out = 2;
-      if (t.name == "gang_attn_split_kv_mi300") n_out = 3;
-      if (t.name == "paged_attention_ck_fmha_split_kv_mi300" || t.name == "paged_attention_split_kv_mi300") n_out = 2;
-      const int n_in = (int)t.ops.size() - n_out;
-      bool first_in = true, first_out = true;
-      for (size_t a = 0; a < t.ops.size(); a++) {
-        if (t.ops[a] < 0) continue;  // optional operand that is absent
-        const Tensor &tn = g->tensors[t.ops[a]];
-        long long off = 0;
-        long long dims[4];
-        for (int d = 0; d < tn.ndims; d++) dims[d] = tn.dims[d];
-        for (int ax = 0; ax < 3; ax++) {
-          const int d = t.maps[a][ax];
-          if (d >= 0 && d < tn.ndims && t.grid[ax] > 0) {
-            const long long per = tn.dims[d] / std::gcd((long long)tn.dims[d], (long long)t.grid[ax]);
-            dims[d] = per;
-            off += per * rt.bid[ax] * tn.strides[d] * (long long)dtype_size(tn.dtype);
-          }
-        }
-        std::string e = fmt("{\"base_ptr\": \"%s\", \"offset\": %lld, \"data_type\": %d, \"dims\": [", tn.name.c_str(), off, tn.dtype);
-        for (int d = 0; d < tn.ndims; d++) e += fmt(d ? ", %lld" : "%lld", dims[d]);
-        e += "], \"strides\": [";
-        for (int d = 0; d < tn.ndims; d++) e += fmt(d ? ", %lld" : "%lld", (long long)tn.strides[d]);
-        e += "]}";
-        if ((int)a < n_in) {
-          j += (first_in ? "" : ", ") + e;
-          first_in = false;
-        } else {
-          outs += (first_out ? "" : ", ") + e;
-          first_out = false;
-        }
+  // one operand of one block: the slice the block's grid indices select (runtime.cc:1215-1414).  A shuffled (fused) tensor
+  // is resolved to the source tensor and row the slice starts in (:1229-1283).
+  auto operand_json = [&](const Task &t, size_t a, const int bid[3]) -> std::string {
+    if (t.ops[a] < 0) return "{\"base_ptr\": \"nullptr\", \"offset\": 0, \"data_type\": 999, \"dims\": [], \"strides\": []}";
+    const Tensor &tn = g->tensors[t.ops[a]];
+    int part[4];
+    partition_of(t, (int)a, part);
+    long long dims[4];
+    for (int d = 0; d < tn.ndims; d++) dims[d] = tn.dims[d] / std::gcd((long long)tn.dims[d], (long long)part[d]);
+    const Tensor *base = &tn;
+    long long off = 0;
+    if (tn.kind == T_SHUFFLED) {
+      const int groups = tn.interleave ? tn.num_groups : 1;
+      std::vector<long long> gs;
+      long long group_rows = 0;
+      for (int sid : tn.sources) {
+        gs.push_back(g->tensors[sid].dims[0] / groups);
+        group_rows += gs.back();
+      }
+      long long row = 0;
+      for (int ax = 0; ax < 3; ax++)
+        if (t.maps[a][ax] == 0) row = tn.dims[0] / t.grid[ax] * bid[ax];
+      long long in_group = row % group_rows;
+      size_t si = 0;
+      while (si + 1 < gs.size() && in_group >= gs[si]) in_group -= gs[si++];
+      base = &g->tensors[tn.sources[si]];
+      const long long sub_row = row / group_rows * gs[si] + in_group;
+      for (int ax = 0; ax < 3; ax++) {
+        const int d = t.maps[a][ax];
+        if (d > 0 && d < base->ndims) off += base->dims[d] / t.grid[ax] * bid[ax] * base->strides[d];
+        else if (d == 0) off += sub_row * base->strides[0];
+      }
+    } else {
+      for (int ax = 0; ax < 3; ax++) {
+        const int d = t.maps[a][ax];
+        if (d >= 0 && d < tn.ndims) off += tn.dims[d] / t.grid[ax] * bid[ax] * tn.strides[d];
       }
     }
+    std::string e = fmt("{\"base_ptr\": \"%s\", \"offset\": %lld, \"data_type\": %d, \"dims\": [", base->name.c_str(), off * (long long)dtype_size(base->dtype), tn.dtype);
+    for (int d = 0; d < tn.ndims; d++) e += fmt(d ? ", %lld" : "%lld", dims[d]);
+    e += "], \"strides\": [";
+    for (int d = 0; d < tn.ndims; d++) e += fmt(d ? ", %lld" : "%lld", (long long)base->strides[d]);
+    e += "]}";
+    return e;
+  };
+  for (size_t k = 0; k < tasks.size(); k++) {
+    const RefTask &rt = tasks[k];
+    const int type = k == 0 ? 0 /*TASK_TERMINATE*/ : (k == 1 ? 10 /*TASK_BEGIN_TASK_GRAPH*/ : task_type_id(g->tasks[rt.op_index].name));
+    j += fmt("  {\"task_type\": %d, \"variant_id\": %d, \"inputs\": [", type, rt.op_index >= 0 ? variant[rt.op_index] : 0);
+    std::string outs;
+    unsigned long long meta = ~0ull;
+    if (rt.op_index >= 0) {
+      const Task &t = g->tasks[rt.op_index];
+      const int n_in = (int)t.ops.size() - num_outputs(t);
+      for (size_t a = 0; a < t.ops.size(); a++) {
+        const std::string e = operand_json(t, a, rt.bid);
+        if ((int)a < n_in) j += ((int)a ? ", " : "") + e;
+        else outs += ((int)a > n_in ? ", " : "") + e;
+      }
+      meta = ref_task_metadata(t, rt.bid);
+    }
     j += "], \"outputs\": [" + outs + "], ";
-    j += fmt("\"trigger_event\": %lld, \"dependent_event\": %lld, \"request_id\": %d, \"expert_offset\": 0, \"kv_idx\": %d, "
-             "\"merge_task_offset\": 0, \"n_tile_start\": 0, \"n_tile_count\": 0}%s\n",
-             rt.trigger_event, rt.dependent_event, rt.bid[0], rt.bid[1], k + 1 < tasks.size() ? "," : "");
+    j += fmt("\"trigger_event\": %llu, \"dependent_event\": %llu, \"request_id\": %d, \"expert_offset\": %d, \"kv_idx\": %d, "
+             "\"merge_task_offset\": %d, \"n_tile_start\": %d, \"n_tile_count\": %d}%s\n",
+             rt.trigger_event, rt.dependent_event, k < 2 ? -1 : (int)(int16_t)(meta & 0xffff), k < 2 ? -1 : (int)(int32_t)(meta & 0xffffffffu),
+             k < 2 ? -1 : (int)((meta >> 16) & 0xffff), k < 2 ? -1 : (int)(int32_t)(meta >> 32), k < 2 ? 0 : (int)(meta & 0xffff),
+             k < 2 ? 0 : (int)((meta >> 16) & 0xffff), k + 1 < tasks.size() ? "," : "");
   }
   j += " ],\n \"all_events\": [\n";
   for (size_t e = 0; e < events.size(); e++)
     j += fmt("  {\"event_type\": %d, \"num_triggers\": %d, \"first_task_id\": %d, \"last_task_id\": %d}%s\n", events[e].type, events[e].num_triggers,
              events[e].first_task, events[e].last_task, e + 1 < events.size() ? "," : "");
-  j += " ],\n \"first_tasks\": [1]\n}\n";
+  j += " ],\n \"first_tasks\": [";
+  for (size_t k = 0; k < first_tasks.size(); k++) j += fmt(k ? ", %d" : "%d", first_tasks[k]);
+  j += "]\n}\n";
   return MK_OK;
 }
 
@@ -1086,7 +1367,18 @@ int do_wait(mk_graph *g, hipStream_t stream, int *finished_out) {
   MkSched sc;
   HIP_TRY(hipMemcpy(&sc, g->d_sched, sizeof(MkSched), hipMemcpyDeviceToHost));
   if (finished_out) *finished_out = sc.finished;
-  if (hs.abort_flag) return fail(MK_EABORT, "kernel watchdog fired (barrier epoch %u): a workgroup waited longer than the spin limit", hs.abort_where);
+  if (hs.abort_flag) {
+    // workgroups that unwound mid-stage may have left the split-K and split-KV arrival counters mid-count (their last
+    // arriver resets them); the next launch on this handle must not inherit that
+    HIP_TRY(hipMemset(g->h_rt.attn_cnt, 0, sizeof(unsigned) * g->attn_cnt_n));
+    HIP_TRY(hipMemset(g->h_rt.splitk_cnt, 0, sizeof(unsigned) * 32 * (size_t)g->G));
+    return fail(MK_EABORT, "kernel watchdog fired (barrier epoch %u): a workgroup waited longer than the spin limit", hs.abort_where);
+  }
+  if (sc.bad_batch) {
+    static const char *why[] = {"", "rows outside [0, max_num_batched_tokens), overlapping, or with gaps", "more rows for one request than max_tokens_per_request",
+                                "a sequence shorter than its new rows, longer than max_seq_length, or without pages"};
+    return fail(MK_EINVAL, "the batch described in qo_indptr / paged_kv_* was rejected and nothing was run: %s", why[sc.bad_batch > 0 && sc.bad_batch <= 3 ? sc.bad_batch : 1]);
+  }
   return MK_OK;
 }
 
@@ -1107,11 +1399,10 @@ constexpr size_t SS_CLEARED_END = SS_ATTN_CNT + align256((size_t)MK_STATIC_MAX_I
 constexpr size_t SS_ARGMAX_PV = SS_CLEARED_END;
 constexpr size_t SS_ARGMAX_PI = SS_ARGMAX_PV + align256((size_t)MK_MAX_TOKENS * MK_STATIC_MAX_WG * sizeof(float));
 constexpr size_t SS_ATTN_PART = SS_ARGMAX_PI + align256((size_t)MK_MAX_TOKENS * MK_STATIC_MAX_WG * sizeof(int));
-// q-head partials of the attention stages: units of one kv head (up to 8 q heads each), or -- iterations of many tokens --
-// one unit per workgroup over all heads of a token (up to 32 q heads)
-constexpr size_t MK_STATIC_ATTN_HEADS = std::max<size_t>((size_t)(MK_STATIC_MAX_ITEMS + MK_ATTN_MAX_CHUNKS) * MK_STATIC_MAX_QPK, (size_t)(MK_STATIC_MAX_WG + MK_ATTN_MAX_CHUNKS) * 32);
+// q-head partials of the attention stages: at most max(workgroups, (token, kv head) pairs) work units of up to 8 q heads each
+constexpr size_t MK_STATIC_ATTN_HEADS = (size_t)std::max(MK_STATIC_MAX_ITEMS, MK_STATIC_MAX_WG) * MK_STATIC_MAX_QPK;
 constexpr size_t SS_SPLITK_PART = SS_ATTN_PART + align256(MK_STATIC_ATTN_HEADS * MK_ATTN_PSTRIDE * sizeof(float));
-constexpr size_t MK_STATIC_SCRATCH_BYTES = SS_SPLITK_PART + (size_t)MK_STATIC_MAX_WG * 4 * 4 * 4 * 64 * 16;  // about 22.8 MB
+constexpr size_t MK_STATIC_SCRATCH_BYTES = SS_SPLITK_PART + (size_t)MK_STATIC_MAX_WG * 4 * 4 * 4 * 64 * 16;  // about 19.6 MB
 
 static __device__ __align__(256) unsigned char scratch[MK_STATIC_SCRATCH_BYTES];
 
@@ -1158,18 +1449,22 @@ int mk_graph_create(const mk_config *cfg, mk_graph **out) {
   if ((int64_t)cfg->max_num_pages * cfg->page_size < cfg->max_seq_length)
     return fail(MK_EINVAL, "max_num_pages*page_size=%lld cannot hold one sequence of max_seq_length=%d", (long long)cfg->max_num_pages * cfg->page_size,
                 cfg->max_seq_length);
-  {
+  // The next two limits protect state only the on-GPU schedulers keep (MK_MODE_OFFLINE, MK_MODE_ONLINE): their page ring
+  // and the LDS snapshot of the page table.  In MK_MODE_ONLINE_NOTOKEN / MK_MODE_ONEPASS the host owns the page table;
+  // max_num_pages is then the serving engine's block count, which may be oversubscribed and much larger.
+  const bool gpu_pages = cfg->mode == MK_MODE_OFFLINE || cfg->mode == MK_MODE_ONLINE;
+  if (gpu_pages) {
     // Every slot can grow to max_seq_length, and the page ring (like the reference's) hands out pages without checking
     // that any are free: with fewer pages than that a page would be given to two requests.
     const int64_t per_req = ((int64_t)cfg->max_seq_length + cfg->page_size - 1) / cfg->page_size;
     if (per_req * cfg->max_num_batched_requests > cfg->max_num_pages)
       return fail(MK_EINVAL, "max_num_pages=%d cannot back %d concurrent requests of up to %lld pages each (max_seq_length=%d, page_size=%d)",
                   cfg->max_num_pages, cfg->max_num_batched_requests, (long long)per_req, cfg->max_seq_length, cfg->page_size);
+    if (cfg->max_num_pages > (MK_LDS_BYTES / 8)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 8);
   }
   if (((int64_t)cfg->max_seq_length + cfg->page_size - 1) / cfg->page_size > MK_ATTN_MAX_REQ_PAGES)
     return fail(MK_EINVAL, "max_seq_length=%d over page_size=%d is more than %d pages per request (the attention stage keeps a request's page list in LDS)",
                 cfg->max_seq_length, cfg->page_size, MK_ATTN_MAX_REQ_PAGES);
-  if (cfg->max_num_pages > (MK_LDS_BYTES / 8)) return fail(MK_EINVAL, "max_num_pages=%d exceeds the scheduler's LDS snapshot (%d)", cfg->max_num_pages, MK_LDS_BYTES / 8);
   if (cfg->device < 0) {
     mk_graph *g = new mk_graph();
     g->cfg = *cfg;
@@ -1327,7 +1622,7 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
   for (int i = 0; i < n_operands; i++) {
     // id -1 = optional operand that is absent: only the q/k-norm weights and the cos/sin tables of the attention tasks
     const bool optional = (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300" || t.name == "paged_attention" ||
-                           t.name == "paged_attention_split_kv_mi300") && i >= 3 && i <= 6;
+                           t.name == "paged_attention_split_kv_mi300" || t.name == "attention") && i >= 3 && i <= 6;
     if (tensor_ids[i] >= (int)g->tensors.size() || tensor_ids[i] < (optional ? -1 : 0))
       return fail(MK_EINVAL, "task '%s': bad tensor id %d for operand %d", task_name, tensor_ids[i], i);
     t.ops.push_back(tensor_ids[i]);
@@ -1344,7 +1639,7 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
                                 "paged_attention_ck_fmha_split_kv_mi300", "argmax_partial", "argmax_reduce", "moe_topk_softmax_mi300", "moe_w13_linear_mi300",
                                 "moe_w2_linear_mi300", "gang_moe_w13_linear_mi300", "gang_moe_w2_linear_mi300", "moe_silu_mul", "moe_mul_sum_add_mi300",
                                 "paged_attention", "paged_attention_split_kv_mi300", "paged_attention_split_kv_merge_mi300",
-                                "paged_attention_ck_fmha_merge_mi300", "gang_attn_merge_mi300", "splitk_reduce_mi300", "silu_mul_linear_with_residual"};
+                                "paged_attention_ck_fmha_merge_mi300", "gang_attn_merge_mi300", "splitk_reduce_mi300", "silu_mul_linear_with_residual", "rmsnorm_linear", "identity", "argmax", "attention"};
   bool ok = linear_kind(t.name, &a, &b, &c);
   for (auto k : known) ok = ok || t.name == k;
   if (!ok) return fail(MK_EUNSUPPORTED, "Unsupported task name: %s", task_name);
@@ -1470,12 +1765,11 @@ int mk_compile(mk_graph *g) {
   rt.attn_part = nullptr;
   for (auto &s : g->stages)
     if (s.op == MK_OP_ATTN) {
-      // units of one kv head: max(G, tokens * kv heads) of q/kv heads each; units of all heads: G of all q heads each
-      const size_t units = (size_t)std::max(g->G, rt.max_tokens * s.num_kv_heads) + MK_ATTN_MAX_CHUNKS;
+      // a work unit is (token, kv head, chunk) with chunks = clamp(G / (tokens * kv heads), 1, MK_ATTN_MAX_CHUNKS): never
+      // more than max(G, tokens * kv heads) units, each holding q/kv head partials
+      const size_t units = (size_t)std::max(g->G, rt.max_tokens * s.num_kv_heads);
       const int qpk = s.num_q_heads / s.num_kv_heads;
-      const size_t heads = std::max(units * qpk, (size_t)(g->G + MK_ATTN_MAX_CHUNKS) * s.num_q_heads);
-      rt.attn_part_cap = rt.attn_part_cap ? std::min<int>(rt.attn_part_cap, (int)heads) : (int)heads;
-      if ((rc = dev_alloc(g, &p, heads * MK_ATTN_PSTRIDE * sizeof(float), false))) return rc;
+      if ((rc = dev_alloc(g, &p, units * qpk * MK_ATTN_PSTRIDE * sizeof(float), false))) return rc;
       s.aux0 = p;
       s.aux1 = rt.attn_cnt + g->attn_cnt_n / 2;
     }
@@ -1557,7 +1851,6 @@ int mk_enqueue_steps_static(mk_graph *g, void *stream, int max_iterations) {
   rt.argmax_pv = (float *)(base + SS_ARGMAX_PV);
   rt.argmax_pi = (int *)(base + SS_ARGMAX_PI);
   rt.attn_part = (float *)(base + SS_ATTN_PART);
-  rt.attn_part_cap = (int)MK_STATIC_ATTN_HEADS;
   rt.splitk_part = base + SS_SPLITK_PART;
   rt.stage_prof = nullptr;  // per-stage timing is library-allocated scratch too: not recorded by this entry point
   rt.timing = nullptr;
@@ -1609,6 +1902,7 @@ int mk_run_once(mk_graph *g, void *stream, int num_tokens, const int32_t *tok_sl
   MkSched sc;
   HIP_TRY(hipMemcpy(&sc, g->d_sched, sizeof(sc), hipMemcpyDeviceToHost));
   sc.num_tokens = num_tokens;
+  sc.bad_batch = 0;
   HIP_TRY(hipMemcpy(g->d_sched, &sc, sizeof(sc), hipMemcpyHostToDevice));
   int rc = do_launch(g, s, 1, MK_SCHED_HOST_ARRAYS);
   if (rc) return rc;

@@ -601,21 +601,45 @@ __device__ __attribute__((noinline)) int mk_prepare_next_batch_wave(const MkRunt
 // on the device (no host round trip, so a serving loop can enqueue launches back to back).  Runs on one thread.
 __device__ __attribute__((noinline)) int mk_batch_from_meta(const MkRuntime &rt) {
   const int R = rt.max_requests, B = rt.max_tokens;
-  int ntok = 0;
-  for (int i = 0; i < R; i++) {
+  // A batch the stages cannot run as described is not run at all: truncating a request's rows would leave the rest with
+  // the slot / position an earlier launch gave them, and they would append K/V rows to some other request's cache.
+  // bad: 1 = rows outside [0, max tokens), overlapping, or with gaps; 2 = more rows for one request than
+  // max_tokens_per_request; 3 = a sequence shorter than its new rows, longer than max_seq_length, or without pages.
+  int ntok = 0, bad = 0;
+  unsigned long long covered = 0ull;
+  for (int i = 0; i < R && !bad; i++) {
     const int q0 = rt.qo_indptr[i], n = rt.qo_indptr[i + 1] - q0;
-    if (n <= 0 || q0 < 0 || q0 + n > B) continue;
+    if (n <= 0) continue;  // an unused slot (hosts that fill only the first entries leave zeros behind them)
+    if (q0 < 0 || q0 + n > B) {
+      bad = 1;
+      break;
+    }
+    if (n > rt.max_new_per_req) {
+      bad = 2;
+      break;
+    }
+    const unsigned long long rows = (n >= 64 ? ~0ull : ((1ull << n) - 1ull)) << q0;
+    if (covered & rows) {
+      bad = 1;
+      break;
+    }
+    covered |= rows;
     const int pages = rt.kv_indptr[i + 1] - rt.kv_indptr[i];
     const int len = (pages - 1) * rt.page_size + rt.kv_last_page_len[i];
-    int nn = n > rt.max_new_per_req ? rt.max_new_per_req : n;  // more rows per request than the attention stage holds are not run
-    if (len - nn < 0 || len > rt.max_seq) continue;
-    for (int j = 0; j < nn; j++) {
+    if (pages < 1 || len < n || len > rt.max_seq) {
+      bad = 3;
+      break;
+    }
+    for (int j = 0; j < n; j++) {
       rt.tok_slot[q0 + j] = i;
       rt.tok_pos[q0 + j] = len - n + j;
       rt.tok_first[q0 + j] = q0;
     }
-    if (q0 + nn > ntok) ntok = q0 + nn;
+    if (q0 + n > ntok) ntok = q0 + n;
   }
+  if (!bad && covered != (ntok >= 64 ? ~0ull : ((1ull << ntok) - 1ull))) bad = 1;
+  if (bad) ntok = 0;
+  rt.sched->bad_batch = bad;
   rt.sched->num_tokens = ntok;
   return ntok;
 }
@@ -2210,6 +2234,16 @@ __device__ __forceinline__ void stage_silu_mul(CStage &st, Ctx &c, int M) {
     const uint16_t *row = in + (size_t)t * st.ld_in + (size_t)g * 2 * half;
     out[(size_t)t * st.ld_out + j] = (uint16_t)f2bf(silu_mul(bf2f(ldc_u16(row + jj)), bf2f(ldc_u16(row + half + jj))));
   }
+}
+
+// Row copy.  Reference task: identity_task_impl (tasks/ampere/identity.cuh:24-37).
+__device__ __forceinline__ void stage_copy(CStage &st, Ctx &c, int M) {
+  barrier_wait(c);
+  const uint16_t *in = (const uint16_t *)st.in;
+  uint16_t *out = (uint16_t *)st.out;
+  const long long total = (long long)M * st.n;
+  for (long long i = (long long)c.vid * MK_THREADS + threadIdx.x; i < total; i += (long long)c.G * MK_THREADS) stc_u16(out + i, ldc_u16(in + i));
+  c.wrote_through = true;
 }
 
 // ----------------------------------------------------------------------------- mixture of experts
@@ -3842,6 +3876,7 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
           }
           break;
         case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
+        case MK_OP_COPY: stage_copy(st, c, M); break;
         case MK_OP_ATTN:
           if constexpr (MAXM == 1) {
             if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4, false>(st, c, rt, M, smem);

@@ -46,6 +46,7 @@ enum MkOp {
   MK_OP_MOE_TOPK = 8,     // router softmax -> top-k -> renormalise, one wavefront per token
   MK_OP_MOE_LINEAR = 9,   // per-expert linear over the active experts (W13 with optional SwiGLU, W2)
   MK_OP_MOE_COMBINE = 10, // out = res + sum_k w[t,k] * x[t,k,:]
+  MK_OP_COPY = 11,        // out[t, :] = in[t, :], n 16-bit units per token row
 };
 
 enum MkStageFlags {
@@ -156,7 +157,9 @@ enum MkSchedMode {
 // Scheduler state that persists across launches (continuous batching, page ring).
 struct MkSched {
   int page_queue_head, page_queue_tail, next_request_id, num_tokens;
-  int num_reqs, finished, online_started, pad1;
+  int num_reqs, finished, online_started;
+  int bad_batch;          // host-described batch (MK_SCHED_FROM_META) that was rejected instead of run: 0 = fine, else the reason
+
   long long iterations;   // decode iterations executed so far (all launches)
   long long pad2;
 };
@@ -191,8 +194,6 @@ struct MkRuntime {
   float *argmax_pv;     // non-null: the sampling stages' per-workgroup partials live here ([tokens][workgroups] values / indices)
   int *argmax_pi;       // instead of in the buffers their descriptors name
   unsigned *attn_cnt;   // [max_tokens * num_kv_heads][32]: one 128-byte line per counter
-  int attn_part_cap;    // q-head partials each attention stage's split-KV workspace (or the shared one) holds
-  int pad_apc;
   void *splitk_part;    // [workgroups][4 wavefronts][4 weight tiles][4 token tiles][64 lanes] f32x4: K-slice partials of the split-K linear
   unsigned *splitk_cnt; // [workgroups][32]: arrival counter per split-K group (one 128-byte line each)
   long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end

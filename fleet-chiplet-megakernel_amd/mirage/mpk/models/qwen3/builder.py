@@ -197,6 +197,7 @@ class Qwen3Builder(GraphBuilder):
                                     grid_dim=(H // 128, 1, 1), block_dim=(256, 1, 1))
             self.x = self.attn_proj_out
             w_norm2 = self._attach(state_dict[f"{prefix}post_attention_layernorm.weight"], f"layer_{i}_post_attn_layernorm")
+            gate_rows = None  # a shuffled view knows its own groups; a weight the caller interleaved needs them spelt out
             if f"{prefix}mlp.gate_proj.weight" in state_dict:
                 rmsnorm_num_tasks = grid_for_rmsnorm_linear_layer(2 * state_dict[f"{prefix}mlp.gate_proj.weight"].shape[0])
                 w_gate = self._attach(state_dict[f"{prefix}mlp.gate_proj.weight"], f"layer_{i}_gate_proj")
@@ -205,13 +206,14 @@ class Qwen3Builder(GraphBuilder):
             elif f"{prefix}mlp.gate_up_proj.weight" in state_dict:  # already interleaved in rmsnorm_num_tasks / 2 groups by the caller
                 rmsnorm_num_tasks = grid_for_rmsnorm_linear_layer(state_dict[f"{prefix}mlp.gate_up_proj.weight"].shape[0])
                 w_gatedup = self._attach(state_dict[f"{prefix}mlp.gate_up_proj.weight"], f"layer_{i}_gatedup_proj")
+                gate_rows = state_dict[f"{prefix}mlp.gate_up_proj.weight"].shape[0] // rmsnorm_num_tasks
             else:
                 raise ValueError(f"No gate or up projection weight found for layer {i}")
             mpk.rmsnorm_layer(input=self.x, weight=w_norm2, output=self.rmsnorm_out, grid_dim=(B, 1, 1), block_dim=(128, 1, 1))
             mpk.linear_layer(input=self.rmsnorm_out, weight=w_gatedup, output=self.mlp_mid, grid_dim=(rmsnorm_num_tasks, 1, 1), block_dim=(128, 1, 1))
             w_down = self._attach(state_dict[f"{prefix}mlp.down_proj.weight"], f"layer_{i}_down_proj")
             mpk.silu_mul_linear_with_residual_layer(input=self.mlp_mid, weight=w_down, residual=self.x, output=self.mlp_out,
-                                                    grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1))
+                                                    grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1), gate_rows_per_group=gate_rows)
             self.x = self.mlp_out
 
     def build_from_dict(self, state_dict: dict, with_lm_head: bool):

@@ -16,7 +16,8 @@ import torch
 from .. import _capi
 from ..kernel import DTensor, KNGraph, bfloat16, convert_torch_type_to_dtype
 
-valid_persistent_kernel_modes = ["offline", "online", "online_notoken", "onepass", "multi_turn"]
+# the reference spells the multi-turn mode "online_multi_turn" (persistent_kernel.py:132); "multi_turn" is kept as an alias
+valid_persistent_kernel_modes = ["offline", "online", "online_notoken", "onepass", "online_multi_turn", "multi_turn"]
 
 _META_ORDER = ["step", "tokens", "input_tokens", "output_tokens", "num_new_tokens", "prompt_lengths",
                "qo_indptr_buffer", "paged_kv_indptr_buffer", "paged_kv_indices_buffer", "paged_kv_last_page_len_buffer"]
@@ -285,18 +286,20 @@ class PersistentKernel:
                    [(workspace, (1, -1, -1), 1), (residual, (1, -1, -1), 1), (output, (1, -1, -1), -1)], [k_splits])
 
     def silu_mul_linear_with_residual_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, grid_dim: tuple,
-                                            block_dim: tuple):
+                                            block_dim: tuple, gate_rows_per_group: int = None):
         """persistent_kernel.py:2174: output = bf16(silu_mul(input) @ weight^T + residual) with input = the gate/up linear's
-        [tokens, 2 * intermediate] result.  The activation is folded into the gate/up linear that produced `input` (whose
-        weight view says which columns are gate and which are up) and the product becomes a linear-with-residual stage; an
-        `input` of unknown origin is read as [gate | up] halves, the layout the reference task kernel reads
-        (tasks/ampere/silu_mul_linear.cuh:78-80)."""
+        [tokens, 2 * intermediate] result.  Which columns are gate and which are up: the shuffled weight view of the linear
+        that produced `input` says so; a caller that interleaved a physical weight itself passes `gate_rows_per_group`
+        (not a reference argument: groups of [gate x n ; up x n]); otherwise `input` is read as [gate | up] halves, the
+        layout the reference task kernel reads (tasks/mi300/silu_mul_linear_mi300.cuh:40-42).  The activation is folded into
+        the producing linear's epilogue when nothing else reads `input`."""
         assert input.num_dims == 2  # (batch_size, 2*intermediate_size)
         assert weight.num_dims == 2  # (hidden_size, intermediate_size)
         assert residual.num_dims == 2  # (batch_size, hidden_size)
         assert input.dim(1) == 2 * weight.dim(1)
         self._task("silu_mul_linear_with_residual", grid_dim, block_dim,
-                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), 1), (output, (1, -1, -1), 1)])
+                   [(input, _REPL, 1), (weight, (0, -1, -1), 1), (residual, (1, -1, -1), 1), (output, (1, -1, -1), 1)],
+                   [int(gate_rows_per_group)] if gate_rows_per_group else [])
 
     # ------------------------------------------------------------------ mixture-of-experts layers
     def moe_topk_softmax_routing_layer(self, input: DTensor, output: tuple, grid_dim: tuple, block_dim: tuple):
@@ -556,7 +559,74 @@ class PersistentKernel:
                    [(input_value, (1, 0, -1), -1), (input_index, (1, 0, -1), -1), (output, (0, 1, -1), -1)],
                    [getattr(self, "argmax_partial_output_size", 0)])
 
+    def rmsnorm_linear_layer(self, input: DTensor, weight_norm: DTensor, weight_linear: DTensor, output: DTensor, grid_dim: tuple,
+                             block_dim: tuple):
+        """persistent_kernel.py:566: output = linear(rmsnorm(input, weight_norm), weight_linear) as one task.  Lowered as
+        the norm + linear pair (a single-token iteration computes the norm inside the linear stage)."""
+        assert input.num_dims == 2
+        assert weight_linear.num_dims == 2
+        assert output.num_dims == 2
+        self._task("rmsnorm_linear", grid_dim, block_dim,
+                   [(input, _REPL, 1), (weight_norm, _REPL, 0), (weight_linear, (0, -1, -1), 1), (output, (1, -1, -1), -1)])
+
+    def attention_layer(self, input: DTensor, k_cache: DTensor, v_cache: DTensor, q_norm: DTensor, k_norm: DTensor, cos_pos_embed: DTensor,
+                        sin_pos_embed: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:587: the form whose caches are [requests, seq_len, kv_heads, head_dim], one contiguous
+        range of rows per request -- a paged cache with pages of max_seq_length rows, so the graph must be built with
+        page_size == seq_len and at least one page per request.  Same stage as every other attention builder."""
+        assert input.num_dims == 2  # (batch_size, fused_outdim)
+        assert output.num_dims == 2  # (batch_size, hidden_size)
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4  # (batch_size, seq_len, kv_heads, head_dim)
+        head_dim, num_kv_heads = k_cache.dim(3), k_cache.dim(2)
+        num_q_heads = output.dim(1) // head_dim
+        qk_norm, rotary_embed = self._attn_flags(q_norm, k_norm, cos_pos_embed, sin_pos_embed, head_dim)
+        assert k_cache.dim(1) == self.page_size, "attention_layer: one page per request (page_size == the cache's seq_len)"
+        self._task("attention", grid_dim, block_dim,
+                   [(input, (0, 1, -1), -1), (k_cache, (0, 2, -1), 1), (v_cache, (0, 2, -1), 1), (q_norm, _REPL, -1), (k_norm, _REPL, -1),
+                    (cos_pos_embed, _REPL, -1), (sin_pos_embed, _REPL, -1), (output, (0, 1, -1), -1)],
+                   [num_q_heads, num_kv_heads, qk_norm, rotary_embed])
+
+    def identity_layer(self, input: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple, dependent_tensor: DTensor = None):
+        """persistent_kernel.py:2153: output = input (the rows of the running iteration)."""
+        last_dim = 0
+        assert input.num_dims == output.num_dims
+        for i in range(input.num_dims):
+            assert input.dim(i) == output.dim(i)
+            last_dim = i
+        assert last_dim == 1 or last_dim == 2
+        self._task("identity", grid_dim, block_dim, [(input, (last_dim, -1, -1), 1), (output, (last_dim, -1, -1), 1)])
+
+    def argmax_layer(self, input: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2195: greedy token of every row in one task (lowest index on ties)."""
+        assert input.num_dims == 2  # (batch_size, vocab_size)
+        assert output.num_dims == 2  # (batch_size, 1)
+        self._task("argmax", grid_dim, block_dim, [(input, _REPL, -1), (output, _REPL, -1)])
+
+    def linear_m_parallel_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:1953: the plain linear task with grid (N tiles, M tiles, 1)."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and output.num_dims == 2
+        self._task("linear", grid_dim, block_dim, [(input, (-1, 0, -1), 1), (weight, (0, -1, -1), 1), (output, (1, 0, -1), -1)])
+
+    def linear_with_residual_m_parallel_layer(self, input: DTensor, weight: DTensor, residual: DTensor, output: DTensor, grid_dim: tuple,
+                                              block_dim: tuple):
+        """persistent_kernel.py:1977."""
+        assert input.num_dims == 2 and weight.num_dims == 2 and residual.num_dims == 2 and output.num_dims == 2
+        self._task("linear_with_residual", grid_dim, block_dim,
+                   [(input, (-1, 0, -1), 1), (weight, (0, -1, -1), 1), (residual, (1, 0, -1), 1), (output, (1, 0, -1), -1)])
+
+    def splitk_linear_res_atomic_m_parallel_layer(self, input: DTensor, weight: DTensor, residual: DTensor, workspace: DTensor,
+                                                  done_counter: DTensor, output: DTensor, k_splits: int, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2002: grid (N tiles, K splits, M tiles); the sum is deterministic here and the workspace and
+        counters stay untouched."""
+        assert input.num_dims == 2 and weight.num_dims == 2
+        self._task("splitk_linear_res_atomic_mi300", grid_dim, block_dim,
+                   [(input, (-1, 1, 0), 1), (weight, (0, 1, -1), 1), (residual, (1, -1, 0), 1), (workspace, (1, -1, 0), 1),
+                    (done_counter, (0, -1, 1), 1), (output, (1, -1, 0), -1)], [k_splits])
+
     # layers of the reference that are outside the one-GPU decode path
+    def tensor_init_layer(self, *args, **kwargs):
+        raise NotImplementedError("tensor_init_layer registers a Blackwell-only task (tasks/blackwell/tensor_init.cuh); it has no MI300-family kernel in the reference either")
+
     def allreduce_layer(self, *args, **kwargs):
         raise NotImplementedError("allreduce_layer: the MI355X megakernel runs on one GPU")
 

@@ -142,7 +142,7 @@ int mk_wait(mk_graph *g, void *stream, int *finished_out);
 /* mk_enqueue_steps for callers that cannot allocate (code under HIP graph capture, tight serving loops, harnesses that
  * forbid hipMalloc); it has no counterpart in the reference.  The call allocates and frees nothing, and every piece
  * of scratch its launch uses -- barrier counters, K-split partial tiles and counters, attention split-KV partials and
- * counters, sampling partials -- lives in one file-scope device array of about 22.8 MB per GPU (held until the process
+ * counters, sampling partials -- lives in one file-scope device array of about 19.6 MB per GPU (held until the process
  * ends) instead of in the buffers mk_compile allocated; it is cleared by a fill kernel on `stream`, not by a memset.
  * Limits (MK_EINVAL beyond them): at most 256 workgroups, max_num_batched_tokens x kv heads <= 512, at most 8 q heads
  * per kv head.  All calls on one GPU share that array: calls that overlap on one GPU race, whatever their handles or

@@ -147,14 +147,120 @@ def test_lowering_fuses_norm_and_swiglu_and_attention():
     assert tg["all_events"][0]["event_type"] == 911 and tg["all_events"][1]["event_type"] == 903 and tg["all_events"][-1]["event_type"] == 910
     assert tg["all_events"][1]["first_task_id"] == 2 and tg["all_events"][1]["last_task_id"] == n_tasks
     lin = [t for t in tg["all_tasks"] if t["task_type"] == 120]
-    assert lin[1]["inputs"][1]["base_ptr"] == "qkv_w" and lin[1]["inputs"][1]["dims"] == [64, 1024]  # 1536 rows over 24 blocks
-    assert lin[1]["inputs"][1]["offset"] == 64 * 1024 * 2 and lin[1]["outputs"][0]["offset"] == 64 * 2
+    # 1536 rows over 24 blocks; a shuffled weight is named by the source its slice starts in (runtime.cc:1229-1283):
+    # groups of [q 512 ; k 128 ; v 128] -> block 1 = q rows 64.., block 9 = k rows 64.., block 13 = q rows 576..
+    w1, w9, w13 = lin[1]["inputs"][1], lin[9]["inputs"][1], lin[13]["inputs"][1]
+    assert (w1["base_ptr"], w1["offset"], w1["dims"], w1["strides"]) == ("q", 64 * 1024 * 2, [64, 1024], [1024, 1])
+    assert (w9["base_ptr"], w9["offset"]) == ("k", 64 * 1024 * 2) and (w13["base_ptr"], w13["offset"]) == ("q", 576 * 1024 * 2)
+    assert lin[1]["outputs"][0]["offset"] == 64 * 2
+    assert tg["first_tasks"] == [2] and tg["all_tasks"][2]["dependent_event"] == 0x7FFFFFFFFFFFFFFE
     for key in ("trigger_event", "dependent_event", "request_id", "expert_offset", "kv_idx", "merge_task_offset", "n_tile_start", "n_tile_count"):
         assert key in lin[0]
     with pytest.raises(_capi.MkError, match="one GPU"):
         mpk.kn_graph.generate_task_graph(2, 1)
     with pytest.raises(_capi.MkError, match="without a device"):
         mpk.compile()
+
+
+def _events(tg):
+    return [(e["event_type"], e["num_triggers"], e["first_task_id"], e["last_task_id"]) for e in tg["all_events"]]
+
+
+def test_task_graph_events_follow_the_reference_partition_rule():
+    """Events between two operators as src/kernel/runtime.cc:53-140,519-612 builds them, expected values derived by hand:
+    one tensor carries the dependency; along each of its dims there are gcd(producer partition, consumer partition)
+    events; an event owns the consumer blocks of its slice (stored event by event, in bid order inside an event) and counts
+    the producer blocks of the matching slice."""
+    INV, EMPTY = 0x7FFFFFFFFFFFFFFE, 900
+    # (i) norm (4) -> 96-block QKV linear -> kv_cache_update (2, 8, 1) -> attention (2, 8, 1) -> o projection (16)
+    mpk = _host_mpk(B=4, R=2)
+    H, nq, nkv, D = 1024, 32, 8, 128
+    x, nw, n = mpk.new_tensor((4, H), name="x"), _t(mpk, "nw", H), mpk.new_tensor((4, H), name="n")
+    qkv_w = mpk.shuffle_tensors([_t(mpk, "q", nq * D, H), _t(mpk, "k", nkv * D, H), _t(mpk, "v", nkv * D, H)], 0, nkv, "qkv_w")
+    qkv = mpk.new_tensor((4, (nq + 2 * nkv) * D), name="qkv")
+    kc, vc = _t(mpk, "kc", 8, 16, nkv, D), _t(mpk, "vc", 8, 16, nkv, D)
+    qws, att, lse = mpk.new_tensor((4, nq * D), name="qws"), mpk.new_tensor((4, nq * D), name="att"), mpk.new_tensor((4, nq), dtype=mi.float32, name="lse")
+    mpk.rmsnorm_layer(input=x, weight=nw, output=n, grid_dim=(4, 1, 1), block_dim=(128, 1, 1))
+    mpk.linear_layer(input=n, weight=qkv_w, output=qkv, grid_dim=(96, 1, 1), block_dim=(128, 1, 1))
+    mpk.kv_cache_update_layer(input=qkv, k_cache=kc, v_cache=vc, q_norm=_t(mpk, "qn", D), k_norm=_t(mpk, "kn", D), cos_pos_embed=_t(mpk, "cos", 64, D),
+                              sin_pos_embed=_t(mpk, "sin", 64, D), q_workspace=qws, grid_dim=(2, nkv, 1), block_dim=(256, 1, 1))
+    mpk.paged_attention_ck_fmha_layer(q_workspace=qws, k_cache=kc, v_cache=vc, o_acc=att, lse_acc=lse, attention_params=(nq, 1, 2),
+                                      grid_dim=(2, nkv, 1), block_dim=(256, 1, 1))
+    mpk.linear_with_residual_layer(input=att, weight=_t(mpk, "wo", H, nq * D), residual=x, output=mpk.new_tensor((4, H), name="x1"),
+                                   grid_dim=(16, 1, 1), block_dim=(256, 1, 1))
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    n_tasks = 2 + 4 + 96 + 16 + 16 + 16
+    expect = [(911, 1, 0, 0), (903, 1, 2, n_tasks),
+              (EMPTY, 4, 6, 102)]                                       # the 4 norm rows -> all 96 linear blocks (the linear reads whole rows)
+    expect += [(EMPTY, 12, 102 + 2 * i, 104 + 2 * i) for i in range(8)]  # gcd(96, 8) = 8 slices of the qkv columns: 12 blocks -> kv head i of both requests
+    expect += [(EMPTY, 16, 118, 134), (EMPTY, 16, 134, 150), (910, 16, 0, 0)]
+    assert _events(tg) == expect
+    T = tg["all_tasks"]
+    assert tg["first_tasks"] == [2, 3, 4, 5]
+    assert [t["trigger_event"] for t in T[2:6]] == [2] * 4 and [t["dependent_event"] for t in T[2:6]] == [INV] * 4
+    assert [t["trigger_event"] for t in T[6:102]] == [3 + b // 12 for b in range(96)] and all(t["dependent_event"] == 2 for t in T[6:102])
+    # kv_cache_update tasks are stored event by event: (request 0, head i), (request 1, head i)
+    assert [(t["request_id"], t["dependent_event"]) for t in T[102:118]] == [(r, 3 + h) for h in range(8) for r in range(2)]
+    assert [t["inputs"][0]["offset"] for t in T[102:118]] == [h * 768 * 2 for h in range(8) for r in range(2)]
+    assert all(t["trigger_event"] == 11 for t in T[102:118]) and all(t["trigger_event"] == 12 for t in T[118:134])
+    assert [t["request_id"] for t in T[118:134]] == [r for r in range(2) for h in range(8)]  # plain bid order again
+    assert [(t["kv_idx"], t["merge_task_offset"]) for t in T[118:134]] == [(0, h) for r in range(2) for h in range(8)]
+    assert all(t["trigger_event"] == 13 and t["dependent_event"] == 12 for t in T[134:150])
+    # a task type that sets no metadata still carries request_id = bid.x in a union that started as all ones
+    assert (T[7]["request_id"], T[7]["n_tile_start"], T[7]["kv_idx"], T[7]["n_tile_count"], T[7]["merge_task_offset"], T[7]["expert_offset"]) == (1, 1, 65535, 65535, -1, -65535)
+    assert T[6]["variant_id"] == 0 and T[134]["variant_id"] == 0 and T[0]["trigger_event"] == INV and T[1]["trigger_event"] == 1
+
+    # (ii) two grids partitioned along both dims of the shared [8, 512] tensor: producer (8 column blocks, 4 row blocks),
+    # consumer (6, 2): rows gcd(4, 2) = 2 slices, columns gcd(8, 1) = 1
+    mpk = _host_mpk(B=8, R=2, pages=8)
+    a, y, z = mpk.new_tensor((8, 1024), name="a"), mpk.new_tensor((8, 512), name="y"), mpk.new_tensor((8, 384), name="z")
+    mpk.linear_m_parallel_layer(input=a, weight=_t(mpk, "W1", 512, 1024), output=y, grid_dim=(8, 4, 1), block_dim=(128, 1, 1))
+    mpk.linear_with_residual_m_parallel_layer(input=y, weight=_t(mpk, "W2", 384, 512), residual=mpk.new_tensor((8, 384), name="r"), output=z,
+                                              grid_dim=(6, 2, 1), block_dim=(128, 1, 1))
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    assert _events(tg) == [(911, 1, 0, 0), (903, 1, 2, 46), (EMPTY, 16, 34, 40), (EMPTY, 16, 40, 46), (910, 12, 0, 0)]
+    T = tg["all_tasks"]
+    assert [t["trigger_event"] for t in T[2:34]] == [2 + (i % 4) // 2 for i in range(32)]  # task 2 + 4 x + y waits on the slice of row block y
+    assert [(t["request_id"], t["inputs"][0]["offset"]) for t in T[34:46]] == [(xb, yb * 4 * 512 * 2) for yb in range(2) for xb in range(6)]
+    assert [t["dependent_event"] for t in T[34:46]] == [2] * 6 + [3] * 6 and all(t["trigger_event"] == 4 for t in T[34:46])
+
+    # (iii) mixture of experts: W13 (10, 24) -> activation (tokens 4, slots 8) -> W2 (8, 32) -> weighted sum (4, 8)
+    mpk = _host_mpk(B=4, R=2)
+    E, topk, Hm, Im = 16, 8, 2048, 768
+    xin, lg = mpk.new_tensor((4, Hm), name="xin"), mpk.new_tensor((4, E), name="lg")
+    tw, ri, mk = mpk.new_tensor((4, topk), dtype=mi.float32, name="tw"), mpk.new_tensor((E, 4), dtype=mi.int32, name="ri"), mpk.new_tensor((E + 1,), dtype=mi.int32, name="mk")
+    mid, act, eo = mpk.new_tensor((4, topk, 2 * Im), name="mid"), mpk.new_tensor((4, topk, Im), name="act"), mpk.new_tensor((4, topk, Hm), name="eo")
+    res, out = mpk.new_tensor((4, Hm), name="res"), mpk.new_tensor((4, Hm), name="out")
+    mpk.moe_topk_softmax_routing_layer(input=lg, output=(tw, ri, mk), grid_dim=(1, 1, 1), block_dim=(256, 1, 1))
+    mpk.moe_w13_linear_layer(input=xin, weight=_t(mpk, "w13", E, 2 * Im, Hm), moe_routing_indices=ri, moe_mask=mk, output=mid, grid_dim=(10, 24, 1), block_dim=(256, 1, 1))
+    mpk.moe_silu_mul_layer(input=mid, output=act, grid_dim=(4, topk, 1), block_dim=(256, 1, 1))
+    mpk.moe_w2_linear_layer(input=act, weight=_t(mpk, "w2", E, Hm, Im), moe_routing_indices=ri, moe_mask=mk, output=eo, grid_dim=(8, 32, 1), block_dim=(256, 1, 1))
+    mpk.moe_mul_sum_add_layer(input=eo, weight=tw, residual=res, output=out, grid_dim=(4, 8, 1), block_dim=(256, 1, 1))
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    base_w2, base_sum = 2 + 1 + 240 + 32, 2 + 1 + 240 + 32 + 256
+    expect = [(911, 1, 0, 0), (903, 1, 2, base_sum + 32), (EMPTY, 1, 3, 243), (EMPTY, 240, 243, 275), (EMPTY, 32, base_w2, base_sum)]
+    # the expert outputs [4, 8, 2048] are cut in 32 column blocks by W2 and in 8 by the weighted sum: gcd = 8 events, each
+    # fired by 8 x 4 W2 blocks and owning the four tokens' tasks of column block i
+    expect += [(EMPTY, 32, base_sum + 4 * i, base_sum + 4 * i + 4) for i in range(8)] + [(910, 32, 0, 0)]
+    assert _events(tg) == expect
+    T = tg["all_tasks"]
+    assert [t["expert_offset"] for t in T[3:243]] == [(yb << 16) | xb for xb in range(10) for yb in range(24)]  # moe tasks pack (bid.y, bid.x)
+    assert [t["trigger_event"] for t in T[base_w2:base_sum]] == [5 + yb // 4 for xb in range(8) for yb in range(32)]
+    assert [(t["request_id"], t["dependent_event"]) for t in T[base_sum:base_sum + 32]] == [(tok, 5 + i) for i in range(8) for tok in range(4)]
+    assert [t["outputs"][0]["offset"] for t in T[base_sum:base_sum + 32]] == [(tok * Hm + i * 256) * 2 for i in range(8) for tok in range(4)]
+
+    # gang tasks: one task per die; n_tile_count = tiles per die, attention tasks also their first work item
+    mpk = _host_mpk(B=4, R=2)
+    n2, w8 = mpk.new_tensor((4, H), name="n"), _t(mpk, "w8", 4096, H)
+    o8 = mpk.new_tensor((4, 4096), name="o8")
+    mpk.gang_rmsnorm_layer(input=mpk.new_tensor((4, H), name="x"), weight=_t(mpk, "nw", H), output=n2)
+    mpk.gang_linear_layer(input=n2, weight=w8, output=o8, tile_n=64, output_stride=4096, m_tiles=1)
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    T = tg["all_tasks"]
+    assert _events(tg) == [(911, 1, 0, 0), (903, 1, 2, 18), (EMPTY, 8, 10, 18), (910, 8, 0, 0)]
+    assert [(t["n_tile_start"], t["n_tile_count"]) for t in T[2:10]] == [(0, 4)] * 8       # gang_rmsnorm: params[0] = batch rows
+    assert [(t["n_tile_start"], t["n_tile_count"]) for t in T[10:18]] == [(0, 8)] * 8      # 4096 / 8 dies / 64 = 8 tiles per die
+    assert [t["inputs"][1]["offset"] for t in T[10:18]] == [d * 512 * H * 2 for d in range(8)]  # die d streams weight chunk d
 
 
 def test_lowering_rejects_bad_graphs():
@@ -352,15 +458,30 @@ def test_split_k_pair_and_fused_activation_lower_to_linear_stages():
     prog = [l.split(None, 1)[1] for l in mpk.describe_program().splitlines()]
     kinds = [l.split()[0] for l in prog]
     assert kinds == ["NORM[multi-token", "LINEAR+norm+res", "NORM[multi-token", "LINEAR+norm", "LINEAR+res"]
-    assert "-> y" in prog[1] and "+silu half=256 folded in" in prog[3] and "silu_mul(mlp_mid) x wd -> out" in prog[4] and "k=1536" in prog[4]
-    # a physically interleaved gate/up weight: the producer's grid (one block per half-group) says where gate ends
+    assert "-> y" in prog[1] and "+silu half=256 " in prog[3] and "folded in" in prog[3] and "silu_mul(mlp_mid) x wd -> out" in prog[4] and "k=1536" in prog[4]
+    # a physical gate/up weight: [gate | up] halves as the reference task kernel reads them (whatever the producer's grid),
+    # unless the caller that interleaved it says how
+    for kw, half in (({}, I), ({"gate_rows_per_group": 128}, 128)):
+        mpk = _host_mpk(B=4, R=2)
+        n, guw = mpk.new_tensor((4, H), name="n"), _t(mpk, "gu", 2 * I, H)
+        mid, wd, y, out = mpk.new_tensor((4, 2 * I), name="mid"), _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="out")
+        mpk.linear_layer(input=n, weight=guw, output=mid, grid_dim=(24, 1, 1), block_dim=(128, 1, 1))
+        mpk.silu_mul_linear_with_residual_layer(input=mid, weight=wd, residual=y, output=out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1), **kw)
+        assert f"+silu half={half} " in mpk.describe_program()
+    with pytest.raises(_capi.MkError, match="do not divide"):
+        mpk = _host_mpk(B=4, R=2)
+        mid, wd, y, out = _t(mpk, "mid", 4, 2 * I), _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="out")
+        mpk.silu_mul_linear_with_residual_layer(input=mid, weight=wd, residual=y, output=out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1), gate_rows_per_group=1000)
+        mpk.describe_program()
+    # a later reader of the gate/up tensor keeps it written: the activation is a stage of its own
     mpk = _host_mpk(B=4, R=2)
     n, guw = mpk.new_tensor((4, H), name="n"), _t(mpk, "gu", 2 * I, H)
     mid, wd, y, out = mpk.new_tensor((4, 2 * I), name="mid"), _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="out")
     mpk.linear_layer(input=n, weight=guw, output=mid, grid_dim=(24, 1, 1), block_dim=(128, 1, 1))
     mpk.silu_mul_linear_with_residual_layer(input=mid, weight=wd, residual=y, output=out, grid_dim=(H // 64, 1, 1), block_dim=(256, 1, 1))
-    prog = mpk.describe_program()
-    assert "+silu half=128 folded in" in prog
+    mpk.silu_mul_layer(input=mid, output=mpk.new_tensor((4, I), name="act"), grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
+    kinds = [l.split()[1] for l in mpk.describe_program().splitlines()]
+    assert kinds == ["LINEAR", "SILU_MUL", "LINEAR+res", "SILU_MUL"]
     # an input of unknown origin is read as [gate | up] halves by a standalone activation stage
     mpk = _host_mpk(B=4, R=2)
     mid, wd, y, out = _t(mpk, "mid", 4, 2 * I), _t(mpk, "wd", H, I), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="out")
@@ -375,6 +496,33 @@ def test_split_k_pair_and_fused_activation_lower_to_linear_stages():
         mpk.describe_program()
 
 
+def test_layer_methods_that_stand_for_other_tasks():
+    """rmsnorm_linear / identity / argmax / attention / *_m_parallel (python/mirage/mpk/persistent_kernel.py:566,587,1953-2043,2153,
+    2195): recorded under the reference's task names and ids, lowered to the stages of the tasks they stand for."""
+    mpk = _host_mpk(B=4, R=2, max_seq=64, pages=2, page_size=64)
+    H, V, D, nq, nkv = 1024, 4096, 128, 8, 2
+    x, nw, W = mpk.new_tensor((4, H), name="x"), _t(mpk, "nw", H), _t(mpk, "W", (nq + 2 * nkv) * D, H)
+    qkv, att, y, z = mpk.new_tensor((4, (nq + 2 * nkv) * D), name="qkv"), mpk.new_tensor((4, nq * D), name="att"), mpk.new_tensor((4, H), name="y"), mpk.new_tensor((4, H), name="z")
+    mpk.rmsnorm_linear_layer(input=x, weight_norm=nw, weight_linear=W, output=qkv, grid_dim=(24, 1, 1), block_dim=(128, 1, 1))
+    kc, vc = _t(mpk, "kc", 2, 64, nkv, D), _t(mpk, "vc", 2, 64, nkv, D)
+    cos, sin = _t(mpk, "cos", 64, D), _t(mpk, "sin", 64, D)
+    mpk.attention_layer(input=qkv, k_cache=kc, v_cache=vc, q_norm=_t(mpk, "qn", D), k_norm=_t(mpk, "kn", D), cos_pos_embed=cos, sin_pos_embed=sin,
+                        output=att, grid_dim=(2, nkv, 1), block_dim=(128, 1, 1))
+    mpk.linear_with_residual_m_parallel_layer(input=att, weight=_t(mpk, "Wo", H, nq * D), residual=x, output=y, grid_dim=(16, 2, 1), block_dim=(128, 1, 1))
+    mpk.identity_layer(input=y, output=z, grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
+    lg = mpk.new_tensor((4, V), name="logits")
+    mpk.linear_m_parallel_layer(input=z, weight=_t(mpk, "head", V, H), output=lg, grid_dim=(64, 2, 1), block_dim=(128, 1, 1))
+    mpk.argmax_layer(input=lg, output=_t(mpk, "tok", 4, 1, dtype=torch.int64), grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
+    kinds = [l.split()[1] for l in mpk.describe_program().splitlines()]
+    assert kinds == ["NORM[multi-token", "LINEAR+norm", "ATTN", "LINEAR+res", "COPY", "LINEAR", "ARGMAX_PARTIAL", "ARGMAX_REDUCE"], kinds
+    tg = json.loads(mpk.kn_graph.generate_task_graph(1, 0)["json_file"])
+    types = [t["task_type"] for t in tg["all_tasks"][2:]]
+    # TASK_RMS_NORM_LINEAR 102 x24, TASK_ATTENTION_1 103 x4, TASK_LINEAR_WITH_RESIDUAL 108 x32, TASK_IDENTITY 121, TASK_LINEAR 120 x128, TASK_ARGMAX 109
+    assert types == [102] * 24 + [103] * 4 + [108] * 32 + [121] + [120] * 128 + [109]
+    with pytest.raises(NotImplementedError, match="Blackwell"):
+        mpk.tensor_init_layer()
+
+
 def test_modes_and_configuration_limits():
     meta = make_meta(2, 64, 4, 2, 8, device="cpu")
     kw = dict(world_size=1, mpi_rank=0, num_workers=256, num_local_schedulers=0, num_remote_schedulers=0, max_seq_length=64,
@@ -382,8 +530,11 @@ def test_modes_and_configuration_limits():
               trace_name=None, spec_decode_config=None, use_cutlass_kernel=False)
     for mode in ("offline", "online", "online_notoken", "onepass"):
         assert mi.PersistentKernel(mode=mode, **kw).mode == mode
-    with pytest.raises(NotImplementedError, match="multi_turn"):
-        mi.PersistentKernel(mode="multi_turn", **kw)
+    for spelling in ("online_multi_turn", "multi_turn"):  # the reference's spelling (persistent_kernel.py:132) and the short one
+        with pytest.raises(NotImplementedError, match=spelling):
+            mi.PersistentKernel(mode=spelling, **kw)
+    with pytest.raises(ValueError, match="Invalid persistent kernel mode"):
+        mi.PersistentKernel(mode="sometimes", **kw)
     assert mi.PersistentKernel(mode="offline", **kw).max_tokens_per_request == 8  # the reference's default on AMD
     assert mi.PersistentKernel(mode="offline", max_tokens_per_request=64, **kw).max_tokens_per_request == 64
     with pytest.raises(_capi.MkError, match="max_tokens_per_request"):
@@ -391,6 +542,17 @@ def test_modes_and_configuration_limits():
     # two requests of up to 4 pages each need 8 pages: the page ring hands pages out without checking
     with pytest.raises(_capi.MkError, match="cannot back 2 concurrent requests"):
         mi.PersistentKernel(mode="offline", **{**kw, "max_num_pages": 7, "meta_tensors": make_meta(2, 64, 4, 2, 7, device="cpu")})
+    # ... which is a limit of the on-GPU page ring only: where the host owns the page table (online_notoken, onepass) the
+    # pool may be oversubscribed, and may hold more pages than the on-GPU scheduler's snapshot could
+    for mode in ("online_notoken", "onepass"):
+        assert mi.PersistentKernel(mode=mode, **{**kw, "max_num_pages": 5, "meta_tensors": make_meta(2, 64, 4, 2, 5, device="cpu")}).mode == mode
+        big = dict(kw, max_num_pages=40000, page_size=1, max_seq_length=64, meta_tensors=make_meta(2, 64, 4, 2, 40000, device="cpu"))
+        assert mi.PersistentKernel(mode=mode, **big).mode == mode
+    with pytest.raises(_capi.MkError, match="LDS snapshot"):
+        mi.PersistentKernel(mode="offline", **dict(kw, max_num_pages=40000, page_size=1, meta_tensors=make_meta(2, 64, 4, 2, 40000, device="cpu")))
+    with pytest.raises(_capi.MkError, match="pages per request"):  # the attention stage's own limit holds in every mode
+        mi.PersistentKernel(mode="online_notoken", **dict(kw, max_num_pages=40000, page_size=1, max_seq_length=9000,
+                                                           meta_tensors=make_meta(2, 9000, 4, 2, 40000, device="cpu")))
     # tensor id -1 is accepted only for the optional operands of the attention tasks
     mpk = _host_mpk()
     x, W = _t(mpk, "x", 4, 1024), _t(mpk, "W", 512, 1024)

@@ -106,3 +106,48 @@ def test_online_mode_walks_host_written_tokens():
         assert int(on.meta["step"][0].item()) >= max_seq - 2
         assert torch.equal(on.meta["tokens"].cpu(), ref_tokens), "online mode must not write tokens"
         on.mpk.finalize()
+
+
+def test_online_notoken_rejects_a_batch_it_cannot_run():
+    """A request with more rows than max_tokens_per_request (or a sequence shorter than its rows, or rows that overlap)
+    is not truncated: the launch runs nothing, mk_wait reports MK_EINVAL, and the K/V cache is untouched."""
+    from mirage import _capi
+    from oracle.qwen3_ref import make_model_weights
+    cfg = _cfg()
+    w = make_model_weights(cfg, seed=43)
+    R, B, max_seq, PS = 3, 16, 48, 16
+    on = _decoder(cfg, w, max_num_batched_tokens=B, max_num_batched_requests=R, max_seq_length=max_seq, page_size=PS, total_requests=R,
+                  kernel_mode="online_notoken")  # max_tokens_per_request defaults to 8
+    m = on.meta
+
+    def describe(qo, kv_ptr, last):
+        m["input_tokens"].copy_(torch.arange(B, dtype=torch.int64).view(-1, 1) % cfg.vocab_size)
+        m["qo_indptr_buffer"].copy_(torch.tensor(qo, dtype=torch.int32))
+        m["paged_kv_indptr_buffer"].copy_(torch.tensor(kv_ptr, dtype=torch.int32))
+        m["paged_kv_indices_buffer"].copy_(torch.arange(m["paged_kv_indices_buffer"].numel(), dtype=torch.int32))
+        m["paged_kv_last_page_len_buffer"].copy_(torch.tensor(last, dtype=torch.int32))
+        torch.cuda.synchronize()
+
+    caches = [on.k_cache, on.v_cache]
+    for c in caches:
+        c.fill_(0.25)
+    # a valid request (4 rows of a 4-long sequence) next to one with 9 rows: over the cap of 8
+    describe([0, 4, 13, 13], [0, 1, 2, 2], [4, 9, 0])
+    with pytest.raises(_capi.MkError, match="max_tokens_per_request"):
+        on.mpk()
+    # a sequence shorter than its new rows (2 positions, 3 rows)
+    describe([0, 3, 3, 3], [0, 1, 1, 1], [2, 0, 0])
+    with pytest.raises(_capi.MkError, match="shorter than its new rows"):
+        on.mpk()
+    # rows beyond max_num_batched_tokens
+    describe([0, 8, 16, 24], [0, 1, 2, 3], [8, 8, 8])
+    with pytest.raises(_capi.MkError, match="rows outside"):
+        on.mpk()
+    torch.cuda.synchronize()
+    assert all(bool((c == 0.25).all()) for c in caches), "a rejected batch must not append K/V rows"
+    # the handle stays usable: the same shape of batch within the limits runs
+    describe([0, 4, 12, 12], [0, 1, 2, 2], [4, 8, 0])
+    on.mpk()
+    assert on.mpk.stats()["aborted"] == 0
+    assert not all(bool((c == 0.25).all()) for c in caches)
+    on.mpk.finalize()
