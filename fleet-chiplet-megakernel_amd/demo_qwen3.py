@@ -109,10 +109,13 @@ class Qwen3Decoder:
     def __init__(self, shape: Qwen3Shape, weights: dict, max_num_batched_tokens: int = 1, max_num_batched_requests: int = None,
                  max_seq_length: int = 1200, page_size: int = 4096, max_num_pages: int = None, total_requests: int = None,
                  mode: str = "fleet", eos_token_id: int = 0x7FFFFFFF, cos_sin=None, device="cuda", num_workers=None, with_head: bool = True,
-                 kernel_mode: str = "offline", max_tokens_per_request: int = None):
+                 kernel_mode: str = "offline", max_tokens_per_request: int = None, tap_last_layer_input: bool = False):
         assert mode in ("fleet", "mpk")
         self.shape, self.w, self.mode = shape, weights, mode
         self.with_head = with_head
+        # (diagnostics) keep a copy of the hidden state entering the last layer in t["layer_in_tap"]: every layer writes the
+        # same activation buffers, so the last layer otherwise overwrites its own input
+        self.tap_last_layer_input = tap_last_layer_input
         B = max_num_batched_tokens
         R = max_num_batched_requests or B
         self.B, self.R = B, R
@@ -213,6 +216,9 @@ class Qwen3Decoder:
 
         for i, lw in enumerate(w["layers"]):
             proj_out, layer_out = attn_proj_out, mlp_out
+            if self.tap_last_layer_input and i == len(w["layers"]) - 1:
+                t["layer_in_tap"] = new("layer_in_tap", H)
+                mpk.identity_layer(input=x, output=t["layer_in_tap"], grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
             w_norm = mpk.attach_input(lw["input_norm"], f"layer_{i}_input_layernorm")
             w_q = mpk.attach_input(lw["q_proj"], f"layer_{i}_q_proj")
             w_k = mpk.attach_input(lw["k_proj"], f"layer_{i}_k_proj")

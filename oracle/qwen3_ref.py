@@ -197,13 +197,14 @@ def moe_routing_tables(experts, num_experts: int):
     return routing, active
 
 
-def moe_mlp_k(h, x_res, gate_up, down, weights, experts):
+def moe_mlp_k(h, x_res, gate_up, down, weights, experts, acc=torch.float32):
     """Kernel-order expert MLP + combine on T tokens.  h: normalised input [T, H] bf16; x_res: residual [T, H] bf16;
     gate_up [E, 2I, H], down [E, H, I].  Rounding points follow the reference's task sequence
     (demo/qwen3/demo_30B_A3B.py:697-754): W13 output [T, topk, 2I] rounded to bf16
     (tasks/mi300/moe_linear_mi300.cuh:53-295), SwiGLU on those bf16 values -> bf16, W2 output [T, topk, H] rounded to
     bf16, then out = bf16(res + sum_k w_k * y_k) accumulated in fp32 in slot order
-    (tasks/mi300/moe_mul_sum_add_mi300.cuh:41-54).  Returns (out, mid, act, y)."""
+    (tasks/mi300/moe_mul_sum_add_mi300.cuh:41-54).  `acc`: accumulation type of the two expert linears (see linear_k).
+    Returns (out, mid, act, y)."""
     T, topk = experts.shape
     I2 = gate_up.shape[1]
     H = down.shape[1]
@@ -215,9 +216,9 @@ def moe_mlp_k(h, x_res, gate_up, down, weights, experts):
         acc = x_res[t].float()
         for s in range(topk):
             e = int(experts[t, s])
-            mid[t, s] = (h[t].float() @ gate_up[e].float().t()).to(BF16)
+            mid[t, s] = (h[t].to(acc) @ gate_up[e].to(acc).t()).to(BF16)
             act[t, s] = silu_mul_k(mid[t, s, :I2 // 2], mid[t, s, I2 // 2:])
-            y[t, s] = (act[t, s].float() @ down[e].float().t()).to(BF16)
+            y[t, s] = (act[t, s].to(acc) @ down[e].to(acc).t()).to(BF16)
             acc = acc + y[t, s].float() * weights[t, s]
         out[t] = acc.to(BF16)
     return out, mid, act, y
@@ -334,7 +335,7 @@ class Qwen3Oracle:
                 gate = linear_k(h, W["router"], acc=acc)
                 self.route_margins.append(float(moe_route_margin(gate, cfg.num_experts_per_tok).min()))
                 wts, exp = moe_route_k(gate, cfg.num_experts_per_tok)
-                return moe_mlp_k(h, x, W["gate_up_proj"], W["down_proj"], wts, exp)[0]
+                return moe_mlp_k(h, x, W["gate_up_proj"], W["down_proj"], wts, exp, acc=acc)[0]
             m = linear_silu_k(h, W["gate_proj"], W["up_proj"], acc=acc)
             return linear_k(m, W["down_proj"], res=x, acc=acc)
         if self.order == "f64":

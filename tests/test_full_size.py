@@ -37,7 +37,10 @@ def test_config3_full_size_teacher_forced(capsys):
     (2) end to end the GPU is no further from the float64-sum oracle than 1.5 x the distance between the two oracles
         (max |diff| and relative L2 of the logits), and its logits have cosine > 0.999 with it;
     (3) the sampled token's logit in the float64-sum oracle is within twice the largest single-logit distance between the
-        two oracles of that oracle's maximum, and it IS that oracle's argmax wherever the top-2 margin exceeds that bound."""
+        two oracles of that oracle's maximum, and it IS that oracle's argmax wherever the top-2 margin exceeds that bound.
+    (2) and (3) are asserted on EVERY row the run produces -- all 80 prompt positions (teacher-forced by construction:
+    the kernel samples a token for every prompt row, the scheduler only does not use it) and the decode rows -- so that
+    the argmax comparison is made on the rows whose margin is decisive: at least eight of them."""
     from demo_qwen3 import Qwen3Decoder, Qwen3Shape, random_weights
     from helpers import bf16_ulp_diff
     from oracle.qwen3_ref import KVCache, Qwen3Config, Qwen3Oracle, argmax_k, linear_k
@@ -51,46 +54,58 @@ def test_config3_full_size_teacher_forced(capsys):
     dec = Qwen3Decoder(shape, wg, max_num_batched_tokens=8, max_num_batched_requests=1, max_seq_length=max_seq, page_size=4096)
     prompt = torch.randint(0, shape.vocab_size, (P,), generator=torch.Generator().manual_seed(0))
     dec.load_prompts([prompt])
-    # GPU: prompt in chunks of 8 tokens, then NEW decode steps; keep the logits, the final normalised hidden state and the
-    # sampled token of the prompt's last token (an 8-row iteration) and of every decode step (1-row iterations)
+    # GPU: prompt in chunks of 8 tokens, then NEW decode steps; keep the logits and the sampled token of every row, and the
+    # final normalised hidden state of the prompt's last token (an 8-row iteration) and of every decode step (1-row iterations)
     gpu_logits, gpu_hidden, gpu_tokens = [], [], []
     for it in range(P // 8 + NEW):
         assert not dec.mpk.run_steps(1)
-        if it >= P // 8 - 1:
-            row = 7 if it == P // 8 - 1 else 0
-            gpu_logits.append(dec.logits()[row].cpu())
-            gpu_hidden.append(dec.t["rmsnorm_out"].to_torch()[row].cpu())
-            gpu_tokens.append(int(dec.meta["output_tokens"][row, 0].item()))
+        rows = range(8) if it < P // 8 else range(1)
+        lg, hd, tk = dec.logits().cpu(), dec.t["rmsnorm_out"].to_torch().cpu(), dec.meta["output_tokens"][:, 0].cpu()
+        for r in rows:
+            gpu_logits.append(lg[r].clone())
+            gpu_hidden.append(hd[r].clone())
+            gpu_tokens.append(int(tk[r]))
+    n_rows = P + NEW
+    assert len(gpu_tokens) == n_rows
     # step[] and tokens[] are committed by the scheduler step that opens the NEXT iteration: the last sampled token is still pending
     assert int(dec.meta["step"][0].item()) == P + NEW - 1
-    assert dec.meta["tokens"][0, P:P + NEW].cpu().tolist() == gpu_tokens[:NEW]
+    assert dec.meta["tokens"][0, P:P + NEW].cpu().tolist() == gpu_tokens[P - 1:P - 1 + NEW]
     assert dec.mpk.stats()["aborted"] == 0
     _say(capsys, "copying the weights to the host")
     w = _weights_to_host(wg)
     dec.mpk.finalize()
     del dec, wg
     torch.cuda.empty_cache()
-    # (1) head + argmax on the GPU's own hidden state
-    for i in range(NEW + 1):
+    # (1) head + argmax on the GPU's own hidden state: the last prompt row and the decode rows (and the first prompt row)
+    for i in [0] + list(range(P - 1, n_rows)):
         head = linear_k(gpu_hidden[i][None], w["lm_head"])[0]
         ulp, mabs = bf16_ulp_diff(gpu_logits[i], head, floor=1.0 / 16)
         frac = float((gpu_logits[i].float() != head.float()).float().mean())
         assert ulp <= 1.0 and frac < 0.02, f"row {i}: LM head differs from the oracle on the same input: {frac:.4f} of 151936 logits, max {ulp} ulp ({mabs})"
+    for i in range(n_rows):
         assert gpu_tokens[i] == int(argmax_k(gpu_logits[i][None])[0]), f"row {i}: sampled token is not the lowest index of the maximum logit"
     _say(capsys, "LM head and argmax exact on the GPU's own hidden state; oracles: 80-token prompt (fp32 sums, then float64 sums)")
     o32, o64 = Qwen3Oracle(cfg, w, "kernel"), Qwen3Oracle(cfg, w, "kernel", acc=torch.float64)
     c32, c64 = KVCache(cfg, P + NEW + 2), KVCache(cfg, P + NEW + 2)
-    a = o32.forward(prompt, c32, 0)[-1].double()
-    b = o64.forward(prompt, c64, 0)[-1].double()
-    hits = 0
-    for i in range(NEW + 1):
+    A = o32.forward(prompt, c32, 0)
+    B = o64.forward(prompt, c64, 0)
+    hits, worst = 0, (0.0, 0.0, 1.0)
+    for i in range(n_rows):
+        if i >= P:  # decode rows: one more oracle step each, fed with the token the GPU sampled
+            ids = torch.tensor([gpu_tokens[i - 1]])
+            a = o32.forward(ids, c32, i)[0].double()
+            b = o64.forward(ids, c64, i)[0].double()
+        else:
+            a, b = A[i].double(), B[i].double()
         g = gpu_logits[i].double()
         d_or, d_gpu = (a - b).abs(), (g - b).abs()
         rel = lambda d: float(d.norm() / b.norm())
         cos = float(torch.nn.functional.cosine_similarity(g, b, dim=0))
-        within = float((d_gpu <= 2e-2 + 1e-2 * b.abs()).double().mean())
-        _say(capsys, f"row {i}: oracle fp32 vs float64 sums max |diff| {float(d_or.max()):.3f} rel L2 {rel(d_or):.4f}; GPU vs float64-sum oracle "
-                     f"max |diff| {float(d_gpu.max()):.3f} rel L2 {rel(d_gpu):.4f} cosine {cos:.5f} ({within:.2f} of logits within 2e-2 / 1e-2)")
+        if i >= P - 1:
+            within = float((d_gpu <= 2e-2 + 1e-2 * b.abs()).double().mean())
+            _say(capsys, f"row {i}: oracle fp32 vs float64 sums max |diff| {float(d_or.max()):.3f} rel L2 {rel(d_or):.4f}; GPU vs float64-sum oracle "
+                         f"max |diff| {float(d_gpu.max()):.3f} rel L2 {rel(d_gpu):.4f} cosine {cos:.5f} ({within:.2f} of logits within 2e-2 / 1e-2)")
+        worst = (max(worst[0], float(d_gpu.max()) / max(float(d_or.max()), 1e-3)), max(worst[1], rel(d_gpu) / max(rel(d_or), 1e-4)), min(worst[2], cos))
         assert float(d_gpu.max()) <= 1.5 * float(d_or.max()) + 1e-2, f"row {i}: GPU is further from the oracle than summation order explains"
         assert rel(d_gpu) <= 1.5 * rel(d_or) + 1e-3 and cos > 0.999
         # the sampled token is a near-maximal token of the oracle: its oracle logit is within the drift of the oracle's maximum
@@ -99,11 +114,9 @@ def test_config3_full_size_teacher_forced(capsys):
         if float(top2[0] - top2[1]) > 2 * float(d_or.max()):
             assert gpu_tokens[i] == int(b.argmax()), f"row {i}: argmax differs from the oracle at a margin of {float(top2[0] - top2[1]):.3f}"
             hits += 1
-        if i < NEW:
-            ids = torch.tensor([gpu_tokens[i]])
-            a = o32.forward(ids, c32, P + i)[0].double()
-            b = o64.forward(ids, c64, P + i)[0].double()
-    _say(capsys, f"done: {NEW + 1} rows checked, {hits} with a decisive margin\n")
+    _say(capsys, f"done: {n_rows} rows checked (worst GPU/oracle distance ratio: max |diff| {worst[0]:.2f}, rel L2 {worst[1]:.2f}; lowest cosine {worst[2]:.5f}), "
+                 f"{hits} with a decisive margin\n")
+    assert hits >= 8, f"only {hits} rows had a top-2 margin above the oracle's own drift: the argmax comparison needs more rows"
 
 
 def _sched_oracle_end_state(prompt_lens, R, B, max_pages, page_size, max_seq):
