@@ -225,6 +225,8 @@ def main():
     ap.add_argument("--model", choices=["qwen3-8b", "qwen3-30b-a3b"], default="qwen3-8b",
                     help="qwen3-8b: the headline dense shape; qwen3-30b-a3b: the mixture-of-experts shape (128 experts, top-8), reported alongside")
     ap.add_argument("--no-cpu-baseline", action="store_true")
+    ap.add_argument("--single-weight-copy", action="store_true",
+                    help="keep every linear weight once, in matrix-core tile order (BS >= 2): what the memory saving costs iterations of one or two tokens")
     ap.add_argument("--calib-copy", action="store_true", help="also run one 1 GiB device-to-device copy (scale for rocprofv3 FETCH_SIZE / WRITE_SIZE)")
     ap.add_argument("--stage-profile", action="store_true",
                     help="after each timed launch, print its last iteration's per-stage timeline over all workgroups to stderr")
@@ -264,7 +266,8 @@ def main():
         # requests sit at different contexts (the range is in `workload`; the KV bytes of the roofline are the real ones);
         # max_seq_len is the configuration's 1200 unless the earliest request's K timed steps would not fit.
         max_seq = max(1200, P + W + K + 2 + (0 if B == 1 else 6 * P))
-        dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode)
+        dec = Qwen3Decoder(shape, weights, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=4096, mode=args.mode,
+                           single_weight_copy=args.single_weight_copy)
         legs.append(run_leg(torch, dec, shape, args.model, B, K, W, P, max_seq, args.mode, args.stage_profile))
         dec.mpk.finalize()
         del dec

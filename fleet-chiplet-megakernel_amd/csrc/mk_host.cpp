@@ -119,6 +119,10 @@ struct mk_graph {
   size_t attn_cnt_n = 0;
   int num_ref_tasks = 0, num_ref_events = 0;
   int last_linear_task = -1, last_linear_stage = -1;  // lowering: the most recent linear task and the stage it became
+  std::vector<int> stage_weight;      // per stage: tensor id of a LINEAR stage's weight operand (-1: none)
+  std::vector<char> releasable;       // per tensor (single-weight-copy graphs, after mk_compile): the handle never reads it again
+  bool single_copy = false;
+  int64_t row_major_bytes = 0;
 };
 
 namespace {
@@ -345,6 +349,8 @@ int lower_linear(mk_graph *g, size_t &i) {
                               (st.flags & MK_F_SILU) ? "+silu" : "", tin.name.c_str(), g->tensors[w_id].name.c_str(), tfo.name.c_str(), st.n, st.k,
                               st.w.nseg));
   g->weight_bytes += (int64_t)st.n * st.k * 2;
+  g->stage_weight.resize(g->stages.size(), -1);
+  g->stage_weight.back() = w_id;
   g->last_linear_task = (int)i;
   g->last_linear_stage = (int)g->stages.size() - 1;
   i += act ? 2 : consumed_linear;
@@ -442,6 +448,8 @@ int lower_silu_mul_linear(mk_graph *g, size_t &i) {
   g->stages.push_back(st);
   g->stage_desc.push_back(fmt("LINEAR+res silu_mul(%s) x %s -> %s n=%d k=%d", x.name.c_str(), w.name.c_str(), o.name.c_str(), st.n, st.k));
   g->weight_bytes += (int64_t)st.n * st.k * 2;
+  g->stage_weight.resize(g->stages.size(), -1);
+  g->stage_weight.back() = t.ops[1];
   i++;
   return MK_OK;
 }
@@ -743,6 +751,7 @@ int lower_moe_combine(mk_graph *g, size_t &i, bool fused_single) {
 int lower(mk_graph *g) {
   g->stages.clear();
   g->stage_desc.clear();
+  g->stage_weight.clear();
   g->weight_bytes = 0;
   g->last_linear_task = g->last_linear_stage = -1;
   const int B = g->cfg.max_num_batched_tokens;
@@ -991,6 +1000,7 @@ int lower(mk_graph *g) {
       return fail(MK_EUNSUPPORTED, "task '%s' has no MI355X lowering", t.name.c_str());
     }
   }
+  g->stage_weight.resize(g->stages.size(), -1);
   g->program_text.clear();
   for (size_t s = 0; s < g->stage_desc.size(); s++) g->program_text += fmt("%3zu ", s) + g->stage_desc[s] + "\n";
   return MK_OK;
@@ -1692,8 +1702,15 @@ static int pack_weights(mk_graph *g, bool allocate) {
 int mk_repack_weights(mk_graph *g) {
   if (!g) return fail(MK_EINVAL, "null argument");
   if (!g->compiled) return fail(MK_ESTATE, "graph not compiled");
+  if (g->single_copy) return fail(MK_ESTATE, "this graph keeps only the tile copies of its weights (MK_CFG_SINGLE_WEIGHT_COPY): the row-major tensors may be gone");
   HIP_TRY(hipSetDevice(g->cfg.device));
   return pack_weights(g, false);
+}
+
+int mk_tensor_releasable(mk_graph *g, int id) {
+  if (!g || id < 0 || id >= (int)g->tensors.size()) return fail(MK_EINVAL, "bad tensor id %d", id);
+  if (!g->compiled || id >= (int)g->releasable.size()) return 0;
+  return g->releasable[id] ? 1 : 0;
 }
 
 int mk_compile(mk_graph *g) {
@@ -1774,6 +1791,52 @@ int mk_compile(mk_graph *g) {
       s.aux1 = rt.attn_cnt + g->attn_cnt_n / 2;
     }
   if ((rc = pack_weights(g, true))) return rc;
+  g->single_copy = (c.flags & MK_CFG_SINGLE_WEIGHT_COPY) && c.max_num_batched_tokens >= 2;
+  rt.packed_only = g->single_copy ? 1 : 0;
+  g->releasable.assign(g->tensors.size(), 0);
+  g->row_major_bytes = 0;
+  {
+    // which attached tensors does a linear stage read in place, and which do other stages read?
+    auto storage_ids = [&](int id, std::vector<int> &out) {
+      if (id < 0) return;
+      const Tensor &t = g->tensors[id];
+      if (t.kind == T_SHUFFLED) out.insert(out.end(), t.sources.begin(), t.sources.end());
+      else out.push_back(id);
+    };
+    std::vector<char> as_linear_weight(g->tensors.size(), 0), otherwise(g->tensors.size(), 0);
+    for (size_t si = 0; si < g->stages.size(); si++) {
+      if (g->stages[si].op != MK_OP_LINEAR || g->stage_weight[si] < 0) continue;
+      // (the forms that stream the tile copy at every token count need whole 64-wide steps per wavefront: k % 256 == 0)
+      if (g->single_copy && (!g->stages[si].wpack || (g->stages[si].k & 255)))
+        return fail(MK_EUNSUPPORTED, "MK_CFG_SINGLE_WEIGHT_COPY: the weight of stage %zu (%s) cannot be laid out in matrix-core tiles (k=%d is not a multiple of 256)", si,
+                    g->stage_desc[si].c_str(), g->stages[si].k);
+      std::vector<int> ids;
+      storage_ids(g->stage_weight[si], ids);
+      for (int id : ids) as_linear_weight[id] = 1;
+    }
+    // every other use of a tensor: any operand of any task except the weight operand (the second) of a linear task
+    for (const Task &t : g->ltasks) {
+      bool r_, s_;
+      int e_;
+      const bool lin = linear_kind(t.name, &r_, &s_, &e_) || t.name == "silu_mul_linear_with_residual";
+      for (size_t a = 0; a < t.ops.size(); a++) {
+        if (t.ops[a] < 0 || (lin && a == 1)) continue;
+        std::vector<int> ids;
+        storage_ids(t.ops[a], ids);
+        for (int k : ids) otherwise[k] = 1;
+      }
+    }
+    // the same memory attached under two ids (tied embedding / LM head) is in use as long as one of them is
+    for (size_t a = 0; a < g->tensors.size(); a++)
+      for (size_t b = 0; b < g->tensors.size(); b++)
+        if (a != b && g->tensors[a].ptr && g->tensors[a].ptr == g->tensors[b].ptr && otherwise[b]) otherwise[a] = 1;
+    for (size_t id = 0; id < g->tensors.size(); id++) {
+      const Tensor &t = g->tensors[id];
+      if (!as_linear_weight[id] || t.kind != T_ATTACHED) continue;
+      if (g->single_copy && !otherwise[id]) g->releasable[id] = 1;
+      else g->row_major_bytes += (int64_t)t.elems() * (int64_t)dtype_size(t.dtype);
+    }
+  }
   if ((rc = dev_alloc(g, &p, sizeof(MkStage) * (g->stages.size() + 1)))) return rc;
   g->d_stages = (MkStage *)p;
   rt.stages = g->d_stages;
@@ -1920,6 +1983,7 @@ int mk_get_stats(mk_graph *g, mk_stats *out) {
   out->aborted = g->last_aborted;
   out->weight_bytes = g->weight_bytes;
   out->packed_weight_bytes = g->packed_bytes;
+  out->row_major_weight_bytes = g->row_major_bytes;
   out->last_launch_ms = g->last_ms;
   if (g->compiled && !g->launch_pending) {
     MkSched sc;

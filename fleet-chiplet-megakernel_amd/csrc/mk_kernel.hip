@@ -3827,8 +3827,11 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
     for (int s = 0; s < rt.num_stages && !c.dead; s++) {
       CStage &st = ((CStage *)(unsigned long long)rt.stages)[s];
       const int op = st.op, flags = st.flags;
-      if ((flags & MK_F_ONLY_MULTI) && M == 1) continue;
-      if ((flags & MK_F_ONLY_MULTI) && op == MK_OP_NORM && s + 1 < rt.num_stages) {
+      // (a handle that holds only the matrix-core copies of its weights runs every linear in a matrix-core form, which
+      // reads normalised rows from the NORM stage's output: that stage then runs for one and two tokens as well)
+      const bool packed_only = MAXM > 1 && rt.packed_only;
+      if ((flags & MK_F_ONLY_MULTI) && M == 1 && !(packed_only && op == MK_OP_NORM)) continue;
+      if ((flags & MK_F_ONLY_MULTI) && op == MK_OP_NORM && s + 1 < rt.num_stages && !packed_only) {
         // the few-token linear normalises its rows itself
         CStage &nx = ((CStage *)(unsigned long long)rt.stages)[s + 1];
         if (nx.op == MK_OP_LINEAR && (nx.flags & MK_F_NORM) && nx.in == st.in && linear_small_ok(nx, c, M)) continue;
@@ -3839,8 +3842,8 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
         case MK_OP_NORM: stage_norm(st, c, M, smem); break;
         case MK_OP_LINEAR:
           if constexpr (MAXM == 1) stage_linear_m1<true>(st, c, smem);
-          else if (M == 1) stage_linear_m1<false>(st, c, smem);
-          else if (linear_small_ok(st, c, M)) {
+          else if (M == 1 && !(packed_only && st.wpack)) stage_linear_m1<false>(st, c, smem);
+          else if (linear_small_ok(st, c, M) && !(packed_only && st.wpack)) {
             if (M <= 2) stage_linear_small_dispatch<2>(st, c, M, smem);
             else if (M <= 4) stage_linear_small_dispatch<4>(st, c, M, smem);
             else stage_linear_small_dispatch<8>(st, c, M, smem);
@@ -3849,7 +3852,7 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
             const bool narrow = ((wt + c.G - 1) / c.G) * ((flags & MK_F_SILU) ? 2 : 1) <= 2;
             const TilePlan plan = linear_tiles_plan(st, c);
             const XresPlan xp = linear_xres_plan(st, c);
-            if (xp.S >= 1 && M > MK_TUNE_SMALL_MAX) {
+            if (xp.S >= 1 && (M > MK_TUNE_SMALL_MAX || packed_only)) {
               if (M <= 32) {
                 if (xp.tpu <= 4) stage_linear_mfma_xres<2, 2>(st, c, rt, M, xp, smem);
                 else stage_linear_mfma_xres<2, 3>(st, c, rt, M, xp, smem);
@@ -3857,7 +3860,7 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
                 if (xp.tpu <= 4) stage_linear_mfma_xres<4, 2>(st, c, rt, M, xp, smem);
                 else stage_linear_mfma_xres<4, 3>(st, c, rt, M, xp, smem);
               }
-            } else if (plan.S >= 1) {
+            } else if (plan.S >= 1 && !(packed_only && st.wpack)) {  // (this form reads the row-major weights)
               if (M <= 16) stage_linear_mfma_tiles<1>(st, c, rt, M, plan, smem);
               else if (M <= 32) stage_linear_mfma_tiles<2>(st, c, rt, M, plan, smem);
               else if (M <= 48) stage_linear_mfma_tiles<3>(st, c, rt, M, plan, smem);

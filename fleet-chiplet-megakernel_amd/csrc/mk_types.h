@@ -197,7 +197,8 @@ struct MkRuntime {
   void *splitk_part;    // [workgroups][4 wavefronts][4 weight tiles][4 token tiles][64 lanes] f32x4: K-slice partials of the split-K linear
   unsigned *splitk_cnt; // [workgroups][32]: arrival counter per split-K group (one 128-byte line each)
   long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end
-  int timing_cap, pad0;
+  int timing_cap;
+  int packed_only;       // the handle keeps ONLY the matrix-core copies of its linear weights: iterations of one or two tokens run the matrix-core forms too
   long long *stage_prof; // [workgroups][num_stages + 1][MK_PROF_TICKS] 100 MHz ticks of the last iteration: entry, wait done, exit, arrived, then
                          // four marks a stage may set in a build with MK_TRACE defined; the extra record holds the scheduler step:
                          // [0] previous iteration complete, [1] batch prepared, [2] batch published to every workgroup

@@ -109,7 +109,8 @@ class Qwen3Decoder:
     def __init__(self, shape: Qwen3Shape, weights: dict, max_num_batched_tokens: int = 1, max_num_batched_requests: int = None,
                  max_seq_length: int = 1200, page_size: int = 4096, max_num_pages: int = None, total_requests: int = None,
                  mode: str = "fleet", eos_token_id: int = 0x7FFFFFFF, cos_sin=None, device="cuda", num_workers=None, with_head: bool = True,
-                 kernel_mode: str = "offline", max_tokens_per_request: int = None, tap_last_layer_input: bool = False):
+                 kernel_mode: str = "offline", max_tokens_per_request: int = None, tap_last_layer_input: bool = False,
+                 single_weight_copy: bool = None):
         assert mode in ("fleet", "mpk")
         self.shape, self.w, self.mode = shape, weights, mode
         self.with_head = with_head
@@ -144,7 +145,8 @@ class Qwen3Decoder:
             mode=kernel_mode, world_size=1, mpi_rank=0, num_workers=num_workers, num_local_schedulers=0, num_remote_schedulers=0,
             max_seq_length=max_seq_length, max_num_batched_requests=R, max_num_batched_tokens=B, max_num_pages=self.max_pages,
             page_size=page_size, eos_token_id=eos_token_id, meta_tensors=self.meta, profiler_tensor=None, trace_name=None,
-            spec_decode_config=None, use_cutlass_kernel=False, max_tokens_per_request=max_tokens_per_request)
+            spec_decode_config=None, use_cutlass_kernel=False, max_tokens_per_request=max_tokens_per_request,
+            single_weight_copy=single_weight_copy)
         n_pos = max(max_seq_length, 16)
         self.cos, self.sin = cos_sin if cos_sin is not None else rope_tables(shape, n_pos, dev)
         L = shape.num_layers

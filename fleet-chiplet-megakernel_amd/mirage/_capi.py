@@ -18,6 +18,7 @@ MK_ESTATE = -3
 MK_EABORT = -4
 MK_EUNSUPPORTED = -5
 
+MK_CFG_SINGLE_WEIGHT_COPY = 1
 MK_MODES = {"offline": 0, "online": 1, "online_notoken": 2, "onepass": 3}
 
 # symbols include/fleet_mk.h declares; tests check that the library exports every one
@@ -25,7 +26,7 @@ EXPORTED_SYMBOLS = [
     "mk_graph_create", "mk_graph_destroy", "mk_tensor_attach", "mk_tensor_new", "mk_tensor_shuffle",
     "mk_tensor_num_dims", "mk_tensor_dim", "mk_tensor_ptr", "mk_add_task", "mk_generate_task_graph",
     "mk_compile", "mk_init_requests", "mk_launch", "mk_launch_steps", "mk_enqueue_steps", "mk_enqueue_steps_static", "mk_wait",
-    "mk_run_once", "mk_repack_weights", "mk_get_stats", "mk_get_stage_profile", "mk_get_stage_marks", "mk_describe_program", "mk_last_error", "mk_version",
+    "mk_run_once", "mk_repack_weights", "mk_tensor_releasable", "mk_get_stats", "mk_get_stage_profile", "mk_get_stage_marks", "mk_describe_program", "mk_last_error", "mk_version",
 ]
 
 
@@ -43,7 +44,7 @@ class MkConfig(ctypes.Structure):
         ("rms_eps", ctypes.c_float),
         ("mode", ctypes.c_int),
         ("max_tokens_per_request", ctypes.c_int),
-        ("reserved0", ctypes.c_int),
+        ("flags", ctypes.c_int),
         ("step", ctypes.c_void_p),
         ("tokens", ctypes.c_void_p),
         ("input_tokens", ctypes.c_void_p),
@@ -69,6 +70,7 @@ class MkStats(ctypes.Structure):
         ("weight_bytes", ctypes.c_int64),
         ("last_launch_ms", ctypes.c_double),
         ("packed_weight_bytes", ctypes.c_int64),
+        ("row_major_weight_bytes", ctypes.c_int64),
     ]
 
 
@@ -118,6 +120,7 @@ def load():
     lib.mk_get_stats.argtypes = [vp, ctypes.POINTER(MkStats)]
     lib.mk_get_stage_profile.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_int64), ci]
     lib.mk_repack_weights.argtypes = [vp]
+    lib.mk_tensor_releasable.argtypes = [vp, ci]
     lib.mk_get_stage_marks.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_int64), ci]
     lib.mk_describe_program.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p)]
     lib.mk_last_error.restype = ctypes.c_char_p

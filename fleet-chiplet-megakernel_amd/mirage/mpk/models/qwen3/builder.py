@@ -41,7 +41,8 @@ class Qwen3Builder(GraphBuilder):
         self.rank = mpk.mpi_rank
         self.eos_token_id = 151645  # default eos token id for Qwen3 (builder.py:27)
         self.returned_hidden_state = None
-        self._keep = []  # torch tensors the graph points at
+        self._keep = []
+        self._kept_as = {}  # torch tensors the graph points at
 
     # ------------------------------------------------------------------ entry points
     def build_from_config(self, model_config: MirageModelConfig):
@@ -97,7 +98,15 @@ class Qwen3Builder(GraphBuilder):
     # ------------------------------------------------------------------ tensors
     def _attach(self, t: torch.Tensor, name: str):
         self._keep.append(t)
+        self._kept_as[name] = t
         return self.mpk.attach_input(torch_tensor=t, name=name)
+
+    def release_weights(self, names):
+        """Drop this builder's references to the attached tensors `names` (those the compiled kernel no longer reads: a
+        graph built with single_weight_copy keeps its linear weights in tile order only)."""
+        gone = [self._kept_as.pop(n) for n in names if n in self._kept_as]
+        self._keep = [t for t in self._keep if not any(t is g for g in gone)]
+        return len(gone)
 
     def new_intermediate_tensors(self):
         """Activations of one iteration.  In online_notoken mode they are torch tensors the caller can read back (the

@@ -66,6 +66,7 @@ class MPKMetadata:
     use_cutlass_kernel: bool = False
     eos_token_id: Optional[int] = None
     max_tokens_per_request: Optional[int] = None
+    single_weight_copy: Optional[bool] = None  # keep every linear weight once, in tile order (see PersistentKernel)
 
     def check_valid(self):
         if self.weight_from_model:
@@ -142,7 +143,7 @@ class MPK:
                 "paged_kv_last_page_len_buffer": self.paged_kv_last_page_len_buffer},
             profiler_tensor=meta.profiler_tensor, trace_name=meta.trace_name, spec_decode_config=meta.spec_decode_config,
             use_cutlass_kernel=False, eos_token_id=meta.eos_token_id if meta.eos_token_id is not None else 151645,
-            max_tokens_per_request=meta.max_tokens_per_request)
+            max_tokens_per_request=meta.max_tokens_per_request, single_weight_copy=meta.single_weight_copy)
         self.is_built = self.task_graph_generated = self.is_compiled = False
 
     def compensate_meta_tensors(self):
@@ -243,6 +244,10 @@ class MPK:
             raise ValueError("Model is not built yet")
         self.persistent_kernel.compile(output_dir=output_dir)
         self.is_compiled = True
+        if self.persistent_kernel.single_weight_copy:
+            # the row-major tensors of the linears now exist in tile order inside the library: drop them here and in the
+            # builder (a state dict the caller still holds keeps its tensors alive until the caller lets go)
+            self.model_builder.release_weights(self.persistent_kernel.release_row_major_weights())
 
     def __call__(self, **kwargs):
         if not self.is_compiled:

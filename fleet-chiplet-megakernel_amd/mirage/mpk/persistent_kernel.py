@@ -46,10 +46,14 @@ class PersistentKernel:
         use_cutlass_kernel: bool = False,
         eos_token_id: int = -1,
         max_tokens_per_request: int = None,
+        single_weight_copy: bool = None,
     ):
         """Arguments as the reference constructor (persistent_kernel.py:368-387).  `max_tokens_per_request` is the
         reference's compile-time MPK_MAX_TOKENS_PER_REQUEST (prompt tokens one request ingests per iteration; 8 on AMD,
-        persistent_kernel.cuh:115-124): None takes the environment variable of that name, else 8; at most 64."""
+        persistent_kernel.cuh:115-124): None takes the environment variable of that name, else 8; at most 64.
+        `single_weight_copy` (no counterpart in the reference; None takes FLEET_MK_SINGLE_WEIGHT_COPY, else False): a graph
+        with max_num_batched_tokens >= 2 then keeps every linear weight ONCE, in the matrix-core tile layout compile()
+        makes; `release_row_major_weights()` afterwards drops the attached tensors nothing reads any more."""
         self.__finalized__ = False
         self._is_compiled = False
         self._handle = None
@@ -124,6 +128,10 @@ class PersistentKernel:
         cfg.rms_eps = 1e-6
         cfg.mode = _capi.MK_MODES[mode]
         cfg.max_tokens_per_request = self.max_tokens_per_request
+        if single_weight_copy is None:
+            single_weight_copy = os.environ.get("FLEET_MK_SINGLE_WEIGHT_COPY", "0") not in ("", "0")
+        self.single_weight_copy = bool(single_weight_copy)
+        cfg.flags = _capi.MK_CFG_SINGLE_WEIGHT_COPY if self.single_weight_copy else 0
         cfg.step = mt["step"].data_ptr()
         cfg.tokens = mt["tokens"].data_ptr()
         cfg.input_tokens = mt["input_tokens"].data_ptr()
@@ -813,6 +821,18 @@ class PersistentKernel:
         (graphs with max_num_batched_tokens > 8 stream a tile-ordered copy made at compile time).  Not in the reference,
         whose kernels read the attached tensors in place."""
         _capi.check(self._lib.mk_repack_weights(self._handle))
+
+    def release_row_major_weights(self) -> list:
+        """After compile() of a graph built with single_weight_copy: drop this object's references to the attached weight
+        tensors the kernel will never read again (each now lives in its tile copy only) and return their names, so that a
+        caller who drops its own references as well gets the memory back.  Without single_weight_copy nothing is released."""
+        assert self._is_compiled, "compile() first"
+        released = []
+        for t in self._tensors:
+            if t.torch_tensor is not None and _capi.check(self._lib.mk_tensor_releasable(self._handle, t.id)) == 1:
+                released.append(t.name)
+                t.torch_tensor = None
+        return released
 
     def stats(self) -> dict:
         st = _capi.MkStats()

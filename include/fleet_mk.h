@@ -52,6 +52,16 @@ enum mk_io_category { MK_IO_DEVICE = 0 /* "cuda_tensor" */, MK_IO_SYMMETRIC = 1 
  *  MK_MODE_ONEPASS         the same single pass (the reference compiles its test graphs in this mode). */
 enum mk_mode { MK_MODE_OFFLINE = 0, MK_MODE_ONLINE = 1, MK_MODE_ONLINE_NOTOKEN = 2, MK_MODE_ONEPASS = 3 };
 
+/* mk_config.flags.  No counterpart in the reference (its kernels read the attached weights in place and its drivers keep an
+ * interleaved second copy of the QKV and gate/up weights, src/kernel/runtime.cc:904-943).
+ *  MK_CFG_SINGLE_WEIGHT_COPY  a graph with max_num_batched_tokens >= 2 normally holds every linear weight twice -- the
+ *      caller's row-major tensor (streamed by iterations of one or two tokens) and a matrix-core tile copy (streamed by larger
+ *      iterations).  With this flag the tile copy is the ONLY one the handle reads after mk_compile: iterations of one and
+ *      two tokens run the matrix-core forms as well (a single-token iteration then costs about what a four-token one
+ *      does), and every tensor for which mk_tensor_releasable() returns 1 may be freed by the caller.  mk_compile fails
+ *      with MK_EUNSUPPORTED if a linear weight cannot be tiled (reduction length not a multiple of 256). */
+enum mk_config_flags { MK_CFG_SINGLE_WEIGHT_COPY = 1 };
+
 /* Constructor arguments of PersistentKernel (persistent_kernel.py:368-387) plus the
  * ten meta tensors in the order the reference hands them to init_func
  * (persistent_kernel.py:2590-2600).  All meta pointers are device pointers. */
@@ -70,7 +80,7 @@ typedef struct mk_config {
   int mode;                     /* enum mk_mode: who prepares the batch of an iteration */
   int max_tokens_per_request;   /* prompt tokens one request may ingest per iteration; 0 => 8, the reference's default for
                                    AMD (MPK_MAX_TOKENS_PER_REQUEST, persistent_kernel.cuh:115-124); at most 64 */
-  int reserved0;
+  int flags;                    /* enum mk_config_flags, or'ed */
   int32_t *step;                /* [total_num_requests] */
   int64_t *tokens;              /* [total_num_requests, max_seq_length] */
   int64_t *input_tokens;        /* [max_num_batched_tokens] */
@@ -155,6 +165,11 @@ int mk_enqueue_steps_static(mk_graph *g, void *stream, int max_iterations);
  * tensors).  A caller that overwrites attached weights after mk_compile calls this to refresh the copies.  Blocking.
  * The environment variable FLEET_MK_PACK_WEIGHTS=0 (read by mk_compile) runs without copies. */
 int mk_repack_weights(mk_graph *g);
+/* After mk_compile of a graph created with MK_CFG_SINGLE_WEIGHT_COPY: 1 if attached tensor `id` is never read again by this
+ * handle (it is a linear weight, or a source of a shuffled linear weight, that now lives in its tile copy and is used by
+ * nothing else), 0 if it must stay alive, negative status on a bad id.  Always 0 without the flag.  A released tensor makes
+ * mk_repack_weights fail with MK_ESTATE. */
+int mk_tensor_releasable(mk_graph *g, int id);
 /* Host-driven single pass (the reference's MODE_ONEPASS / online modes, persistent_kernel.cuh:538-582): the caller
  * supplies the batch -- for each of `num_tokens` rows its batch slot, absolute position and the index of the first
  * row of the same request -- and has filled input_tokens / paged_kv_* itself.  Runs the stage program once. */
@@ -173,6 +188,8 @@ typedef struct mk_stats {
   int64_t weight_bytes;    /* bytes of weight matrices streamed by one iteration */
   double last_launch_ms;   /* HIP-event time of the last launch's kernel, on the stream it ran on */
   int64_t packed_weight_bytes; /* device memory the handle holds for matrix-core copies of the weights (0: none) */
+  int64_t row_major_weight_bytes; /* bytes of attached linear weights the handle still reads in place (0 with
+                                     MK_CFG_SINGLE_WEIGHT_COPY: every linear weight lives in its tile copy only) */
 } mk_stats;
 int mk_get_stats(mk_graph *g, mk_stats *out);
 /* Device-side stage timing of the LAST decode iteration, as seen by virtual workgroup `workgroup`: for each stage four

@@ -84,6 +84,66 @@ def test_builder_task_sequence_lowers_on_the_host():
     mpk.finalize()
 
 
+def _write_checkpoint(ck, cfg, w, tokenizer=False):
+    from safetensors.torch import save_file
+    ck.mkdir()
+    save_file({k: v.cpu().contiguous() for k, v in _state_dict(w, "cpu").items()}, str(ck / "model.safetensors"))
+    (ck / "config.json").write_text(json.dumps({
+        "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
+        "num_attention_heads": cfg.num_q_heads, "num_key_value_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
+        "num_hidden_layers": cfg.num_layers, "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_eps, "tie_word_embeddings": False,
+        "eos_token_id": 0x7FFFFFF0}))
+    if tokenizer:
+        # a hand-written word-level tokenizer with the two chat markers as special tokens and a chat template of the Qwen kind
+        from tokenizers import Tokenizer, models, pre_tokenizers
+        words = ["<unk>", "<|im_start|>", "<|im_end|>", "system", "user", "assistant", "You", "are", "Qwen", ",", "created", "by", "Alibaba", "Cloud", ".",
+                 "a", "helpful", "hello", "world", "decode", "me"]
+        tok = Tokenizer(models.WordLevel(vocab={wd: i for i, wd in enumerate(words)}, unk_token="<unk>"))
+        tok.pre_tokenizer = pre_tokenizers.Whitespace()
+        tok.add_special_tokens(["<|im_start|>", "<|im_end|>"])
+        tok.save(str(ck / "tokenizer.json"))
+        (ck / "tokenizer_config.json").write_text(json.dumps({
+            "tokenizer_class": "PreTrainedTokenizerFast", "unk_token": "<unk>", "eos_token": "<|im_end|>",
+            "chat_template": "{% for m in messages %}<|im_start|> {{ m['role'] }} {{ m['content'] }} <|im_end|> {% endfor %}"
+                             "{% if add_generation_prompt %}<|im_start|> assistant {% endif %}"}))
+        return words
+
+
+def test_checkpoint_with_tokenizer_load_new_request_and_decode(tmp_path):
+    """No GPU: a local checkpoint directory WITH tokenizer files -- the string path of load_new_request (chat template, system
+    prompt, generation marker: python/mirage/mpk/mpk.py:281-307) and decode().  Skipped if `transformers` cannot load a local
+    tokenizer.json offline."""
+    from mirage.mpk import MPK
+    from oracle.qwen3_ref import make_model_weights
+    cfg = _cfg(layers=1, vocab=256)
+    w = make_model_weights(cfg, seed=65)
+    ck = tmp_path / "qwen3-tiny-tok"
+    words = _write_checkpoint(ck, cfg, w, tokenizer=True)
+    try:
+        from transformers import AutoTokenizer
+        AutoTokenizer.from_pretrained(str(ck), local_files_only=True)
+    except Exception as e:  # pragma: no cover
+        pytest.skip(f"transformers cannot load a local tokenizer here: {e}")
+    mpk = MPK(_metadata(cfg, w, "cpu", R=2, T=4, total=2, max_seq=64, PS=16, from_path=str(ck), num_workers=256))
+    with pytest.raises(ValueError, match="not built"):
+        mpk.load_new_request("hello world")
+    mpk.build()
+    assert mpk.tokenizer is not None
+    ident = {wd: i for i, wd in enumerate(words)}
+    mpk.load_new_request("hello world")  # with the chat template
+    sys_text = "You are Qwen , created by Alibaba Cloud . You are a helpful assistant ."
+    want = [ident[t] for t in ("<|im_start|> system " + sys_text + " <|im_end|> <|im_start|> user hello world <|im_end|> <|im_start|> assistant").split()]
+    L = int(mpk.prompt_lengths[0])
+    assert L == len(want) and mpk.prompt_lengths.tolist() == [L, L]
+    assert mpk.tokens[0, :L].tolist() == want and mpk.tokens[1, :L].tolist() == want and int(mpk.tokens[0, L:].abs().sum()) == 0
+    mpk.load_new_request("decode me", use_template=False)
+    assert mpk.tokens[0, :int(mpk.prompt_lengths[0])].tolist() == [ident["decode"], ident["me"]]
+    assert mpk.decode(torch.tensor([ident["hello"], ident["world"], ident["<|im_end|>"]])) == "hello world"
+    mpk.load_new_request([5, 6, 7])  # token ids still work
+    assert mpk.tokens[1, :3].tolist() == [5, 6, 7] and mpk.prompt_lengths.tolist() == [3, 3]
+    mpk.finalize()
+
+
 @pytest.mark.gpu
 def test_mpk_offline_generation_matches_layer_api_driver_and_oracle(tmp_path):
     from mirage.mpk import MPK
@@ -113,15 +173,8 @@ def test_mpk_offline_generation_matches_layer_api_driver_and_oracle(tmp_path):
     assert mpk.persistent_kernel.stats()["aborted"] == 0
     mpk.finalize()
     # a local checkpoint directory: config.json + model.safetensors under the checkpoint's names
-    from safetensors.torch import save_file
     ck = tmp_path / "qwen3-tiny"
-    ck.mkdir()
-    save_file({k: v.cpu().contiguous() for k, v in _state_dict(w, "cpu").items()}, str(ck / "model.safetensors"))
-    (ck / "config.json").write_text(json.dumps({
-        "hidden_size": cfg.hidden_size, "intermediate_size": cfg.intermediate_size, "vocab_size": cfg.vocab_size,
-        "num_attention_heads": cfg.num_q_heads, "num_key_value_heads": cfg.num_kv_heads, "head_dim": cfg.head_dim,
-        "num_hidden_layers": cfg.num_layers, "rope_theta": cfg.rope_theta, "rms_norm_eps": cfg.rms_eps, "tie_word_embeddings": False,
-        "eos_token_id": 0x7FFFFFF0}))
+    _write_checkpoint(ck, cfg, w)
     mpk2 = MPK(_metadata(cfg, w, "cuda", R=R, T=T, total=total, max_seq=max_seq, PS=PS, from_path=str(ck)))
     mpk2.build()
     assert mpk2.tokenizer is None  # no tokenizer files in the directory: token ids in, token ids out

@@ -8,7 +8,7 @@ from helpers import check_layer_stages as _check
 pytestmark = pytest.mark.gpu
 
 
-def _run_layer(cfg, L_cached, n_new, mode, seed=0, norm_std=0.02, mutate=None):
+def _run_layer(cfg, L_cached, n_new, mode, seed=0, norm_std=0.02, mutate=None, batch_tokens=None, single_weight_copy=None):
     """One request with L_cached positions already in the KV cache and n_new new tokens in this pass."""
     from demo_qwen3 import Qwen3Decoder, Qwen3Shape
     from oracle.qwen3_ref import KVCache, Qwen3Oracle, make_layer_weights, rope_tables
@@ -30,9 +30,14 @@ def _run_layer(cfg, L_cached, n_new, mode, seed=0, norm_std=0.02, mutate=None):
     cos, sin = rope_tables(cfg, max(max_seq, 16))
     page_size = 64
     n_pages = (max_seq + page_size - 1) // page_size
-    dec = Qwen3Decoder(shape, w, max_num_batched_tokens=max(n_new, 1), max_num_batched_requests=1, max_seq_length=max_seq,
+    dec = Qwen3Decoder(shape, w, max_num_batched_tokens=batch_tokens or max(n_new, 1), max_num_batched_requests=1, max_seq_length=max_seq, single_weight_copy=single_weight_copy,
                        page_size=page_size, max_num_pages=n_pages + 3, mode=mode, cos_sin=(cos.to(dev), sin.to(dev)), with_head=False,
                        max_tokens_per_request=max(8, n_new))
+    if single_weight_copy:
+        released = dec.mpk.release_row_major_weights()
+        assert len(released) == 7  # q, k, v, o, gate, up, down (the zero LM head of this one-layer graph is not lowered)
+        for k in ("q_proj", "k_proj", "v_proj", "o_proj", "gate_proj", "up_proj", "down_proj"):
+            w["layers"][0][k].fill_(float("nan"))  # whoever still reads the row-major tensors will show it
     # scatter the cached positions over non-trivially ordered pages: request slot 0 owns pages [n_pages+2, n_pages+1, ... ]
     pages = list(range(n_pages + 2, 2, -1))[:n_pages]
     dec.meta["paged_kv_indptr_buffer"].copy_(torch.tensor([0, n_pages], dtype=torch.int32))
@@ -47,7 +52,7 @@ def _run_layer(cfg, L_cached, n_new, mode, seed=0, norm_std=0.02, mutate=None):
     dec.v_cache[0].copy_(vc)
     # run only the layer's stages: feed hidden through the embedding table trick (ids pick rows of a table = hidden)
     dec.w["embed"][:n_new].copy_(hidden.to(dev))
-    dec.meta["input_tokens"].copy_(torch.arange(n_new, dtype=torch.int64).view(-1, 1))
+    dec.meta["input_tokens"][:n_new].copy_(torch.arange(n_new, dtype=torch.int64).view(-1, 1))
     torch.cuda.synchronize()
     dec.mpk.run_once([0] * n_new, list(range(L_cached, L_cached + n_new)))
     out_gpu = dec.t["hidden_out"].to_torch()[:n_new].cpu()
