@@ -122,6 +122,8 @@ struct mk_graph {
   std::vector<int> stage_weight;      // per stage: tensor id of a LINEAR stage's weight operand (-1: none)
   std::vector<char> releasable;       // per tensor (single-weight-copy graphs, after mk_compile): the handle never reads it again
   bool single_copy = false;
+  void *profiler_ptr = nullptr;  // the caller's profiler tensor (mk_set_profiler)
+  long long profiler_cap = 0;
   int64_t row_major_bytes = 0;
 };
 
@@ -1001,6 +1003,21 @@ int lower(mk_graph *g) {
     }
   }
   g->stage_weight.resize(g->stages.size(), -1);
+  for (auto &st : g->stages) {  // the task type a stage is shown as in a profiler trace (runtime_header.h:91-188)
+    switch (st.op) {
+      case MK_OP_EMBED: st.prof_event = 101; break;
+      case MK_OP_NORM: st.prof_event = 119; break;
+      case MK_OP_LINEAR: st.prof_event = (st.flags & MK_F_NORM) ? 102 : ((st.flags & MK_F_RES) ? 108 : 120); break;
+      case MK_OP_SILU_MUL: st.prof_event = 118; break;
+      case MK_OP_ATTN: st.prof_event = 116; break;
+      case MK_OP_ARGMAX_PARTIAL: st.prof_event = 110; break;
+      case MK_OP_ARGMAX_REDUCE: st.prof_event = 111; break;
+      case MK_OP_MOE_TOPK: st.prof_event = 172; break;
+      case MK_OP_MOE_LINEAR: st.prof_event = (st.flags & MK_F_MOE_COMBINE) || st.ld_in_slot ? 171 : 170; break;
+      case MK_OP_MOE_COMBINE: st.prof_event = 173; break;
+      default: st.prof_event = 121; break;
+    }
+  }
   g->program_text.clear();
   for (size_t s = 0; s < g->stage_desc.size(); s++) g->program_text += fmt("%3zu ", s) + g->stage_desc[s] + "\n";
   return MK_OK;
@@ -1851,6 +1868,10 @@ int mk_compile(mk_graph *g) {
   rt.timing_cap = g->timing_cap;
   if ((rc = dev_alloc(g, &p, sizeof(long long) * MK_PROF_TICKS * (g->stages.size() + 1) * g->G))) return rc;
   rt.stage_prof = (long long *)p;
+  if ((rc = dev_alloc(g, &p, sizeof(unsigned) * (size_t)g->G))) return rc;
+  rt.profiler_count = (unsigned *)p;
+  rt.profiler = (unsigned long long *)g->profiler_ptr;
+  rt.profiler_cap = g->profiler_cap;
   if ((rc = dev_alloc(g, &p, sizeof(MkRuntime)))) return rc;
   g->d_rt = (MkRuntime *)p;
   if ((rc = upload_runtime(g))) return rc;
@@ -1881,6 +1902,25 @@ int mk_init_requests(mk_graph *g) {
   HIP_TRY(hipMemcpy(g->d_sched, &sc, sizeof(sc), hipMemcpyHostToDevice));
   HIP_TRY(hipMemset(rt.attn_cnt, 0, sizeof(unsigned) * g->attn_cnt_n));
   HIP_TRY(hipMemset(rt.splitk_cnt, 0, sizeof(unsigned) * 32 * (size_t)g->G));
+  HIP_TRY(hipMemset(rt.profiler_count, 0, sizeof(unsigned) * (size_t)g->G));
+  if (rt.profiler) HIP_TRY(hipMemset(rt.profiler, 0, sizeof(unsigned long long) * (size_t)rt.profiler_cap));
+  return MK_OK;
+}
+
+int mk_set_profiler(mk_graph *g, void *device_u64, int64_t num_entries) {
+  if (!g) return fail(MK_EINVAL, "null argument");
+  if (g->launch_pending) return fail(MK_ESTATE, "a launch is still pending");
+  if (device_u64 && num_entries < 2) return fail(MK_EINVAL, "a profiler tensor needs at least two entries");
+  g->profiler_ptr = device_u64;
+  g->profiler_cap = device_u64 ? num_entries : 0;
+  if (g->compiled) {
+    HIP_TRY(hipSetDevice(g->cfg.device));
+    g->h_rt.profiler = (unsigned long long *)device_u64;
+    g->h_rt.profiler_cap = g->profiler_cap;
+    HIP_TRY(hipMemset(g->h_rt.profiler_count, 0, sizeof(unsigned) * (size_t)g->G));
+    if (device_u64) HIP_TRY(hipMemset(device_u64, 0, sizeof(unsigned long long) * (size_t)num_entries));
+    return upload_runtime(g);
+  }
   return MK_OK;
 }
 

@@ -84,6 +84,7 @@ struct Ctx {
   int *sh_ticket;     // two LDS work counters, used alternately by consecutive executed stages; [2] = seq of the single-token
                       // MoE stage that last filled the workgroup's expert list (kept outside the stages' scratch LDS)
   int seq;            // stages executed so far by this workgroup
+  unsigned prof_n;    // entries this workgroup has written into the caller's profiler tensor
   bool wrote_through; // the stage that just ran wrote all its outputs with write-through stores: no L2 write-back at its barrier
   bool arrive_w0;     // ... and all of them from wavefront 0, after a workgroup barrier, having reset the next stage's work
                       // counter itself: the arrival then needs no workgroup barrier of its own (see barrier_arrive)
@@ -3908,6 +3909,16 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
       }
       const long long t_out = (long long)wall_clock64();
       barrier_arrive(c);
+      if (threadIdx.x == 0 && rt.profiler) {
+        // begin = this stage's inputs were complete (the previous stage's barrier seen), end = its outputs were posted
+        const long long at = 1 + c.vid + (long long)c.prof_n * c.G;
+        if (at + c.G < rt.profiler_cap) {
+          const unsigned tag = ((unsigned)(c.seq & 0x1FFF) << 19) | ((unsigned)(c.vid & 0xFF) << 11) | ((unsigned)(st.prof_event & 0x1FF) << 2);
+          rt.profiler[at] = (unsigned long long)tag | (((unsigned long long)(c.t_wait * 10) & 0xFFFFFFFFull) << 32);
+          rt.profiler[at + c.G] = (unsigned long long)(tag | 1u) | (((unsigned long long)((long long)wall_clock64() * 10) & 0xFFFFFFFFull) << 32);
+          c.prof_n += 2;
+        }
+      }
       if (threadIdx.x == 0 && rt.stage_prof) {
         long long *pr = rt.stage_prof + MK_PROF_TICKS * ((size_t)c.vid * (rt.num_stages + 1) + s);
         pr[0] = t_in;
@@ -3948,6 +3959,7 @@ __device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRunt
   c.sh_tok = &sh_tok[0][0];
   c.sh_ticket = sh_ticket;
   c.seq = 0;
+  c.prof_n = 0;
   c.defer_S = 0;
   c.wrote_through = false;
   c.arrive_w0 = false;
@@ -3993,6 +4005,10 @@ __device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRunt
   c.even_xcds = true;
   for (int i = 0; i < 8; i++) c.even_xcds = c.even_xcds && (c.quotas[i] == 0 || c.quotas[i] == (unsigned)c.quota);
   __syncthreads();
+  if (rt.profiler) {
+    c.prof_n = (unsigned)__builtin_amdgcn_readfirstlane((int)ldc_u32(&rt.profiler_count[c.vid]));
+    if (c.vid == 0 && threadIdx.x == 0) rt.profiler[0] = (unsigned long long)(unsigned)c.G | (1ull << 32);
+  }
 
   for (int it = 0; it < max_iters && !c.dead; it++) {
     // ---- scheduler step on one thread of virtual workgroup 0, published through the barrier
@@ -4046,6 +4062,7 @@ __device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRunt
     run_stage_program<MAXM>(rt, c, MAXM == 1 ? 1 : M, smem);
   }
   barrier_wait(c);  // drain: nobody leaves while another workgroup may still poll
+  if (rt.profiler && threadIdx.x == 0) rt.profiler_count[c.vid] = c.prof_n;
   if (c.vid == 0 && threadIdx.x == 0 && rt.timing) rt.timing[0] = (long long)wall_clock64();
 }
 

@@ -103,7 +103,7 @@ struct MkStage {
   int num_q_heads, num_kv_heads, head_dim, ld_qws;
   int ld_cos, ld_norm;  // ld_norm: leading dimension of norm_out
   float sm_scale_log2;  // log2(e) / sqrt(head_dim)
-  int pad3;
+  int prof_event;       // the reference's task-type number this stage is recorded under in a caller's profiler tensor
   // argmax
   void *aux0, *aux1;
   // mixture of experts.  MOE_LINEAR: x(t,slot) = in + t*ld_in + slot*ld_in_slot, expert e's weights are rows
@@ -199,6 +199,13 @@ struct MkRuntime {
   long long *timing;    // [1 + timing_cap] wall-clock ticks (100 MHz) at the start of each iteration; [0] = kernel end
   int timing_cap;
   int packed_only;       // the handle keeps ONLY the matrix-core copies of its linear weights: iterations of one or two tokens run the matrix-core forms too
+  // A caller's profiler tensor (null: none): (tag, time) entries of EVERY executed stage of every iteration, in the
+  // reference's layout (include/mirage/persistent_kernel/profiler.h:129-180): entry 0 = (workgroups, 1); the k-th entry of
+  // workgroup b sits at 1 + b + k * workgroups; low word tag = stage instance << 19 | b << 11 | task type << 2 | (0 begin, 1
+  // end), high word = low 32 bits of the time in ns.  Recording stops when the tensor is full.
+  unsigned long long *profiler;
+  long long profiler_cap;        // entries the tensor holds
+  unsigned *profiler_count;      // [workgroups] entries written so far by each workgroup (kept across launches)
   long long *stage_prof; // [workgroups][num_stages + 1][MK_PROF_TICKS] 100 MHz ticks of the last iteration: entry, wait done, exit, arrived, then
                          // four marks a stage may set in a build with MK_TRACE defined; the extra record holds the scheduler step:
                          // [0] previous iteration complete, [1] batch prepared, [2] batch published to every workgroup

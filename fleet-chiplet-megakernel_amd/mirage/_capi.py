@@ -26,7 +26,7 @@ EXPORTED_SYMBOLS = [
     "mk_graph_create", "mk_graph_destroy", "mk_tensor_attach", "mk_tensor_new", "mk_tensor_shuffle",
     "mk_tensor_num_dims", "mk_tensor_dim", "mk_tensor_ptr", "mk_add_task", "mk_generate_task_graph",
     "mk_compile", "mk_init_requests", "mk_launch", "mk_launch_steps", "mk_enqueue_steps", "mk_enqueue_steps_static", "mk_wait",
-    "mk_run_once", "mk_repack_weights", "mk_tensor_releasable", "mk_get_stats", "mk_get_stage_profile", "mk_get_stage_marks", "mk_describe_program", "mk_last_error", "mk_version",
+    "mk_run_once", "mk_repack_weights", "mk_tensor_releasable", "mk_set_profiler", "mk_get_stats", "mk_get_stage_profile", "mk_get_stage_marks", "mk_describe_program", "mk_last_error", "mk_version",
 ]
 
 
@@ -121,6 +121,7 @@ def load():
     lib.mk_get_stage_profile.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_int64), ci]
     lib.mk_repack_weights.argtypes = [vp]
     lib.mk_tensor_releasable.argtypes = [vp, ci]
+    lib.mk_set_profiler.argtypes = [vp, vp, ctypes.c_int64]
     lib.mk_get_stage_marks.argtypes = [vp, ci, ctypes.POINTER(ctypes.c_int64), ci]
     lib.mk_describe_program.argtypes = [vp, ctypes.POINTER(ctypes.c_char_p)]
     lib.mk_last_error.restype = ctypes.c_char_p

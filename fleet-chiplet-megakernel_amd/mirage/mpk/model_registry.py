@@ -1,21 +1,21 @@
-"""Name -> graph-builder registry (reference: python/mirage/mpk/model_registry.py)."""
+"""Which graph-builder class serves which model name (reference: python/mirage/mpk/model_registry.py)."""
 _MODEL_BUILDERS = {}
 
 
 def register_model_builder(*names):
-    """Class decorator: register a builder under one or several model names."""
-    flat = list(names[0]) if len(names) == 1 and isinstance(names[0], (list, tuple, set)) else list(names)
+    """Class decorator.  Takes the model names one by one or as a single list / tuple / set of them."""
+    if len(names) == 1 and not isinstance(names[0], str):
+        names = tuple(names[0])
 
-    def decorator(cls):
-        for n in flat:
-            _MODEL_BUILDERS[n] = cls
-        return cls
+    def bind(builder_cls):
+        _MODEL_BUILDERS.update(dict.fromkeys(names, builder_cls))
+        return builder_cls
 
-    return decorator
+    return bind
 
 
 def get_builder(name: str):
-    builder = _MODEL_BUILDERS.get(name)
-    if builder is None:
-        raise ValueError(f"Unknown builder: {name}. Registered: {list(_MODEL_BUILDERS.keys())}")
-    return builder
+    try:
+        return _MODEL_BUILDERS[name]
+    except KeyError:
+        raise ValueError(f"no graph builder is registered for model {name!r} (known: {sorted(_MODEL_BUILDERS)})") from None

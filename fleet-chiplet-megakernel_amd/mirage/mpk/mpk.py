@@ -148,36 +148,23 @@ class MPK:
 
     def compensate_meta_tensors(self):
         """Allocate the meta tensors the caller left out (mpk.py:229-267)."""
-        dev, R, B, T = self.device, self.max_num_batched_requests, self.max_num_batched_tokens, self.total_num_requests
-        mk = lambda shape, dt, fill=0: torch.full(shape, fill, dtype=dt, device=dev)
-        if self.step is None:
-            self.step = mk((T,), torch.int32)
-        if self.tokens is None:
-            self.tokens = mk((T, self.max_seq_length), torch.int64)
-        if self.input_tokens is None:
-            self.input_tokens = mk((B, 1), torch.int64)
-        if self.output_tokens is None:
-            self.output_tokens = mk((B, 1), torch.int64)
-        if self.num_new_tokens is None:
-            self.num_new_tokens = mk((T,), torch.int32, 1)
-        if self.prompt_lengths is None:
-            self.prompt_lengths = mk((T,), torch.int32)
-        if self.qo_indptr_buffer is None:
-            self.qo_indptr_buffer = mk((R + 1,), torch.int32)
-        if self.paged_kv_indptr_buffer is None:
-            self.paged_kv_indptr_buffer = mk((R + 1,), torch.int32)
-        if self.paged_kv_indices_buffer is None:
-            self.paged_kv_indices_buffer = mk((self.max_num_pages,), torch.int32)
-        if self.paged_kv_last_page_len_buffer is None:
-            self.paged_kv_last_page_len_buffer = mk((R,), torch.int32)
+        R, B, T = self.max_num_batched_requests, self.max_num_batched_tokens, self.total_num_requests
+        # name -> (shape, dtype, initial value); one new token per request per pass is the reference's default as well
+        layout = {"step": ((T,), torch.int32, 0), "tokens": ((T, self.max_seq_length), torch.int64, 0),
+                  "input_tokens": ((B, 1), torch.int64, 0), "output_tokens": ((B, 1), torch.int64, 0),
+                  "num_new_tokens": ((T,), torch.int32, 1), "prompt_lengths": ((T,), torch.int32, 0),
+                  "qo_indptr_buffer": ((R + 1,), torch.int32, 0), "paged_kv_indptr_buffer": ((R + 1,), torch.int32, 0),
+                  "paged_kv_indices_buffer": ((self.max_num_pages,), torch.int32, 0), "paged_kv_last_page_len_buffer": ((R,), torch.int32, 0)}
+        for name, (shape, dtype, fill) in layout.items():
+            if getattr(self, name) is None:
+                setattr(self, name, torch.full(shape, fill, dtype=dtype, device=self.device))
         self.total_num_requests = self.tokens.shape[0]
 
     # ------------------------------------------------------------------ requests
     def load_new_request(self, prompt, use_template: bool = True):
         """Every request slot gets `prompt` (mpk.py:281-307): a string (needs the checkpoint's tokenizer) or a 1-D sequence
         of token ids."""
-        if not self.is_built:
-            raise ValueError("Model is not built yet, so tokenizer is not available")
+        self._require_built()
         if isinstance(prompt, str):
             if self.tokenizer is None:
                 raise ValueError("no tokenizer was loaded with the model: pass token ids")
@@ -207,41 +194,44 @@ class MPK:
     def run(self, prompt):
         """Offline generation of one prompt in every request slot; returns the decoded text (or the token ids when the
         model came without a tokenizer), mpk.py:336-349."""
-        if not self.is_compiled:
-            self.compile()
+        self._ensure_compiled()
         self.load_new_request(prompt)
-        torch.cuda.synchronize()
+        torch.cuda.synchronize()  # the prompt rows are in place before the request state is reset and the kernel starts
         self.init_per_request()
         self()
         torch.cuda.synchronize()
-        out = []
-        for r in range(self.total_num_requests):
-            ids = self.tokens[r, : int(self.step[r]) + 1]
-            out.append(self.tokenizer.decode(ids, skip_special_tokens=True) if self.tokenizer is not None else ids.cpu())
-        return out
+        rows = [self.tokens[r, : int(n) + 1] for r, n in enumerate(self.step.tolist())]
+        if self.tokenizer is None:
+            return [ids.cpu() for ids in rows]
+        return [self.tokenizer.decode(ids, skip_special_tokens=True) for ids in rows]
 
     # ------------------------------------------------------------------ graph
+    def _require_built(self):
+        if not self.is_built:
+            raise ValueError("the model graph is not built yet: call build() first")
+
+    def _ensure_compiled(self):
+        if not self.is_compiled:
+            self.compile()
+
     def build(self):
-        builder_cls = get_builder(self.model_name) if self.model_name else get_builder("Qwen3")
-        self.model_builder = builder_cls(self.persistent_kernel)
-        if self.weight_from_model:
+        """Record the model graph through the builder registered for the model name (mpk.py:351-367)."""
+        self.model_builder = get_builder(self.model_name or "Qwen3")(self.persistent_kernel)
+        if not self.weight_from_model:
+            self.model_builder.build_from_config(self.model_config)
+        else:
             self.model_builder.build_from_model(model_name=self.metadata.model_name, model_path=self.metadata.model_path)
             self.tokenizer = self.model_builder.tokenizer
-        else:
-            self.model_builder.build_from_config(self.model_config)
         self.with_lm_head = self.model_builder.with_lm_head
         self.is_built = True
 
     def generate_task_graph(self):
-        if not self.is_built:
-            raise ValueError("Model is not built yet")
-        results = self.persistent_kernel.kn_graph.generate_task_graph(num_gpus=1, my_gpu_id=0)
+        self._require_built()
         self.task_graph_generated = True
-        return results
+        return self.persistent_kernel.kn_graph.generate_task_graph(num_gpus=1, my_gpu_id=0)
 
     def compile(self, output_dir: str = None):
-        if not self.is_built:
-            raise ValueError("Model is not built yet")
+        self._require_built()
         self.persistent_kernel.compile(output_dir=output_dir)
         self.is_compiled = True
         if self.persistent_kernel.single_weight_copy:
@@ -250,13 +240,14 @@ class MPK:
             self.model_builder.release_weights(self.persistent_kernel.release_row_major_weights())
 
     def __call__(self, **kwargs):
-        if not self.is_compiled:
-            self.compile()
-        if self.need_cpy_input:
-            self.input_tokens.copy_(self.src_input_tokens.to(torch.int64))
+        """One launch (mpk.py:405-421).  Returns the normalised last hidden state when the graph was built without an LM
+        head and the caller drives single passes, None otherwise."""
+        self._ensure_compiled()
+        if self.src_input_tokens is not None:  # the caller's ids are not int64: refresh the staging copy the kernel reads
+            self.input_tokens.copy_(self.src_input_tokens)
         self.persistent_kernel(**kwargs)
-        if not self.with_lm_head and self.persistent_kernel.mode == "online_notoken":
-            return self.model_builder.returned_hidden_state  # the normalised last hidden state, for the caller's own head
+        headless_pass = self.persistent_kernel.mode == "online_notoken" and not self.with_lm_head
+        return self.model_builder.returned_hidden_state if headless_pass else None
 
     def decode(self, ids: torch.Tensor):
         return self.model_builder.decode(ids)

@@ -81,7 +81,8 @@ class PersistentKernel:
         self.page_size = page_size
         self.eos_token_id = eos_token_id
         self.meta_tensors = meta_tensors
-        self.profiler_tensor = profiler_tensor
+        self._profiler_tensor = profiler_tensor
+        self._profiler_attached = False
         self.trace_name = trace_name
         self.use_nvshmem = False
         self.spec_decode_config = None
@@ -742,6 +743,8 @@ class PersistentKernel:
         output_dir = kwargs.get("output_dir", None)
         _capi.check(self._lib.mk_compile(self._handle))
         self._is_compiled = True
+        if self._profiler_tensor is not None:
+            self._attach_profiler()
         if output_dir is not None:
             import os
             os.makedirs(output_dir, exist_ok=True)
@@ -750,6 +753,28 @@ class PersistentKernel:
                 f.write(res["json_file"])
             with open(os.path.join(output_dir, "stage_program.txt"), "w") as f:
                 f.write(self.describe_program())
+
+    @property
+    def profiler_tensor(self):
+        return self._profiler_tensor
+
+    @profiler_tensor.setter
+    def profiler_tensor(self, t):
+        """A uint64 device tensor the kernel records begin/end of every stage of every iteration into (reference: the
+        profiler_tensor constructor argument, persistent_kernel.py:2590-2600); None stops recording."""
+        self._profiler_tensor = t
+        if self._is_compiled:
+            self._attach_profiler()
+
+    def _attach_profiler(self):
+        t = self._profiler_tensor
+        if t is None:
+            _capi.check(self._lib.mk_set_profiler(self._handle, None, 0))
+            self._profiler_attached = False
+            return
+        assert t.is_cuda and t.dtype in (torch.uint64, torch.int64) and t.dim() == 1 and t.is_contiguous(), "the profiler tensor is a flat uint64 device tensor"
+        _capi.check(self._lib.mk_set_profiler(self._handle, ctypes.c_void_p(t.data_ptr()), t.numel()))
+        self._profiler_attached = True
 
     @staticmethod
     def _stream_ptr(stream):
@@ -770,13 +795,11 @@ class PersistentKernel:
             self.export_profile()
 
     def export_profile(self, trace_name: str = None):
-        """With a profiler tensor (reference: persistent_kernel.py:2644-2658): the per-stage device timeline of the last
-        iteration goes into the tensor in the reference's (tag, timestamp) format and out as `<trace_name>.perfetto-trace`
-        (default mirage_<rank>), the raw tensor beside it as `.pt`.  Returns the trace's path."""
-        from .profiler_persistent import export_to_perfetto_trace, fill_profiler_tensor
+        """With a profiler tensor (reference: persistent_kernel.py:2644-2658): what the kernel recorded into it (every stage
+        of every iteration since the tensor was attached or the requests were last initialised, as far as it had room) goes
+        out as `<trace_name>.perfetto-trace` (default mirage_<rank>), the raw tensor beside it as `.pt`.  Returns the path."""
+        from .profiler_persistent import export_to_perfetto_trace
         assert self.profiler_tensor is not None, "no profiler tensor was passed to the constructor"
-        n_wg = self.stats()["num_workgroups"]
-        fill_profiler_tensor(self.profiler_tensor, [self.stage_profile(w, raw=True) for w in range(n_wg)])
         name = (trace_name or self.trace_name or f"mirage_{self.mpi_rank}") + ".perfetto-trace"
         export_to_perfetto_trace(self.profiler_tensor, name)
         torch.save(self.profiler_tensor.cpu(), name.replace(".perfetto-trace", ".pt"))

@@ -3,12 +3,15 @@
 The reference's kernels write (tag, timestamp) entries into a caller-supplied uint64 tensor when a profiler tensor is
 passed (include/mirage/persistent_kernel/profiler.h:42-54,129-180) and `PersistentKernel.__call__` turns it into a
 Perfetto trace afterwards (python/mirage/mpk/persistent_kernel.py:2644-2658, python/mirage/mpk/profiler_persistent.py).
-Here the kernel always records per-stage device timestamps of the last iteration (mk_get_stage_profile); `fill_profiler_
-tensor` re-expresses them in the reference's entry format, so a caller's tooling that decodes that tensor keeps working:
+Here the kernel does the same once the tensor is attached (mk_set_profiler; `PersistentKernel(profiler_tensor=...)` does
+it at compile time): begin and end of every stage each workgroup executes, every iteration, until the tensor is full.
+Independently of that the kernel always keeps finer per-stage ticks of the LAST iteration (mk_get_stage_profile), and
+`fill_profiler_tensor` re-expresses those in the same entry format for a tensor that was not attached:
 
     entry 0            : int32 pair (num_blocks, num_groups)
     entry i (non-zero) : low 32 bits  tag = event_no << 19 | (block * num_groups + group) << 11 | event_idx << 2 | type
-                         high 32 bits timestamp (100 MHz ticks here, relative to the earliest tick of the iteration)
+                         high 32 bits timestamp in ns (low word of the 100 MHz device clock x 10, as the reference keeps the low word
+                         of its ns timer; fill_profiler_tensor counts from the iteration's earliest tick)
     type               : 0 begin, 1 end, 2 instant; event_idx is the reference's task-type number of the stage
 
 `export_to_perfetto_trace` decodes such a tensor.  With the `tg4perfetto` package (what the reference uses; not present in
@@ -68,10 +71,10 @@ def fill_profiler_tensor(profiler_tensor: torch.Tensor, profiles, num_groups: in
             if begin <= 0 or end <= 0 or len(words) + 1 > cap:
                 continue
             ev = stage_event_idx(p[0])
-            words.append(encode_tag(s, w, 0, num_groups, ev, 0) | (((begin - t0) & 0xFFFFFFFF) << 32))
-            words.append(encode_tag(s, w, 0, num_groups, ev, 1) | (((end - t0) & 0xFFFFFFFF) << 32))
+            words.append(encode_tag(s, w, 0, num_groups, ev, 0) | ((((begin - t0) * 10) & 0xFFFFFFFF) << 32))
+            words.append(encode_tag(s, w, 0, num_groups, ev, 1) | ((((end - t0) * 10) & 0xFFFFFFFF) << 32))
     host = torch.zeros(profiler_tensor.numel(), dtype=torch.int64)
-    # (values above 2^63 do not occur: timestamps are relative and below 2^31 for any iteration shorter than 21 s)
+    # (values above 2^63 do not occur: timestamps are relative and below 2^31 for any iteration shorter than 2 s)
     host[:len(words)] = torch.tensor(words, dtype=torch.int64)
     profiler_tensor.copy_(host.view(profiler_tensor.dtype) if profiler_tensor.dtype != torch.int64 else host)
     return len(words) - 1
@@ -87,6 +90,9 @@ def export_to_perfetto_trace(profiler_buffer: torch.Tensor, file_name: str) -> s
             continue
         tag, ts = wd & 0xFFFFFFFF, (wd >> 32) & 0xFFFFFFFF
         entries.append(decode_tag(tag, num_blocks, num_groups) + (ts,))
+    # entries of one workgroup in the order they were written (begin before end on equal times); times count from the first
+    t0 = min((e[5] for e in entries), default=0)
+    entries = sorted((e[:5] + (e[5] - t0,) for e in entries), key=lambda e: (e[1], e[2], e[5], e[0], e[4]))
     try:
         from tg4perfetto import TraceGenerator  # the reference's writer
     except ImportError:
@@ -117,7 +123,7 @@ def export_to_perfetto_trace(profiler_buffer: torch.Tensor, file_name: str) -> s
         events.append({"ph": "M", "name": "process_name", "pid": b, "args": {"name": f"block_{b}"}})
     for event_no, b, g, ev, typ, ts in entries:
         name = f"{EVENT_NAMES.get(ev, 'TASK_' + str(ev))}_{event_no}"
-        events.append({"ph": "B" if typ == 0 else ("E" if typ == 1 else "i"), "name": name, "pid": b, "tid": g, "ts": ts * 0.01})  # 100 MHz ticks -> us
+        events.append({"ph": "B" if typ == 0 else ("E" if typ == 1 else "i"), "name": name, "pid": b, "tid": g, "ts": ts * 0.001})  # ns -> us
     with open(file_name, "w") as f:
         json.dump({"traceEvents": events, "displayTimeUnit": "ns"}, f)
     return "json"

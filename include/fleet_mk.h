@@ -202,6 +202,13 @@ int mk_get_stage_profile(mk_graph *g, int workgroup, int64_t *ticks_out, int max
 /* Same layout, four further ticks per stage: marks that stage code sets inside its work in a library built with
  * -DMK_TRACE (zero in a regular build).  Used to see where a stage's time goes. */
 int mk_get_stage_marks(mk_graph *g, int workgroup, int64_t *ticks_out, int max_stages);
+/* Counterpart of the reference's profiler buffer (include/mirage/persistent_kernel/profiler.h:129-180; handed to
+ * init_func as profiler_ptr, python/mirage/mpk/persistent_kernel.py:2590-2600): a caller-owned device tensor of
+ * `num_entries` uint64 that receives a (tag, time) pair for the begin and the end of EVERY stage every workgroup executes,
+ * iteration after iteration, until it is full.  Entry 0 = (workgroups, 1 group); the k-th entry of workgroup b is entry
+ * 1 + b + k * workgroups; low 32 bits tag = stage instance << 19 | b << 11 | task type << 2 | (0 begin / 1 end), high 32
+ * bits = low word of the device time in ns.  The tensor is cleared here and by mk_init_requests; NULL stops recording. */
+int mk_set_profiler(mk_graph *g, void *device_u64, int64_t num_entries);
 /* Stage listing (one line per stage) for debugging and tests; owned by the handle. */
 int mk_describe_program(mk_graph *g, const char **text_out);
 

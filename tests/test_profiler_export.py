@@ -21,9 +21,9 @@ def test_profiler_tensor_round_trip(tmp_path):
     words = buf.view(torch.int64).tolist()
     assert words[0] & 0xFFFFFFFF == 2 and words[0] >> 32 == 1
     event_no, block, group, ev, typ = decode_tag(words[1] & 0xFFFFFFFF, 2, 1)
-    assert (event_no, block, group, ev, typ) == (0, 0, 0, 101, 0) and words[1] >> 32 == 10  # begins at its barrier tick, relative to tick 1000
+    assert (event_no, block, group, ev, typ) == (0, 0, 0, 101, 0) and words[1] >> 32 == 100  # begins at its barrier tick, in ns relative to tick 1000
     event_no, block, group, ev, typ = decode_tag(words[8] & 0xFFFFFFFF, 2, 1)
-    assert (event_no, block, group, ev, typ) == (2, 1, 0, 102, 1) and words[8] >> 32 == 960
+    assert (event_no, block, group, ev, typ) == (2, 1, 0, 102, 1) and words[8] >> 32 == 9600
     out = tmp_path / "t.perfetto-trace"
     kind = export_to_perfetto_trace(buf, str(out))
     assert out.exists()
@@ -31,14 +31,15 @@ def test_profiler_tensor_round_trip(tmp_path):
         tr = json.loads(out.read_text())["traceEvents"]
         slices = [e for e in tr if e["ph"] in ("B", "E")]
         assert len(slices) == 8 and slices[0]["name"] == "TASK_EMBEDDING_0" and slices[0]["pid"] == 0
-        assert abs(slices[-1]["ts"] - 9.6) < 1e-9  # 960 ticks = 9.6 us
+        assert abs(slices[-1]["ts"] - (9.6 - 0.1)) < 1e-9  # 960 ticks = 9.6 us, counted from the first entry (at 0.1 us)
     # a tensor too small for everything keeps what fits
     small = torch.zeros(4, dtype=torch.uint64)
     assert fill_profiler_tensor(small, profiles) == 2
 
 
 @pytest.mark.gpu
-def test_profiler_tensor_after_a_run(tmp_path):
+def test_profiler_tensor_records_every_iteration(tmp_path):
+    """The kernel itself writes the tensor (profiler.h:129-180): every stage of every iteration, workgroup-interleaved."""
     from mirage.mpk.profiler_persistent import decode_tag
     from oracle.qwen3_ref import make_model_weights, make_prompt
     from test_qwen3_decode import _decoder, _small_cfg
@@ -46,22 +47,51 @@ def test_profiler_tensor_after_a_run(tmp_path):
     w = make_model_weights(cfg, seed=5)
     dec = _decoder(cfg, w, max_num_batched_tokens=1, max_seq_length=24, page_size=16)
     dec.load_prompts([make_prompt(cfg, 6, 2)])
-    dec.mpk.profiler_tensor = torch.zeros(1 << 16, dtype=torch.uint64, device="cuda")
+    dec.mpk.profiler_tensor = torch.zeros(1 << 18, dtype=torch.uint64, device="cuda")  # attached after compile
+    dec.load_prompts([make_prompt(cfg, 6, 2)])
     dec.mpk.trace_name = str(tmp_path / "run")
-    dec.mpk()  # one persistent launch; the profile of its last iteration is exported afterwards
+    dec.mpk()  # one persistent launch; exported afterwards
     words = dec.mpk.profiler_tensor.cpu().view(torch.int64).tolist()
     st = dec.mpk.stats()
-    assert words[0] & 0xFFFFFFFF == st["num_workgroups"] and words[0] >> 32 == 1
-    entries = [(decode_tag(wd & 0xFFFFFFFF, st["num_workgroups"], 1), wd >> 32) for wd in words[1:] if wd != 0]
-    assert len(entries) >= 2 * st["num_workgroups"] * 5
-    # per workgroup and stage: a begin followed by a later end; the linears of the single-token path are among the stages
-    open_ = {}
-    for (event_no, block, _, ev, typ), ts in entries:
-        if typ == 0:
-            open_[(block, event_no)] = ts
-        else:
-            assert ts >= open_.pop((block, event_no))
-    assert not open_
-    assert {ev for (_, _, _, ev, _), _ in entries} >= {101, 102, 116, 108, 110, 111}
+    G, iters = st["num_workgroups"], st["iterations"]
+    assert iters >= 10
+    assert words[0] & 0xFFFFFFFF == G and words[0] >> 32 == 1
+    per_wg = {}
+    for i, wd in enumerate(words[1:]):
+        if wd == 0:
+            continue
+        event_no, block, group, ev, typ = decode_tag(wd & 0xFFFFFFFF, G, 1)
+        assert block == i % G and group == 0  # entry k of workgroup b sits at 1 + b + k * G
+        per_wg.setdefault(block, []).append((event_no, ev, typ, (wd >> 32) & 0xFFFFFFFF))
+    assert len(per_wg) == G
+    n0 = len(per_wg[0])
+    for b, ent in per_wg.items():
+        assert len(ent) == n0 and n0 % 2 == 0  # every workgroup passes the same stages
+        for k in range(0, n0, 2):
+            (e0, ev0, t0, ts0), (e1, ev1, t1, ts1) = ent[k], ent[k + 1]
+            assert (e0, ev0, t0, t1) == (e1, ev1, 0, 1) and ts1 >= ts0
+            if k:
+                assert ts0 >= ent[k - 1][3] and 0 < ((e0 - ent[k - 2][0]) & 0x1FFF) < 8  # stages follow one another (skipped ones leave gaps in the numbering)
+    # one embedding and one sampling stage per iteration; the fused single-token forms are among the stages
+    evs = [e[1] for e in per_wg[0][::2]]
+    assert evs.count(101) == iters and evs.count(111) == iters
+    assert set(evs) >= {101, 102, 116, 108, 110, 111}
+    # a stage's begin on one workgroup is never before the previous stage's end... on the slowest workgroup of that stage is
+    # what the barrier gives; checked on whole microseconds of slack for clock skew between dies
+    for k in range(2, min(n0, 200), 2):
+        assert min(per_wg[b][k][3] for b in per_wg) + 2000 >= max(per_wg[b][k - 2][3] for b in per_wg)
     assert (tmp_path / "run.perfetto-trace").exists() and (tmp_path / "run.pt").exists()
+    # a tensor that is too small keeps the first entries and nothing is written past its end
+    guard = torch.zeros(4 * G + 1 + 64, dtype=torch.uint64, device="cuda")
+    dec.mpk.profiler_tensor = guard[:4 * G + 1]
+    dec.load_prompts([make_prompt(cfg, 6, 2)])
+    dec.mpk()
+    gw = guard.cpu().view(torch.int64)
+    assert int((gw[1:4 * G + 1] != 0).sum()) == 4 * G and int((gw[4 * G + 1:] != 0).sum()) == 0
+    # detached: the kernel records nothing
+    dec.mpk.profiler_tensor = None
+    guard.zero_()
+    dec.load_prompts([make_prompt(cfg, 6, 2)])
+    dec.mpk()
+    assert int((guard.cpu().view(torch.int64) != 0).sum()) == 0
     dec.mpk.finalize()
