@@ -3290,9 +3290,17 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
     }
   };
 
-  for (int u = c.vid; u < n_units; u += c.G) {
+  for (int uu = c.vid; uu < n_units; uu += c.G) {
     AttnUnit a;
-    const bool first = u == c.vid;
+    const bool first = uu == c.vid;
+    // More (token, kv head) pairs than workgroups: every other round deals them in reverse order, so a workgroup that
+    // drew a long context in one round draws from the other end of the batch in the next (requests that entered the
+    // batch together sit next to each other and are about equally far along).
+    int u = uu;
+    if (cmax == 1 && ((uu / c.G) & 1)) {
+      const int r0 = (uu / c.G) * c.G, rn = min(c.G, n_units - r0);
+      u = r0 + rn - 1 - (uu - r0);
+    }
     if (first) {
       if (!have0) continue;
       a = a0;
@@ -3477,6 +3485,9 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
           for (int s_ = 0; s_ < 4; s_++) kk[s_] = __builtin_nontemporal_load((const bf16x8 *)(kc + base + s_ * 4));
         }
         // to LDS: request s brings rows 4 s .. 4 s + 3 whole (lane (row in group, 16-byte piece))
+        // (streaming requests -- the cache-policy bit the nontemporal loads of the other paths carry: a cached K/V row is
+        // read once per iteration and need not displace the activations the linears share through the L2)
+        constexpr int KV_NT = 2;
         size_t gb[4];
 #pragma unroll
         for (int s_ = 0; s_ < 4; s_++) gb[s_] = row_base(p0 + 4 * s_ + lg) + lr;
@@ -3484,12 +3495,12 @@ __device__ __forceinline__ void stage_attn(CStage &st, Ctx &c, const MkRuntime &
 #pragma unroll
           for (int s_ = 0; s_ < 4; s_++)
             __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(kc + gb[s_]),
-                                             (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + TS + s_ * GS), 16, 0, 0);
+                                             (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + TS + s_ * GS), 16, 0, KV_NT);
         }
 #pragma unroll
         for (int s_ = 0; s_ < 4; s_++)
           __builtin_amdgcn_global_load_lds((const MK_GLOBAL void *)(unsigned long long)(vc + gb[s_]),
-                                           (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + s_ * GS), 16, 0, 0);
+                                           (__attribute__((address_space(3))) void *)(__attribute__((address_space(3))) char *)(vbuf + s_ * GS), 16, 0, KV_NT);
       };
       const int vlane = lg * GS + lr * 2;
       const int klane = (lr >> 2) * GS + (lr & 3) * 256 + lg * 16;
