@@ -122,6 +122,7 @@ struct mk_graph {
   std::vector<int> stage_weight;      // per stage: tensor id of a LINEAR stage's weight operand (-1: none)
   std::vector<char> releasable;       // per tensor (single-weight-copy graphs, after mk_compile): the handle never reads it again
   bool single_copy = false;
+  int spec_len = 0;  // guesses per decoding request (set by a find_ngram_global task)
   void *profiler_ptr = nullptr;  // the caller's profiler tensor (mk_set_profiler)
   long long profiler_cap = 0;
   int64_t row_major_bytes = 0;
@@ -481,10 +482,12 @@ int lower_attention(mk_graph *g, size_t &i) {
     nq = t0.params[0];
     chunks = t0.params[6];
     merge = "gang_attn_merge_mi300";
-  } else if (t0.name == "paged_attention" || t0.name == "paged_attention_split_kv_mi300" || t0.name == "attention") {
+  } else if (t0.name == "paged_attention" || t0.name == "paged_attention_split_kv_mi300" || t0.name == "attention" || t0.name == "single_batch_extend_attention") {
     // "attention" (python/mirage/mpk/persistent_kernel.py:587-650) is the form with one contiguous cache row range per
     // request, [requests, seq_len, kv heads, head_dim]: a paged cache whose pages are max_seq_length long
     const bool split = t0.name == "paged_attention_split_kv_mi300";
+    // ("single_batch_extend_attention", persistent_kernel.py:653-730: the same cache form for the rows of a speculating
+    // request -- its newest token and the guesses behind it; params 4, 5 = number of guesses, output stride)
     const size_t need_params = t0.name == "attention" ? 4u : (split ? 7u : 6u);
     if (t0.ops.size() != (split ? 9u : 8u) || t0.params.size() < need_params) return fail(MK_EINVAL, "%s: wrong number of operands / params", t0.name.c_str());
     in_id = t0.ops[0]; kc_id = t0.ops[1]; vc_id = t0.ops[2]; qn_id = t0.ops[3]; kn_id = t0.ops[4]; cos_id = t0.ops[5]; sin_id = t0.ops[6];
@@ -876,7 +879,7 @@ int lower(mk_graph *g) {
       g->stage_desc.push_back(fmt("SILU_MUL %s -> %s n=%d half=%d", x.name.c_str(), o.name.c_str(), st.n, st.silu_half));
       i++;
     } else if (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300" || t.name == "paged_attention" ||
-               t.name == "paged_attention_split_kv_mi300" || t.name == "attention") {
+               t.name == "paged_attention_split_kv_mi300" || t.name == "attention" || t.name == "single_batch_extend_attention") {
       int rc = lower_attention(g, i);
       if (rc) return rc;
     } else if (t.name == "moe_topk_softmax_mi300") {
@@ -995,6 +998,68 @@ int lower(mk_graph *g) {
       g->stages.push_back(sr);
       g->stage_desc.push_back(fmt("ARGMAX_REDUCE -> %s", o.name.c_str()));
       i += 2;
+    } else if (t.name == "find_ngram_partial") {
+      // (tokens, partial) + [ngram size]; src/kernel/task_register.cc:1689-1719
+      if (t.ops.size() != 2 || t.params.size() != 1) return fail(MK_EINVAL, "find_ngram_partial expects (tokens, partial results) and the n-gram size");
+      const Tensor &tk = g->tensors[t.ops[0]], &po = g->tensors[t.ops[1]];
+      if (tk.ptr != (void *)g->cfg.tokens) return fail(MK_EINVAL, "find_ngram_partial searches the `tokens` meta tensor: attach that tensor as its input");
+      if (po.ndims != 2 || po.dtype != MK_DT_I64 || po.dims[0] < g->cfg.max_num_batched_requests || po.dims[1] < 1)
+        return fail(MK_EINVAL, "find_ngram_partial: the partial results are an int64 [batch slots >= %d, tasks] tensor", g->cfg.max_num_batched_requests);
+      if (t.params[0] < 1 || t.params[0] > 16) return fail(MK_EINVAL, "find_ngram_partial: n-gram size %d outside [1, 16]", t.params[0]);
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_NGRAM_PARTIAL;
+      st.n = (int)po.dims[1];
+      st.k = t.params[0];
+      st.out = po.ptr;
+      st.ld_out = (int)po.strides[0];
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("NGRAM_PARTIAL %s -> %s ngram=%d tasks=%d", tk.name.c_str(), po.name.c_str(), st.k, st.n));
+      i++;
+    } else if (t.name == "find_ngram_global") {
+      // (partial, tokens, spec tokens) + [ngram size, spec length]; task_register.cc:1721-1754
+      if (t.ops.size() != 3 || t.params.size() != 2) return fail(MK_EINVAL, "find_ngram_global expects (partial results, tokens, spec tokens) and (n-gram size, spec length)");
+      const Tensor &pi = g->tensors[t.ops[0]], &tk = g->tensors[t.ops[1]], &so = g->tensors[t.ops[2]];
+      if (tk.ptr != (void *)g->cfg.tokens) return fail(MK_EINVAL, "find_ngram_global reads the `tokens` meta tensor: attach that tensor as its input");
+      if (pi.ndims != 2 || pi.dtype != MK_DT_I64 || pi.dims[0] < g->cfg.max_num_batched_requests) return fail(MK_EINVAL, "find_ngram_global: bad partial-result tensor");
+      if (so.dtype != MK_DT_I64 || (long long)so.elems() < B) return fail(MK_EINVAL, "find_ngram_global: the spec-token tensor holds one int64 id per token row of an iteration (>= %d)", B);
+      const int spec_len = t.params[1];
+      if (spec_len < 1) return fail(MK_EINVAL, "find_ngram_global: spec length %d < 1", spec_len);
+      if (g->cfg.mode != MK_MODE_OFFLINE) return fail(MK_EUNSUPPORTED, "speculative decoding needs the offline scheduler (mode offline): it sizes the token groups of decoding requests");
+      if (B < spec_len + 1) return fail(MK_EINVAL, "speculative decoding with %d guesses needs max_num_batched_tokens >= %d", spec_len, spec_len + 1);
+      if ((g->cfg.max_tokens_per_request > 0 ? g->cfg.max_tokens_per_request : 8) < spec_len + 1)
+        return fail(MK_EINVAL, "speculative decoding with %d guesses needs max_tokens_per_request >= %d (a decoding request brings that many rows)", spec_len, spec_len + 1);
+      if (g->spec_len && g->spec_len != spec_len) return fail(MK_EINVAL, "two find_ngram_global tasks with different spec lengths");
+      g->spec_len = spec_len;
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_NGRAM_GLOBAL;
+      st.n = (int)pi.dims[1];
+      st.k = t.params[0];
+      st.topk = spec_len;
+      st.in = pi.ptr;
+      st.ld_in = (int)pi.strides[0];
+      st.out = so.ptr;
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("NGRAM_GLOBAL %s, %s -> %s ngram=%d spec=%d", pi.name.c_str(), tk.name.c_str(), so.name.c_str(), st.k, spec_len));
+      i++;
+    } else if (t.name == "target_verify_greedy") {
+      // (spec tokens, target tokens, accepted length); task_register.cc:1756-1784
+      if (t.ops.size() != 3) return fail(MK_EINVAL, "target_verify_greedy expects (spec tokens, target tokens, output)");
+      const Tensor &sp = g->tensors[t.ops[0]], &tg = g->tensors[t.ops[1]], &vo = g->tensors[t.ops[2]];
+      if (sp.dtype != MK_DT_I64 || tg.dtype != MK_DT_I64 || vo.dtype != MK_DT_I64 || (long long)sp.elems() < B || (long long)tg.elems() < B || vo.elems() < 1)
+        return fail(MK_EINVAL, "target_verify_greedy: spec and target tokens hold one int64 id per token row (>= %d), the output one int64", B);
+      if (!g->cfg.num_new_tokens) return fail(MK_EINVAL, "target_verify_greedy writes the num_new_tokens meta tensor: it must be given");
+      if (!g->spec_len) return fail(MK_EINVAL, "target_verify_greedy without a find_ngram_global task before it");
+      MkStage st;
+      memset(&st, 0, sizeof(st));
+      st.op = MK_OP_VERIFY;
+      st.in = sp.ptr;
+      st.aux0 = tg.ptr;
+      st.out = vo.ptr;
+      g->stages.push_back(st);
+      g->stage_desc.push_back(fmt("VERIFY %s vs %s -> num_new_tokens, %s", sp.name.c_str(), tg.name.c_str(), vo.name.c_str()));
+      i++;
     } else if (t.name == "paged_attention_split_kv_merge_mi300" || t.name == "paged_attention_ck_fmha_merge_mi300" || t.name == "gang_attn_merge_mi300" ||
                t.name == "splitk_reduce_mi300") {
       return fail(MK_EUNSUPPORTED, "task '%s' must directly follow the split task whose partial results it combines", t.name.c_str());
@@ -1015,6 +1080,9 @@ int lower(mk_graph *g) {
       case MK_OP_MOE_TOPK: st.prof_event = 172; break;
       case MK_OP_MOE_LINEAR: st.prof_event = (st.flags & MK_F_MOE_COMBINE) || st.ld_in_slot ? 171 : 170; break;
       case MK_OP_MOE_COMBINE: st.prof_event = 173; break;
+      case MK_OP_NGRAM_PARTIAL: st.prof_event = 112; break;
+      case MK_OP_NGRAM_GLOBAL: st.prof_event = 113; break;
+      case MK_OP_VERIFY: st.prof_event = 114; break;
       default: st.prof_event = 121; break;
     }
   }
@@ -1065,7 +1133,7 @@ int task_type_id(const std::string &n) {
       {"paged_attention", 116}, {"paged_attention_split_kv_mi300", 130}, {"paged_attention_split_kv_merge_mi300", 131},
       {"paged_attention_ck_fmha_merge_mi300", 131}, {"gang_attn_merge_mi300", 139}, {"splitk_reduce_mi300", 132},
       {"silu_mul_linear_with_residual", 105}, {"rmsnorm_linear", 102}, {"identity", 121}, {"argmax", 109}, {"attention", 103},
-      {"find_ngram_partial", 112}, {"find_ngram_global", 113}, {"target_verify_greedy", 114}};
+      {"find_ngram_partial", 112}, {"find_ngram_global", 113}, {"target_verify_greedy", 114}, {"single_batch_extend_attention", 115}};
   auto it = ids.find(n);
   return it == ids.end() ? 0 : it->second;
 }
@@ -1649,7 +1717,7 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
   for (int i = 0; i < n_operands; i++) {
     // id -1 = optional operand that is absent: only the q/k-norm weights and the cos/sin tables of the attention tasks
     const bool optional = (t.name == "gang_attn_split_kv_mi300" || t.name == "kv_cache_update_mi300" || t.name == "paged_attention" ||
-                           t.name == "paged_attention_split_kv_mi300" || t.name == "attention") && i >= 3 && i <= 6;
+                           t.name == "paged_attention_split_kv_mi300" || t.name == "attention" || t.name == "single_batch_extend_attention") && i >= 3 && i <= 6;
     if (tensor_ids[i] >= (int)g->tensors.size() || tensor_ids[i] < (optional ? -1 : 0))
       return fail(MK_EINVAL, "task '%s': bad tensor id %d for operand %d", task_name, tensor_ids[i], i);
     t.ops.push_back(tensor_ids[i]);
@@ -1666,7 +1734,8 @@ int mk_add_task(mk_graph *g, const char *task_name, const int grid_dim[3], const
                                 "paged_attention_ck_fmha_split_kv_mi300", "argmax_partial", "argmax_reduce", "moe_topk_softmax_mi300", "moe_w13_linear_mi300",
                                 "moe_w2_linear_mi300", "gang_moe_w13_linear_mi300", "gang_moe_w2_linear_mi300", "moe_silu_mul", "moe_mul_sum_add_mi300",
                                 "paged_attention", "paged_attention_split_kv_mi300", "paged_attention_split_kv_merge_mi300",
-                                "paged_attention_ck_fmha_merge_mi300", "gang_attn_merge_mi300", "splitk_reduce_mi300", "silu_mul_linear_with_residual", "rmsnorm_linear", "identity", "argmax", "attention"};
+                                "paged_attention_ck_fmha_merge_mi300", "gang_attn_merge_mi300", "splitk_reduce_mi300", "silu_mul_linear_with_residual", "rmsnorm_linear", "identity", "argmax", "attention",
+                                "find_ngram_partial", "find_ngram_global", "target_verify_greedy", "single_batch_extend_attention"};
   bool ok = linear_kind(t.name, &a, &b, &c);
   for (auto k : known) ok = ok || t.name == k;
   if (!ok) return fail(MK_EUNSUPPORTED, "Unsupported task name: %s", task_name);
@@ -1757,6 +1826,7 @@ int mk_compile(mk_graph *g) {
   rt.max_pages = c.max_num_pages;
   rt.total_requests = c.total_num_requests;
   rt.max_new_per_req = c.max_tokens_per_request > 0 ? c.max_tokens_per_request : 8;
+  rt.spec_len = g->spec_len;
   rt.eos_token_id = c.eos_token_id;
   rt.step = c.step;
   rt.tokens = (long long *)c.tokens;

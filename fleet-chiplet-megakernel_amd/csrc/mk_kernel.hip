@@ -219,6 +219,12 @@ __device__ __forceinline__ void stc_u16(uint16_t *p, uint16_t v) {
 __device__ __forceinline__ void stc_f32(float *p, float v) {
   __hip_atomic_store((__attribute__((address_space(1))) unsigned *)(unsigned long long)p, __float_as_uint(v), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
 }
+__device__ __forceinline__ void stc_u64(void *p, unsigned long long v) {
+  __hip_atomic_store((__attribute__((address_space(1))) unsigned long long *)(unsigned long long)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
+__device__ __forceinline__ void stc_i32(int *p, int v) {
+  __hip_atomic_store((__attribute__((address_space(1))) int *)(unsigned long long)p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
+}
 __device__ __forceinline__ void stc_16B(u32x4 *p, u32x4 v) {
   __attribute__((address_space(1))) unsigned long long *q = (__attribute__((address_space(1))) unsigned long long *)(unsigned long long)p;
   __hip_atomic_store(q, (unsigned long long)v.x | ((unsigned long long)v.y << 32), __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT);
@@ -349,11 +355,15 @@ __device__ __attribute__((noinline)) int mk_prepare_next_batch(const MkRuntime &
     const int q0 = rt.qo_indptr[i];
     const int n = rt.qo_indptr[i + 1] - q0;
     const int plen = rt.prompt_lengths[req];
-    for (int j = 0; j < n; j++) {
+    // a decoding request of a speculating graph keeps what its verify stage accepted: the sampled token of its first
+    // row, and one more for every candidate row in front that turned out right (persistent_kernel.cuh:541-552)
+    int nc = n;
+    if (rt.spec_len > 0 && st >= plen && n > 0) nc = max(1, min(n, ldc_i32(&rt.num_new_tokens[req])));
+    for (int j = 0; j < nc; j++) {
       const int pos = st + j + 1;
       if (pos >= plen && pos < rt.max_seq) rt.tokens[(long long)req * rt.max_seq + pos] = rt.output_tokens[q0 + j];
     }
-    const int ns = st + n;
+    const int ns = st + nc;
     rt.step[req] = ns;
     const bool full = ns + 1 >= rt.max_seq;
     const bool eos = ns >= plen && rt.tokens[(long long)req * rt.max_seq + ns] == rt.eos_token_id;
@@ -382,7 +392,8 @@ __device__ __attribute__((noinline)) int mk_prepare_next_batch(const MkRuntime &
     const int st = rt.step[req];
     int n = rt.prompt_lengths[req] - st;
     if (n > 0) n = min(n, min(rt.max_new_per_req, B - ntok));  // prefill chunk
-    else n = min(1, B - ntok);                                 // decode
+    else n = min(1 + min(rt.spec_len, min(rt.max_new_per_req - 1, rt.max_seq - 2 - st)), B - ntok);  // decode: the newest token (+ candidate rows,
+                                                                                                      // whose ids the n-gram stage fills in)
     for (int j = 0; j < n; j++) {
       rt.input_tokens[ntok + j] = rt.tokens[(long long)req * rt.max_seq + st + j];
       rt.tok_slot[ntok + j] = nreq;
@@ -3834,8 +3845,126 @@ __device__ __forceinline__ void stage_argmax_reduce(CStage &st, Ctx &c, const Mk
 
 // ----------------------------------------------------------------------------- the kernel
 // One pass over the stage program for the M tokens of this iteration.
+// ----------------------------------------------------------------------------- prompt-lookup speculative decoding
+// A decoding request of a speculating graph brings n = 1 + (up to spec_len) rows into an iteration (the scheduler sizes
+// the group): row 0 is its newest token at position s, rows 1.. are guesses -- the tokens that followed the EARLIEST
+// earlier occurrence of its last N tokens (reference tasks find_ngram_partial_kernel / find_ngram_global_kernel,
+// tasks/speculative_decoding/prompt_lookup.cuh:22-140, called with input_token_num = step + 1 and step,
+// src/kernel/task_register.cc:1713-1752).  All rows run through the model as a chunk of the same request (causal
+// attention inside the chunk, K/V appended at s .. s + n - 1); the verify stage then keeps the sampled token of row 0
+// and one more for every guess in front that the model agrees with (target_verify_greedy_kernel,
+// tasks/speculative_decoding/target_verify.cuh:21-62), and the next scheduler step advances the request by that many
+// positions.  K/V rows of rejected guesses are rewritten before anything reads them.  These three stages are plain
+// integer work on a few kilobytes; they are kept out of line so that the stage loop's register allocation does not see
+// them.
+//
+// The search space of a request with T = s + 1 known tokens is idx in [0, T - N); position idx belongs to task
+// (idx / 128) % P, as in the reference (128 threads per task, P tasks round-robin).  A match compares the real tokens
+// idx .. idx + N - 1; the reference compares against a shared-memory window whose last N - 1 entries it leaves unset
+// when they lie at or beyond T - N (prompt_lookup.cuh:62-72), so for the few idx > T - 2 N it reads unset memory.
+__device__ __attribute__((noinline)) void mk_ngram_partial(int stage, const MkRuntime *rtp, int vid, int G, int *lds) {
+  const MkStage *stp = rtp->stages + stage;
+  const int P = stp->n, N = stp->k, ld = stp->ld_out;
+  long long *part = (long long *)stp->out;
+  const int R = rtp->max_requests, tid = threadIdx.x;
+  for (int u = vid; u < R * P; u += G) {
+    const int slot = u / P, k = u - slot * P;
+    const int q0 = ldc_i32(&rtp->qo_indptr[slot]), n = ldc_i32(&rtp->qo_indptr[slot + 1]) - q0;
+    const int req = ldc_i32(&rtp->request_ids[slot]);
+    __syncthreads();
+    if (tid == 0) lds[0] = 0x7fffffff;
+    __syncthreads();
+    if (req >= 0 && n > 1) {
+      const int s = ldc_i32(&rtp->tok_pos[q0]);
+      if (s >= rtp->prompt_lengths[req]) {  // decoding
+        const long long *tok = rtp->tokens + (long long)req * rtp->max_seq;
+        const int T = s + 1, total = T - N;
+        for (int it = tid >> 7;; it += 2) {  // the reference's 128-thread block, two of its rounds at a time
+          const long long base = ((long long)it * P + k) * 128;
+          if (base >= total) break;
+          const int idx = (int)base + (tid & 127);
+          if (idx < total) {
+            bool eq = true;
+            for (int i = 0; i < N; i++) eq = eq && ldc_u64(&tok[idx + i]) == ldc_u64(&tok[T - N + i]);
+            if (eq) {
+              atomicMin(&lds[0], idx);
+              break;  // this thread's later rounds only hold larger positions
+            }
+          }
+        }
+      }
+    }
+    __syncthreads();
+    if (tid == 0) {
+      const int m = lds[0];
+      stc_u64(part + (size_t)slot * ld + k, m == 0x7fffffff ? 0x7fffffffffffffffull : (unsigned long long)m);
+    }
+  }
+}
+
+__device__ __attribute__((noinline)) void mk_ngram_global(int stage, const MkRuntime *rtp, int vid, int G, int *lds) {
+  const MkStage *stp = rtp->stages + stage;
+  const int P = stp->n, N = stp->k, ld = stp->ld_in;
+  const long long *part = (const long long *)stp->in;
+  long long *spec = (long long *)stp->out;
+  const int R = rtp->max_requests, tid = threadIdx.x;
+  for (int slot = vid; slot < R; slot += G) {
+    const int q0 = ldc_i32(&rtp->qo_indptr[slot]), n = ldc_i32(&rtp->qo_indptr[slot + 1]) - q0;
+    const int req = ldc_i32(&rtp->request_ids[slot]);
+    if (req < 0 || n <= 0) continue;  // (uniform)
+    const int s = ldc_i32(&rtp->tok_pos[q0]);
+    const bool guess = n > 1 && s >= rtp->prompt_lengths[req];
+    __syncthreads();
+    if (tid == 0) lds[0] = 0x7fffffff;
+    __syncthreads();
+    if (guess) {
+      for (int k = tid; k < P; k += MK_THREADS) {
+        const unsigned long long v = ldc_u64(part + (size_t)slot * ld + k);
+        if (v < 0x7fffffffull) atomicMin(&lds[0], (int)v);
+      }
+    }
+    __syncthreads();
+    const int first = lds[0];
+    const long long *tok = rtp->tokens + (long long)req * rtp->max_seq;
+    for (int j = tid; j < n; j += MK_THREADS) {
+      long long v;
+      if (!guess || j == 0) {
+        v = (long long)ldc_u64(&rtp->input_tokens[q0 + j]);  // the scheduler's token (prompt chunk, or the newest token)
+      } else {
+        const long long ci = (long long)first + N + (j - 1);
+        v = (first != 0x7fffffff && ci <= s) ? (long long)ldc_u64(&tok[ci]) : -1;
+      }
+      stc_u64(spec + q0 + j, (unsigned long long)v);
+    }
+  }
+}
+
+__device__ __attribute__((noinline)) void mk_verify_greedy(int stage, const MkRuntime *rtp, int vid, int G) {
+  const MkStage *stp = rtp->stages + stage;
+  const long long *spec = (const long long *)stp->in, *target = (const long long *)stp->aux0;
+  const int R = rtp->max_requests;
+  for (int slot = vid * MK_THREADS + threadIdx.x; slot < R; slot += G * MK_THREADS) {
+    const int q0 = ldc_i32(&rtp->qo_indptr[slot]), n = ldc_i32(&rtp->qo_indptr[slot + 1]) - q0;
+    const int req = ldc_i32(&rtp->request_ids[slot]);
+    if (req < 0 || n <= 0) continue;
+    int nc = n;
+    if (ldc_i32(&rtp->tok_pos[q0]) >= rtp->prompt_lengths[req]) {
+      // token j of this iteration is what the model sampled on row j; it counts while every guess before it was right
+      // (guess j + 1 is the input of row j + 1) and nothing before it ended the request
+      nc = 1;
+      for (int j = 0; j + 1 < n; j++) {
+        const long long tj = (long long)ldc_u64(&target[q0 + j]);
+        if (tj == rtp->eos_token_id || (long long)ldc_u64(&spec[q0 + j + 1]) != tj) break;
+        nc = j + 2;
+      }
+    }
+    stc_i32(&rtp->num_new_tokens[req], nc);
+    if (slot == 0 && stp->out) stc_u64(stp->out, (unsigned long long)nc);
+  }
+}
+
 template <int MAXM>
-__device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, const int M, char *smem) {
+__device__ __forceinline__ void run_stage_program(const MkRuntime &rt, const MkRuntime *rtp, Ctx &c, const int M, char *smem) {
     for (int s = 0; s < rt.num_stages && !c.dead; s++) {
       CStage &st = ((CStage *)(unsigned long long)rt.stages)[s];
       const int op = st.op, flags = st.flags;
@@ -3892,6 +4021,17 @@ __device__ __forceinline__ void run_stage_program(const MkRuntime &rt, Ctx &c, c
           break;
         case MK_OP_SILU_MUL: stage_silu_mul(st, c, M); break;
         case MK_OP_COPY: stage_copy(st, c, M); break;
+        case MK_OP_NGRAM_PARTIAL:
+        case MK_OP_NGRAM_GLOBAL:
+        case MK_OP_VERIFY:
+          barrier_wait(c);
+          if constexpr (MAXM > 1) {  // (a graph of one token per iteration has no room for guesses)
+            if (st.op == MK_OP_NGRAM_PARTIAL) mk_ngram_partial(s, rtp, c.vid, c.G, (int *)smem);
+            else if (st.op == MK_OP_NGRAM_GLOBAL) mk_ngram_global(s, rtp, c.vid, c.G, (int *)smem);
+            else mk_verify_greedy(s, rtp, c.vid, c.G);
+            c.wrote_through = true;
+          }
+          break;
         case MK_OP_ATTN:
           if constexpr (MAXM == 1) {
             if (st.num_q_heads == 4 * st.num_kv_heads) stage_attn<4, false>(st, c, rt, M, smem);
@@ -4028,7 +4168,7 @@ __device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRunt
       barrier_wait(c);  // the previous iteration's sampled tokens are complete
       t_sched0 = (long long)wall_clock64();
       // a handful of slots: one thread walks them; more: a wavefront, one lane per slot
-      const bool wave_sched = run_scheduler == MK_SCHED_OFFLINE && rt.max_requests > 2;
+      const bool wave_sched = run_scheduler == MK_SCHED_OFFLINE && rt.max_requests > 2 && rt.spec_len == 0;
       int ntok_w = 0;
       if (c.vid == 0 && threadIdx.x < 64 && wave_sched) ntok_w = mk_prepare_next_batch_wave(*rtp, (int *)smem, threadIdx.x);
       if (c.vid == 0 && threadIdx.x == 0) {
@@ -4070,7 +4210,7 @@ __device__ __forceinline__ void mk_kernel_body(const MkRuntime &rt, const MkRunt
       pr[2] = (long long)wall_clock64();
     }
     if (M == 0 || c.dead) break;
-    run_stage_program<MAXM>(rt, c, MAXM == 1 ? 1 : M, smem);
+    run_stage_program<MAXM>(rt, rtp, c, MAXM == 1 ? 1 : M, smem);
   }
   barrier_wait(c);  // drain: nobody leaves while another workgroup may still poll
   if (rt.profiler && threadIdx.x == 0) rt.profiler_count[c.vid] = c.prof_n;

@@ -47,6 +47,10 @@ enum MkOp {
   MK_OP_MOE_LINEAR = 9,   // per-expert linear over the active experts (W13 with optional SwiGLU, W2)
   MK_OP_MOE_COMBINE = 10, // out = res + sum_k w[t,k] * x[t,k,:]
   MK_OP_COPY = 11,        // out[t, :] = in[t, :], n 16-bit units per token row
+  // prompt-lookup speculative decoding (integer stages; tasks/speculative_decoding/prompt_lookup.cuh, target_verify.cuh)
+  MK_OP_NGRAM_PARTIAL = 12,  // out[slot, task] = earliest position among the task's share where the request's last k tokens occurred before
+  MK_OP_NGRAM_GLOBAL = 13,   // out[row] = this iteration's token ids: the scheduler's, and for a decoding request the tokens after that position
+  MK_OP_VERIFY = 14,         // num_new_tokens[request] = 1 + leading candidates the sampled tokens agree with
 };
 
 enum MkStageFlags {
@@ -167,6 +171,7 @@ struct MkSched {
 struct MkRuntime {
   int num_stages, max_tokens, max_requests, max_seq;
   int page_size, max_pages, total_requests, max_new_per_req;
+  int spec_len, pad_spec;  // speculative candidates a decoding request brings into an iteration beside its newest token (0: none)
   long long eos_token_id;
   // meta tensors (persistent_kernel.py:2590-2600 order)
   int *step;

@@ -110,7 +110,7 @@ class Qwen3Decoder:
                  max_seq_length: int = 1200, page_size: int = 4096, max_num_pages: int = None, total_requests: int = None,
                  mode: str = "fleet", eos_token_id: int = 0x7FFFFFFF, cos_sin=None, device="cuda", num_workers=None, with_head: bool = True,
                  kernel_mode: str = "offline", max_tokens_per_request: int = None, tap_last_layer_input: bool = False,
-                 single_weight_copy: bool = None):
+                 single_weight_copy: bool = None, spec_decode_config=None):
         assert mode in ("fleet", "mpk")
         self.shape, self.w, self.mode = shape, weights, mode
         self.with_head = with_head
@@ -145,7 +145,7 @@ class Qwen3Decoder:
             mode=kernel_mode, world_size=1, mpi_rank=0, num_workers=num_workers, num_local_schedulers=0, num_remote_schedulers=0,
             max_seq_length=max_seq_length, max_num_batched_requests=R, max_num_batched_tokens=B, max_num_pages=self.max_pages,
             page_size=page_size, eos_token_id=eos_token_id, meta_tensors=self.meta, profiler_tensor=None, trace_name=None,
-            spec_decode_config=None, use_cutlass_kernel=False, max_tokens_per_request=max_tokens_per_request,
+            spec_decode_config=spec_decode_config, use_cutlass_kernel=False, max_tokens_per_request=max_tokens_per_request,
             single_weight_copy=single_weight_copy)
         n_pos = max(max_seq_length, 16)
         self.cos, self.sin = cos_sin if cos_sin is not None else rope_tables(shape, n_pos, dev)
@@ -165,6 +165,13 @@ class Qwen3Decoder:
         gang = self.mode == "fleet"
         t = self.t
         x = mpk.attach_input(self.meta["input_tokens"], "input_token")
+        spec, spec_tokens = mpk.spec_decode_config, None
+        if spec is not None:
+            # prompt lookup (the reference's demo/llama3/demo.py:760-770): the n-gram tasks produce the ids the embedding reads
+            all_tokens = mpk.attach_input(self.meta["tokens"], "all_tokens")
+            spec_tokens = mpk.draft_forward_layer_dispatcher(spec_decode_config=spec, tokens=all_tokens, grid_dim=(96, 1, 1), block_dim=(128, 1, 1))
+            x = spec_tokens
+            t["spec_tokens"] = spec_tokens
         cos = mpk.attach_input(self.cos, "cos_position_embedding")
         sin = mpk.attach_input(self.sin, "sin_position_embedding")
         new = lambda name, cols, dt=mi.bfloat16: mpk.new_tensor(dims=(B, cols), dtype=dt, name=name, io_category="cuda_tensor")
@@ -302,6 +309,9 @@ class Qwen3Decoder:
         mpk.linear_layer(input=rmsnorm_out, weight=w_lm, output=argmax_in, grid_dim=(argmax_tasks, 1, 1), block_dim=(128, 1, 1))
         mpk.argmax_partial_layer(input=argmax_in, output=(argmax_part_value, argmax_part_index), grid_dim=(argmax_tasks, 1, 1), block_dim=(128, 1, 1))
         mpk.argmax_reduce_layer(input=(argmax_part_value, argmax_part_index), output=argmax_out, grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
+        if spec_tokens is not None:
+            t["verify_out"] = mpk.verify_layer_dispatcher(spec_decode_config=spec, spec_tokens=spec_tokens, target_output=argmax_out,
+                                                          grid_dim=(1, 1, 1), block_dim=(128, 1, 1))
 
     # ------------------------------------------------------------------ running
     def load_prompts(self, prompts):

@@ -8,7 +8,8 @@ from .kernel import (DTensor, KNGraph, bfloat16, convert_dtype_to_torch_type, co
                      float32, int32, int64, uint64)
 from . import mpk
 from .mpk.persistent_kernel import PersistentKernel
+from .mpk import speculative
 from .utils import get_configurations_from_gpu
 
 __all__ = ["PersistentKernel", "DTensor", "KNGraph", "dtype", "bfloat16", "float16", "float32", "int32", "int64", "uint64",
-           "get_configurations_from_gpu", "mpk", "convert_torch_type_to_dtype", "convert_dtype_to_torch_type"]
+           "get_configurations_from_gpu", "mpk", "speculative", "convert_torch_type_to_dtype", "convert_dtype_to_torch_type"]

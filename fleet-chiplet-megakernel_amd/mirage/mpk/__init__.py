@@ -2,11 +2,7 @@
 from .persistent_kernel import PersistentKernel
 from .mpk import MPK, MPKMetadata
 from .models import MirageModelConfig
+from . import speculative
+from .speculative import spec_decode_class
 
-
-def spec_decode_class(method, **kwargs):
-    """Speculative decoding is outside the decode megakernel's scope; only `None` is accepted
-    (reference: python/mirage/mpk/speculative.py)."""
-    if method is None:
-        return None
-    raise NotImplementedError(f"speculative decoding method '{method}' is not supported by the MI355X megakernel")
+__all__ = ["MPK", "MPKMetadata", "spec_decode_class", "PersistentKernel", "MirageModelConfig", "speculative"]

@@ -14,7 +14,7 @@ import sys
 import torch
 
 from .. import _capi
-from ..kernel import DTensor, KNGraph, bfloat16, convert_torch_type_to_dtype
+from ..kernel import DTensor, KNGraph, bfloat16, convert_torch_type_to_dtype, int64
 
 # the reference spells the multi-turn mode "online_multi_turn" (persistent_kernel.py:132); "multi_turn" is kept as an alias
 valid_persistent_kernel_modes = ["offline", "online", "online_notoken", "onepass", "online_multi_turn", "multi_turn"]
@@ -67,7 +67,14 @@ class PersistentKernel:
         if world_size != 1 or mpi_rank != 0:
             raise NotImplementedError("the MI355X megakernel runs on one GPU (world_size=1, mpi_rank=0)")
         if spec_decode_config is not None:
-            raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
+            if getattr(spec_decode_config, "method", None) != "promptlookup":
+                # (the reference registers handlers for prompt lookup only, persistent_kernel.py:410-415)
+                raise NotImplementedError(f"speculative decoding method '{getattr(spec_decode_config, 'method', spec_decode_config)}' has no tasks; supported: promptlookup")
+            if mode != "offline":
+                raise NotImplementedError("speculative decoding needs mode 'offline': the on-GPU scheduler sizes the token groups of decoding requests")
+            need = spec_decode_config.spec_length + 1
+            if max_num_batched_tokens < need or self.max_tokens_per_request < need:
+                raise ValueError(f"prompt lookup with {spec_decode_config.spec_length} guesses needs max_num_batched_tokens and max_tokens_per_request >= {need}")
         self.mode = mode
         self.world_size = world_size
         self.mpi_rank = mpi_rank
@@ -85,7 +92,9 @@ class PersistentKernel:
         self._profiler_attached = False
         self.trace_name = trace_name
         self.use_nvshmem = False
-        self.spec_decode_config = None
+        self.spec_decode_config = spec_decode_config
+        self._spec_decode_handlers = {"promptlookup": self.prompt_lookup_spec_handler}
+        self._spec_verify_handlers = {"promptlookup": self.prompt_lookup_verify_handler}
         self.use_cutlass_kernel = False
         self.is_rocm = True
         self.target_cc = 94  # the reference's tag for its MI300/MI350 task set (persistent_kernel.py:425-427)
@@ -639,14 +648,83 @@ class PersistentKernel:
     def allreduce_layer(self, *args, **kwargs):
         raise NotImplementedError("allreduce_layer: the MI355X megakernel runs on one GPU")
 
-    def draft_forward_layer_dispatcher(self, *args, **kwargs):
-        raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
+    # ------------------------------------------------------------------ prompt-lookup speculative decoding
+    def find_ngram_partial_layer(self, input: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple, ngram_size: int = 3):
+        """persistent_kernel.py:2279.  input = the `tokens` meta tensor; output[slot, task] = the earliest position in the
+        task's share of the request's history where its last `ngram_size` tokens occurred before (int64 max: nowhere)."""
+        assert input.num_dims == 2  # (requests, seq_len)
+        assert output.num_dims == 2  # (batch slots, num_tasks)
+        self._task("find_ngram_partial", grid_dim, block_dim, [(input, _REPL, -1), (output, (1, -1, -1), -1)], [ngram_size])
 
-    def verify_layer_dispatcher(self, *args, **kwargs):
-        raise NotImplementedError("speculative decoding is not supported by the MI355X megakernel")
+    def find_ngram_global_layer(self, input: tuple, output: DTensor, grid_dim: tuple, block_dim: tuple, ngram_size: int = 3, spec_length: int = 5):
+        """persistent_kernel.py:2290.  output = the token ids of the iteration's rows: the scheduler's, and behind a decoding
+        request's newest token the `spec_length` tokens that followed the earliest match (-1 where there are none)."""
+        assert len(input) == 2
+        partial_results, tokens = input
+        assert partial_results.num_dims == 2  # (batch slots, num_tasks)
+        assert tokens.num_dims == 2
+        assert output.num_dims == 2
+        self._task("find_ngram_global", grid_dim, block_dim, [(partial_results, _REPL, -1), (tokens, _REPL, -1), (output, _REPL, -1)],
+                   [ngram_size, spec_length])
 
-    def single_batch_extend_attention_layer(self, *args, **kwargs):
-        raise NotImplementedError("single_batch_extend_attention_layer belongs to speculative decoding, which the MI355X megakernel does not support")
+    def prompt_lookup_spec_handler(self, spec_decode_config, tokens: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2305: the two n-gram tasks; returns the tensor the embedding layer reads its ids from.
+        Sized for every token row of an iteration (the reference sizes it for its single request: [1, spec_length + 1])."""
+        slots = max(tokens.dim(0), self.max_num_batched_requests)
+        partial_ngram_output = self.new_tensor(dims=(slots, 96), dtype=int64, name="partial_ngram_output", io_category="cuda_tensor")
+        self.find_ngram_partial_layer(input=tokens, output=partial_ngram_output, grid_dim=grid_dim, block_dim=block_dim,
+                                      ngram_size=spec_decode_config.ngram_size)
+        width = spec_decode_config.spec_length + 1
+        rows = max(tokens.dim(0), -(-self.max_num_batched_tokens // width))  # one id per token row of an iteration, row-major
+        spec_tokens = self.new_tensor(dims=(rows, width), dtype=int64, name="spec_tokens", io_category="cuda_tensor")
+        self.find_ngram_global_layer(input=(partial_ngram_output, tokens), output=spec_tokens, grid_dim=(1, 1, 1), block_dim=(128, 1, 1),
+                                     ngram_size=spec_decode_config.ngram_size, spec_length=spec_decode_config.spec_length)
+        return spec_tokens
+
+    def draft_forward_layer_dispatcher(self, spec_decode_config, tokens: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2341."""
+        handler = self._spec_decode_handlers.get(spec_decode_config.method)
+        if handler is None:
+            raise ValueError(f"Invalid spec decode method: {spec_decode_config.method}")
+        return handler(spec_decode_config, tokens, grid_dim, block_dim)
+
+    def target_verify_greedy_layer(self, input: tuple, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2354.  Counts, per decoding request, the sampled tokens it keeps (1 + the leading guesses the
+        model agreed with) into the num_new_tokens meta tensor; `output` receives batch slot 0's count."""
+        assert len(input) == 2
+        spec_tokens, target_tokens = input
+        assert spec_tokens.num_dims == 2 and target_tokens.num_dims == 2 and output.num_dims == 2
+        self._task("target_verify_greedy", grid_dim, block_dim, [(spec_tokens, _REPL, -1), (target_tokens, _REPL, -1), (output, _REPL, -1)])
+
+    def prompt_lookup_verify_handler(self, spec_decode_config, spec_tokens: DTensor, target_output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:2370."""
+        verify_out = self.new_tensor(dims=(1, 1), dtype=int64, name="verify_out", io_category="cuda_tensor")
+        self.target_verify_greedy_layer(input=(spec_tokens, target_output), output=verify_out, grid_dim=grid_dim, block_dim=block_dim)
+        return verify_out
+
+    def verify_layer_dispatcher(self, spec_decode_config, spec_tokens: DTensor, target_output: DTensor, grid_dim: tuple = (1, 1, 1),
+                                block_dim: tuple = (128, 1, 1)):
+        """persistent_kernel.py:2389."""
+        handler = self._spec_verify_handlers.get(spec_decode_config.method)
+        if handler is None:
+            raise ValueError(f"Invalid spec decode method: {spec_decode_config.method}")
+        return handler(spec_decode_config, spec_tokens, target_output, grid_dim, block_dim)
+
+    def single_batch_extend_attention_layer(self, input: DTensor, k_cache: DTensor, v_cache: DTensor, q_norm: DTensor, k_norm: DTensor,
+                                            cos_pos_embed: DTensor, sin_pos_embed: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple):
+        """persistent_kernel.py:653: attention over the rows of a speculating request (its newest token and the guesses
+        behind it, causal among themselves), caches [requests, seq_len, kv_heads, head_dim].  The attention stage handles
+        several new rows of one request in any case, so this lowers like attention_layer."""
+        assert input.num_dims == 2 and output.num_dims == 2
+        assert k_cache.num_dims == 4 and v_cache.num_dims == 4
+        head_dim, num_kv_heads = k_cache.dim(3), k_cache.dim(2)
+        num_q_heads = output.dim(1) // head_dim
+        qk_norm, rotary_embed = self._attn_flags(q_norm, k_norm, cos_pos_embed, sin_pos_embed, head_dim)
+        assert k_cache.dim(1) == self.page_size, "single_batch_extend_attention_layer: one page per request (page_size == the cache's seq_len)"
+        self._task("single_batch_extend_attention", grid_dim, block_dim,
+                   [(input, (0, 1, -1), -1), (k_cache, (0, 2, -1), 1), (v_cache, (0, 2, -1), 1), (q_norm, _REPL, -1), (k_norm, _REPL, -1),
+                    (cos_pos_embed, _REPL, -1), (sin_pos_embed, _REPL, -1), (output, (0, 1, -1), -1)],
+                   [num_q_heads, num_kv_heads, qk_norm, rotary_embed, input.dim(0) - 1, output.dim(1)])
 
     # ------------------------------------------------------------------ attention variants that lower to the same stage
     def _attn_flags(self, q_norm, k_norm, cos_pos_embed, sin_pos_embed, head_dim):

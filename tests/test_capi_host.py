@@ -71,8 +71,17 @@ def test_constructor_contract():
     mpk = mi.PersistentKernel(mode="offline", **kw)
     assert mpk.total_num_requests == 2 and mpk.target_cc == 94 and mpk.max_num_batched_tokens == 4
     assert mi.mpk.spec_decode_class(None, ngram_size=3, spec_length=4) is None
-    with pytest.raises(NotImplementedError):
-        mi.mpk.spec_decode_class("promptlookup")
+    # prompt lookup is the one speculative method with tasks behind it (persistent_kernel.py:410-415); it needs the offline
+    # scheduler and room for the guesses in an iteration
+    pl = mi.mpk.spec_decode_class("promptlookup", ngram_size=3, spec_length=3)
+    with pytest.raises(NotImplementedError, match="lookahead"):
+        mi.PersistentKernel(mode="offline", **{**kw, "spec_decode_config": mi.mpk.spec_decode_class("lookahead", 3, 3)})
+    with pytest.raises(NotImplementedError, match="offline"):
+        mi.PersistentKernel(mode="online_notoken", **{**kw, "spec_decode_config": pl})
+    with pytest.raises(ValueError, match="max_num_batched_tokens"):
+        mi.PersistentKernel(mode="offline", **{**kw, "spec_decode_config": mi.mpk.spec_decode_class("promptlookup", 3, 5)})
+    sp = mi.PersistentKernel(mode="offline", **{**kw, "spec_decode_config": pl})
+    assert sp.spec_decode_config is pl
 
 
 def test_tensor_api_and_shape_errors():
@@ -432,9 +441,13 @@ def test_every_attention_flavour_lowers_to_one_stage():
                                                 q_workspace=t["qws"], attention_params=(nq, 1, nq * D))
     with pytest.raises(_capi.MkError, match="fewer than max_num_pages"):
         program(small_cache)
-    m = _host_mpk()
-    with pytest.raises(NotImplementedError, match="speculative"):
-        m.single_batch_extend_attention_layer()
+
+    def extend(mpk):  # the speculating request's rows (persistent_kernel.py:653): the cache form with one page per request
+        t = _attn_tensors(mpk)
+        mpk.single_batch_extend_attention_layer(input=t["qkv"], k_cache=t["kc"], v_cache=t["vc"], q_norm=t["qn"], k_norm=t["kn"],
+                                                cos_pos_embed=t["cos"], sin_pos_embed=t["sin"], output=t["out"], grid_dim=(1, nkv, 1), block_dim=(128, 1, 1))
+    p = program(extend)
+    assert len(p) == 1 and p[0].startswith("ATTN qkv -> attn_out") and "norm=1 rope=1" in p[0]
 
 
 def test_split_k_pair_and_fused_activation_lower_to_linear_stages():
