@@ -135,8 +135,8 @@ def cpu_baseline_extrapolated(shape, n_layers_sample=2, steps=3, context=80):
 # excess at BS=1, where K/V is all there is besides the weights) give the per-step part -- weights, activations,
 # K-slice partials written and read back --, and the K/V rows of THIS launch's contexts are added to it.  A model, depth
 # or batch size without a committed counter pass reports null.
-MEASURED_PER_STEP_BYTES_EXCL_KV = {("qwen3-8b", 36, 1): (15.6246e12 + 15.74e9 - 623104 * 147456) / 1024,
-                                   ("qwen3-8b", 36, 64): (25.8955e12 + 1.4045e12 - (24.192e12 - 1024 * 15136194560)) / 1024}
+MEASURED_PER_STEP_BYTES_EXCL_KV = {("qwen3-8b", 36, 1): (15.6246e12 + 15.75e9 - 623104 * 147456) / 1024,
+                                   ("qwen3-8b", 36, 64): (25.9037e12 + 1.4046e12 - (24191940165632 - 1024 * 15136194560)) / 1024}
 
 
 def print_stage_profile(dec, B, out=sys.stderr):

@@ -349,13 +349,22 @@ def main():
     ap.add_argument("--num-layers", type=int, default=36)
     ap.add_argument("--mode", choices=["fleet", "mpk"], default="fleet")
     ap.add_argument("--model", choices=["qwen3-8b", "qwen3-30b-a3b"], default="qwen3-8b")
+    ap.add_argument("--spec-decode", choices=["promptlookup"], default=None,
+                    help="prompt-lookup speculative decoding: a decoding request also runs the tokens that followed the earliest earlier "
+                         "occurrence of its last --ngram-size tokens and keeps those the model agrees with")
+    ap.add_argument("--ngram-size", type=int, default=3)
+    ap.add_argument("--spec-length", type=int, default=5)
     args = ap.parse_args()
     shape = Qwen3Shape(num_layers=args.num_layers) if args.model == "qwen3-8b" else Qwen3Shape.qwen3_30b_a3b(min(args.num_layers, 48))
     B = args.max_num_batched_tokens
     R = args.max_num_batched_requests or B
     max_seq = min(args.max_seq_length, args.prompt_length + args.max_new_tokens + 1)
     w = random_weights(shape, 0)
-    dec = Qwen3Decoder(shape, w, B, R, max_seq, args.page_size, mode=args.mode)
+    spec = mi.mpk.spec_decode_class(args.spec_decode, ngram_size=args.ngram_size, spec_length=args.spec_length)
+    if spec is not None:
+        B = max(B, R * (spec.spec_length + 1))
+    dec = Qwen3Decoder(shape, w, B, R, max_seq, args.page_size, mode=args.mode, spec_decode_config=spec,
+                       max_tokens_per_request=None if spec is None else max(8, spec.spec_length + 1))
     prompts = [torch.randint(0, shape.vocab_size, (args.prompt_length,), generator=torch.Generator().manual_seed(r)) for r in range(R)]
     dec.load_prompts(prompts)
     prefill_iters = math.ceil(args.prompt_length * R / B)
@@ -369,6 +378,10 @@ def main():
     t2 = time.perf_counter()
     st = dec.mpk.stats()
     decode_iters = st["iterations"] - prefill_iters
+    if spec is not None:
+        new_tokens = int((dec.meta["step"].cpu() - args.prompt_length).clamp(min=0).sum())
+        print(f"prompt lookup (n-gram {spec.ngram_size}, {spec.spec_length} guesses): {new_tokens} tokens in {st['iterations']} iterations "
+              f"({new_tokens / max(1, decode_iters):.2f} per decode iteration), {new_tokens / max(1e-9, t2 - t1):.0f} tokens/s")
     print(f"prefill: {prefill_iters} iterations in {(t1 - t0) * 1e3:.1f} ms; decode: {decode_iters} iterations in {(t2 - t1) * 1e3:.1f} ms "
           f"({(t2 - t1) * 1e3 / max(1, decode_iters):.3f} ms/token at BS={R}); finished={done}")
 
