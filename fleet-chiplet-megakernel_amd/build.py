@@ -1,6 +1,7 @@
 """Build libfleet_mk.so (HIP kernel + C-ABI host library) for gfx950 with hipcc.
 
-Usage: python build.py            (from anywhere; output lands next to this file)
+Usage: python build.py            (from anywhere; output lands next to this file: the library, then the Cython binding
+                                   mirage/_cython/core.*.so that links against it)
 """
 import os
 import shutil
@@ -40,7 +41,29 @@ def build(verbose: bool = True, defines=(), out: str = None) -> str:
     return lib
 
 
+def build_cython(verbose: bool = True) -> str:
+    """Compile the Cython binding (mirage/_cython/core.pyx -> core.<abi>.so) against include/fleet_mk.h and link it to the
+    library next to this file.  Needs the library to be built first."""
+    import sysconfig
+    cy_dir = os.path.join(HERE, "mirage", "_cython")
+    c_file = os.path.join(cy_dir, "core.c")
+    out = os.path.join(cy_dir, "core" + sysconfig.get_config_var("EXT_SUFFIX"))
+    steps = [
+        [sys.executable, "-m", "cython", "-3", "--module-name", "mirage._cython.core", "core.pyx", "-o", c_file],
+        [shutil.which("gcc") or "gcc", "-O2", "-fPIC", "-shared", "-Wno-unused-function", "-I" + sysconfig.get_paths()["include"],
+         "-I" + os.path.join(os.path.dirname(HERE), "include"), c_file, "-o", out, "-L" + HERE, "-lfleet_mk", "-Wl,-rpath,$ORIGIN/../.."],
+    ]
+    for cmd in steps:
+        if verbose:
+            print(" ".join(cmd), flush=True)
+        res = subprocess.run(cmd, cwd=cy_dir, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
+        if res.returncode != 0:
+            raise RuntimeError("building the Cython binding failed:\n" + res.stdout)
+    return out
+
+
 if __name__ == "__main__":
     build()
     print("built", LIB)
+    print("built", build_cython())
     sys.exit(0)

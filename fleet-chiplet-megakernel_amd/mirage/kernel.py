@@ -67,7 +67,7 @@ class DTensor:
         return self._dims
 
     def data_ptr(self):
-        return _capi.load().mk_tensor_ptr(self._graph._handle, self.id)
+        return self._graph._g.tensor_ptr(self.id) or None
 
     def to_torch(self):
         """A torch view of this tensor's device memory (library-owned tensors included)."""
@@ -90,11 +90,10 @@ class KNGraph:
         return self._owner._handle
 
     def generate_task_graph(self, num_gpus: int, my_gpu_id: int):
-        out = ctypes.c_char_p()
-        _capi.check(_capi.load().mk_generate_task_graph(self.handle, num_gpus, my_gpu_id, ctypes.byref(out)))
+        json_text = self._owner._g.generate_task_graph(num_gpus, my_gpu_id)
         note = ("// The MI355X decode megakernel is precompiled (libfleet_mk.so) and data-driven:\n"
                 "// no per-graph source is generated.  Stage program:\n")
-        return {"json_file": out.value.decode(), "cuda_code": note + "// " + self._owner.describe_program().replace("\n", "\n// ")}
+        return {"json_file": json_text, "cuda_code": note + "// " + self._owner.describe_program().replace("\n", "\n// ")}
 
     def _torch_view(self, t):
         return self._owner._torch_view(t)

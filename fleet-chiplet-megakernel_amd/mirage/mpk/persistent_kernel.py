@@ -47,13 +47,15 @@ class PersistentKernel:
         eos_token_id: int = -1,
         max_tokens_per_request: int = None,
         single_weight_copy: bool = None,
+        binding: str = None,
     ):
         """Arguments as the reference constructor (persistent_kernel.py:368-387).  `max_tokens_per_request` is the
         reference's compile-time MPK_MAX_TOKENS_PER_REQUEST (prompt tokens one request ingests per iteration; 8 on AMD,
         persistent_kernel.cuh:115-124): None takes the environment variable of that name, else 8; at most 64.
         `single_weight_copy` (no counterpart in the reference; None takes FLEET_MK_SINGLE_WEIGHT_COPY, else False): a graph
         with max_num_batched_tokens >= 2 then keeps every linear weight ONCE, in the matrix-core tile layout compile()
-        makes; `release_row_major_weights()` afterwards drops the attached tensors nothing reads any more."""
+        makes; `release_row_major_weights()` afterwards drops the attached tensors nothing reads any more.
+        `binding`: "ctypes" or "cython" -- which binding of the C ABI carries the calls (None: FLEET_MK_BINDING, else ctypes)."""
         self.__finalized__ = False
         self._is_compiled = False
         self._handle = None
@@ -124,38 +126,24 @@ class PersistentKernel:
         # but compile() / __call__ raise -- the megakernel has no CPU path
         self.host_only = device.type != "cuda"
         self.device = device
-        lib = _capi.load()
-        cfg = _capi.MkConfig()
-        cfg.num_workers = int(num_workers) if num_workers else 0
-        cfg.max_seq_length = max_seq_length
-        cfg.max_num_batched_requests = max_num_batched_requests
-        cfg.max_num_batched_tokens = max_num_batched_tokens
-        cfg.max_num_pages = max_num_pages
-        cfg.page_size = page_size
-        cfg.total_num_requests = self.total_num_requests
-        cfg.device = -1 if self.host_only else (device.index if device.index is not None else torch.cuda.current_device())
-        cfg.eos_token_id = int(eos_token_id)
-        cfg.rms_eps = 1e-6
-        cfg.mode = _capi.MK_MODES[mode]
-        cfg.max_tokens_per_request = self.max_tokens_per_request
         if single_weight_copy is None:
             single_weight_copy = os.environ.get("FLEET_MK_SINGLE_WEIGHT_COPY", "0") not in ("", "0")
         self.single_weight_copy = bool(single_weight_copy)
-        cfg.flags = _capi.MK_CFG_SINGLE_WEIGHT_COPY if self.single_weight_copy else 0
-        cfg.step = mt["step"].data_ptr()
-        cfg.tokens = mt["tokens"].data_ptr()
-        cfg.input_tokens = mt["input_tokens"].data_ptr()
-        cfg.output_tokens = mt["output_tokens"].data_ptr()
-        cfg.num_new_tokens = mt["num_new_tokens"].data_ptr()
-        cfg.prompt_lengths = mt["prompt_lengths"].data_ptr()
-        cfg.qo_indptr = mt["qo_indptr_buffer"].data_ptr()
-        cfg.paged_kv_indptr = mt["paged_kv_indptr_buffer"].data_ptr()
-        cfg.paged_kv_indices = mt["paged_kv_indices_buffer"].data_ptr()
-        cfg.paged_kv_last_page_len = mt["paged_kv_last_page_len_buffer"].data_ptr()
-        handle = ctypes.c_void_p()
-        _capi.check(lib.mk_graph_create(ctypes.byref(cfg), ctypes.byref(handle)))
-        self._handle = handle
-        self._lib = lib
+        cfg = dict(
+            num_workers=int(num_workers) if num_workers else 0, max_seq_length=max_seq_length, max_num_batched_requests=max_num_batched_requests,
+            max_num_batched_tokens=max_num_batched_tokens, max_num_pages=max_num_pages, page_size=page_size,
+            total_num_requests=self.total_num_requests,
+            device=-1 if self.host_only else (device.index if device.index is not None else torch.cuda.current_device()),
+            eos_token_id=int(eos_token_id), rms_eps=1e-6, mode=_capi.MK_MODES[mode], max_tokens_per_request=self.max_tokens_per_request,
+            flags=_capi.MK_CFG_SINGLE_WEIGHT_COPY if self.single_weight_copy else 0,
+            step=mt["step"].data_ptr(), tokens=mt["tokens"].data_ptr(), input_tokens=mt["input_tokens"].data_ptr(),
+            output_tokens=mt["output_tokens"].data_ptr(), num_new_tokens=mt["num_new_tokens"].data_ptr(),
+            prompt_lengths=mt["prompt_lengths"].data_ptr(), qo_indptr=mt["qo_indptr_buffer"].data_ptr(),
+            paged_kv_indptr=mt["paged_kv_indptr_buffer"].data_ptr(), paged_kv_indices=mt["paged_kv_indices_buffer"].data_ptr(),
+            paged_kv_last_page_len=mt["paged_kv_last_page_len_buffer"].data_ptr())
+        # the C ABI through the ctypes binding, or through the compiled Cython one (FLEET_MK_BINDING=cython / binding=)
+        self._g = _capi.make_graph(cfg, binding)
+        self._handle = ctypes.c_void_p(self._g.handle)  # for callers that talk to the C ABI directly
         self.kn_graph = KNGraph(self)
         self._tensors = []
 
@@ -169,9 +157,7 @@ class PersistentKernel:
         dt = convert_torch_type_to_dtype(torch_tensor.dtype)
         if (torch_tensor.device.type != "cuda") != self.host_only:
             raise RuntimeError(f"{name}: attached tensors must live on the same kind of device as the meta tensors")
-        tid = _capi.check(self._lib.mk_tensor_attach(
-            self._handle, ctypes.c_void_p(torch_tensor.data_ptr()), len(dims), _capi.int_array(dims, ctypes.c_int64),
-            _capi.int_array(strides, ctypes.c_int64), dt.code, name.encode()))
+        tid = self._g.tensor_attach(torch_tensor.data_ptr(), dims, strides, dt.code, name)
         t = DTensor(self, tid, dims, dt, name, torch_tensor)
         self._tensors.append(t)
         return t
@@ -186,9 +172,7 @@ class PersistentKernel:
         else:
             raise RuntimeError(f"Invalid io_category: {io_category}")
         dims = tuple(int(d) for d in dims)
-        sp = _capi.int_array(strides, ctypes.c_int64) if strides is not None else None
-        tid = _capi.check(self._lib.mk_tensor_new(self._handle, len(dims), _capi.int_array(dims, ctypes.c_int64), sp,
-                                                  dtype.code, name.encode(), cat))
+        tid = self._g.tensor_new(dims, None if strides is None else tuple(int(x) for x in strides), dtype.code, name, cat)
         t = DTensor(self, tid, dims, dtype, name)
         t._strides = tuple(strides) if strides is not None else None
         self._tensors.append(t)
@@ -196,8 +180,7 @@ class PersistentKernel:
 
     def _shuffle(self, inputs, dim, num_groups, name, interleave):
         ids = [t.id for t in inputs]
-        tid = _capi.check(self._lib.mk_tensor_shuffle(self._handle, _capi.int_array(ids), len(ids), dim, num_groups,
-                                                      1 if interleave else 0, (name or "shuffled").encode()))
+        tid = self._g.tensor_shuffle(ids, dim, num_groups, bool(interleave), name or "shuffled")
         rows = sum(t.dim(0) for t in inputs)
         t = DTensor(self, tid, (rows,) + tuple(inputs[0].shape[1:]), inputs[0].dtype, name)
         t.sources = list(inputs)
@@ -213,7 +196,7 @@ class PersistentKernel:
         return self._shuffle(inputs, shuffled_dim, num_groups, name, True)
 
     def _torch_view(self, t: DTensor):
-        ptr = self._lib.mk_tensor_ptr(self._handle, t.id)
+        ptr = self._g.tensor_ptr(t.id)
         if not ptr:
             raise RuntimeError(f"tensor {t.name} has no device storage (shuffled views are resolved at run time)")
         n = 1
@@ -240,9 +223,7 @@ class PersistentKernel:
             maps.extend(int(x) for x in m)
             fl.append(int(f))
         params = [int(p) for p in params]
-        _capi.check(self._lib.mk_add_task(self._handle, name.encode(), _capi.int_array(grid_dim), _capi.int_array(block_dim),
-                                          len(ids), _capi.int_array(ids), _capi.int_array(maps), _capi.int_array(fl),
-                                          len(params), _capi.int_array(params)))
+        self._g.add_task(name, grid_dim, block_dim, ids, maps, fl, params)
 
     # ------------------------------------------------------------------ layers (reference line numbers in each docstring)
     def embed_layer(self, input: DTensor, weight: DTensor, output: DTensor, grid_dim: tuple, block_dim: tuple, input_source: int = 0):
@@ -811,15 +792,13 @@ class PersistentKernel:
 
     # ------------------------------------------------------------------ compile / run
     def describe_program(self) -> str:
-        out = ctypes.c_char_p()
-        _capi.check(self._lib.mk_describe_program(self._handle, ctypes.byref(out)))
-        return out.value.decode()
+        return self._g.describe_program()
 
     def compile(self, **kwargs):
         """persistent_kernel.py:2404.  Lowers the recorded tasks and uploads descriptors; nothing is compiled at run time."""
         assert not self._is_compiled
         output_dir = kwargs.get("output_dir", None)
-        _capi.check(self._lib.mk_compile(self._handle))
+        self._g.compile()
         self._is_compiled = True
         if self._profiler_tensor is not None:
             self._attach_profiler()
@@ -847,11 +826,11 @@ class PersistentKernel:
     def _attach_profiler(self):
         t = self._profiler_tensor
         if t is None:
-            _capi.check(self._lib.mk_set_profiler(self._handle, None, 0))
+            self._g.set_profiler(0, 0)
             self._profiler_attached = False
             return
         assert t.is_cuda and t.dtype in (torch.uint64, torch.int64) and t.dim() == 1 and t.is_contiguous(), "the profiler tensor is a flat uint64 device tensor"
-        _capi.check(self._lib.mk_set_profiler(self._handle, ctypes.c_void_p(t.data_ptr()), t.numel()))
+        self._g.set_profiler(t.data_ptr(), t.numel())
         self._profiler_attached = True
 
     @staticmethod
@@ -868,7 +847,7 @@ class PersistentKernel:
         """persistent_kernel.py:2622: run every request to completion in one persistent launch (blocking)."""
         assert self._is_compiled, "call compile() first"
         sp = self._stream_ptr(kwargs.get("default_stream", None))
-        _capi.check(self._lib.mk_launch(self._handle, ctypes.c_void_p(sp)))
+        self._g.launch(sp)
         if self.profiler_tensor is not None:
             self.export_profile()
 
@@ -885,22 +864,17 @@ class PersistentKernel:
 
     def init_request_resources(self):
         """Reset step[], batch slots and the page ring (reference: init_request_func, persistent_kernel.py:63-68)."""
-        _capi.check(self._lib.mk_init_requests(self._handle))
+        self._g.init_requests()
 
     def run_steps(self, max_iterations: int, default_stream=None) -> bool:
         """Run at most `max_iterations` decode iterations; returns True when all requests have finished."""
-        fin = ctypes.c_int(0)
-        sp = self._stream_ptr(default_stream)
-        _capi.check(self._lib.mk_launch_steps(self._handle, ctypes.c_void_p(sp), int(max_iterations), ctypes.byref(fin)))
-        return bool(fin.value)
+        return self._g.launch_steps(self._stream_ptr(default_stream), int(max_iterations))
 
     def enqueue_steps(self, max_iterations: int, default_stream=None):
-        _capi.check(self._lib.mk_enqueue_steps(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), int(max_iterations)))
+        self._g.enqueue_steps(self._stream_ptr(default_stream), int(max_iterations))
 
     def wait(self, default_stream=None) -> bool:
-        fin = ctypes.c_int(0)
-        _capi.check(self._lib.mk_wait(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), ctypes.byref(fin)))
-        return bool(fin.value)
+        return self._g.wait(self._stream_ptr(default_stream))
 
     def run_once(self, tok_slot, tok_pos, tok_first=None, default_stream=None):
         """Host-driven single pass over the stage program (onepass mode): row t belongs to batch slot tok_slot[t] at
@@ -913,15 +887,13 @@ class PersistentKernel:
                     tok_first.append(tok_first[-1])
                 else:
                     tok_first.append(t)
-        i32 = ctypes.c_int32
-        _capi.check(self._lib.mk_run_once(self._handle, ctypes.c_void_p(self._stream_ptr(default_stream)), n,
-                                          _capi.int_array(tok_slot, i32), _capi.int_array(tok_pos, i32), _capi.int_array(tok_first, i32)))
+        self._g.run_once(self._stream_ptr(default_stream), [int(x) for x in tok_slot], [int(x) for x in tok_pos], [int(x) for x in tok_first])
 
     def repack_weights(self):
         """Refresh the library's matrix-core copies of the linear weights after attached weight tensors were overwritten
         (graphs with max_num_batched_tokens > 8 stream a tile-ordered copy made at compile time).  Not in the reference,
         whose kernels read the attached tensors in place."""
-        _capi.check(self._lib.mk_repack_weights(self._handle))
+        self._g.repack_weights()
 
     def release_row_major_weights(self) -> list:
         """After compile() of a graph built with single_weight_copy: drop this object's references to the attached weight
@@ -930,15 +902,13 @@ class PersistentKernel:
         assert self._is_compiled, "compile() first"
         released = []
         for t in self._tensors:
-            if t.torch_tensor is not None and _capi.check(self._lib.mk_tensor_releasable(self._handle, t.id)) == 1:
+            if t.torch_tensor is not None and self._g.tensor_releasable(t.id):
                 released.append(t.name)
                 t.torch_tensor = None
         return released
 
     def stats(self) -> dict:
-        st = _capi.MkStats()
-        _capi.check(self._lib.mk_get_stats(self._handle, ctypes.byref(st)))
-        return {name: getattr(st, name) for name, _ in st._fields_}
+        return self._g.stats()
 
     def stage_profile(self, workgroup: int = 0, raw: bool = False, marks: bool = False):
         """Per-stage timing of the last iteration on one virtual workgroup: list of (description, entered,
@@ -947,19 +917,17 @@ class PersistentKernel:
         step that opened the iteration: (previous iteration complete, batch prepared [workgroup 0], batch published, 0).
         marks=True returns the four in-stage marks of a library built with -DMK_TRACE instead."""
         n = self.stats()["num_stages"] + 1
-        buf = (ctypes.c_int64 * (4 * n))()
-        fn = self._lib.mk_get_stage_marks if marks else self._lib.mk_get_stage_profile
-        got = _capi.check(fn(self._handle, int(workgroup), buf, n))
+        rows = self._g.stage_ticks(int(workgroup), n, bool(marks))
         desc = self.describe_program().splitlines() + ["SCHEDULER"]
         if raw:
-            return [(desc[i], *[int(buf[4 * i + k]) for k in range(4)]) for i in range(got)]
-        t0 = min(buf[4 * i] for i in range(got - 1) if buf[4 * i] > 0) if got > 1 else 0
-        return [(desc[i], *[(buf[4 * i + k] - t0) * 0.01 if buf[4 * i + k] > 0 else -1.0 for k in range(4)]) for i in range(got)]
+            return [(desc[i], *row) for i, row in enumerate(rows)]
+        t0 = min(row[0] for row in rows[:-1] if row[0] > 0) if len(rows) > 1 else 0
+        return [(desc[i], *[(x - t0) * 0.01 if x > 0 else -1.0 for x in row]) for i, row in enumerate(rows)]
 
     def finalize(self):
         assert not self.__finalized__
         if self._handle is not None:
-            self._lib.mk_graph_destroy(self._handle)
+            self._g.destroy()
             self._handle = None
         self.__finalized__ = True
 
