@@ -229,6 +229,14 @@ class Qwen3Builder(GraphBuilder):
         mpk, B = self.mpk, self.mpk.max_num_batched_tokens
         self.with_lm_head = with_lm_head
         self.x = self._attach(self.input_tokens, "input_token")
+        # prompt lookup (what the reference's builder leaves as a TODO at builder.py:719-745,811-816 and its llama demo
+        # does, demo/llama3/demo.py:760-821): the n-gram tasks write the ids the embedding reads, a verify task follows
+        # the sampling
+        spec, spec_tokens = mpk.spec_decode_config, None
+        if spec is not None:
+            all_tokens = self._attach(mpk.meta_tensors["tokens"], "all_tokens")
+            spec_tokens = mpk.draft_forward_layer_dispatcher(spec_decode_config=spec, tokens=all_tokens, grid_dim=(96, 1, 1), block_dim=(128, 1, 1))
+            self.x = spec_tokens
         cos, sin = self.position_embeddings
         n_pos = min(cos.shape[-2], 4096) if cos.dim() == 3 else cos.shape[0]
         cos2 = (cos[0, :n_pos, :] if cos.dim() == 3 else cos).contiguous()
@@ -251,6 +259,10 @@ class Qwen3Builder(GraphBuilder):
                                      grid_dim=(mpk.num_workers, 1, 1), block_dim=(128, 1, 1))
             mpk.argmax_reduce_layer(input=(self.argmax_part_value, self.argmax_part_index), output=argmax_out, grid_dim=(1, 1, 1),
                                     block_dim=(128, 1, 1))
+            if spec_tokens is not None:
+                self.verify_out = mpk.verify_layer_dispatcher(spec_decode_config=spec, spec_tokens=spec_tokens, target_output=argmax_out)
+        elif spec_tokens is not None:
+            raise ValueError("speculative decoding needs the LM head and the sampling stages in the graph (with_lm_head)")
 
     # ------------------------------------------------------------------ tokenizer pass-through
     def encode(self, text: str):

@@ -19,6 +19,7 @@ from ..utils import get_configurations_from_gpu
 from .model_registry import get_builder
 from .models.graph_builder import MirageModelConfig
 from .persistent_kernel import PersistentKernel
+from .speculative import spec_decode_class
 
 
 @dataclass
@@ -61,7 +62,9 @@ class MPKMetadata:
     profiler_tensor: Optional[torch.Tensor] = None
     trace_name: Optional[str] = None
     # spec decode config
-    spec_decode: Optional[str] = None
+    spec_decode: Optional[str] = None       # "promptlookup": builds `spec_decode_config` from the two numbers below (mpk.py:283-288)
+    ngram_size: int = 3
+    spec_length: int = 5
     spec_decode_config: Optional[object] = None
     use_cutlass_kernel: bool = False
     eos_token_id: Optional[int] = None
@@ -132,6 +135,9 @@ class MPK:
             self.num_workers, self.num_schedulers = get_configurations_from_gpu(dev.index if dev.index is not None else torch.cuda.current_device())
         else:
             self.num_workers, self.num_schedulers = meta.num_workers, max(meta.num_schedulers, 0)
+        if meta.spec_decode_config is None and meta.spec_decode:
+            meta.spec_decode_config = spec_decode_class(meta.spec_decode, ngram_size=meta.ngram_size, spec_length=meta.spec_length)
+        self.spec_decode_config = meta.spec_decode_config
         self.persistent_kernel = PersistentKernel(
             mode=meta.mode, world_size=1, mpi_rank=0, num_workers=self.num_workers, num_local_schedulers=self.num_schedulers,
             num_remote_schedulers=0, max_seq_length=self.max_seq_length, max_num_batched_requests=meta.max_num_batched_requests,

@@ -251,3 +251,36 @@ def test_speculative_generation_equals_plain_greedy():
     assert s_spec.tolist() == s_plain.tolist() == [max_seq - 1] * 2
     assert torch.equal(t_spec, t_plain)
     assert it_spec < it_plain, (it_spec, it_plain)  # accepted guesses save iterations
+
+
+@pytest.mark.gpu
+def test_mpk_wrapper_with_prompt_lookup():
+    """MPKMetadata(spec_decode="promptlookup"): the Qwen3 builder puts the n-gram tasks in front of the embedding and the
+    verify task behind the sampling (the reference's builder leaves this as a TODO, models/qwen3/builder.py:719-745); the
+    generation equals the wrapper's plain run."""
+    from mirage.mpk import MPK
+    from oracle.qwen3_ref import make_model_weights
+    from test_mpk_builder import _cfg, _load_prompts, _metadata
+    cfg = _cfg()
+    w = make_model_weights(cfg, seed=62)
+    R, total, max_seq, PS = 2, 2, 72, 16
+    prompts = _prompts(cfg, 2)
+    runs = {}
+    for spec in (None, "promptlookup"):
+        md = _metadata(cfg, w, "cuda", R=R, T=12, total=total, max_seq=max_seq, PS=PS)
+        md.spec_decode, md.ngram_size, md.spec_length = spec, 2, 5
+        md.max_tokens_per_request = 8
+        mpk = MPK(md)
+        mpk.build()
+        mpk.compile()
+        prog = mpk.persistent_kernel.describe_program()
+        assert ("NGRAM_GLOBAL" in prog and "VERIFY" in prog) == (spec is not None)
+        _load_prompts(mpk, prompts)
+        torch.cuda.synchronize()
+        mpk.init_per_request()
+        mpk()
+        torch.cuda.synchronize()
+        runs[spec] = (mpk.tokens.cpu(), mpk.step.cpu(), mpk.persistent_kernel.stats()["iterations"])
+        mpk.finalize()
+    assert torch.equal(runs[None][0], runs["promptlookup"][0]) and torch.equal(runs[None][1], runs["promptlookup"][1])
+    assert runs["promptlookup"][2] < runs[None][2]
