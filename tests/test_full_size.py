@@ -182,3 +182,33 @@ def test_config5_full_size_properties(capsys, B):
     """48-layer Qwen3-30B-A3B shape (128 experts, top-8), 80-token prompts, 512 new tokens."""
     from demo_qwen3 import Qwen3Shape
     _property_run(capsys, Qwen3Shape.qwen3_30b_a3b(48), B, 80, 512, chunk=29)
+
+
+def test_config4_full_size_bs8_several_pages_per_request(capsys):
+    """36-layer Qwen3-8B shape at B=8: the same generation with one 4096-position page per request and with 64-position
+    pages (six to seven per request, handed out by the on-GPU scheduler as the contexts grow, so the requests' pages
+    interleave) gives the same tokens -- where a K/V row lives must not matter -- and the page tables end as the C
+    restatement of the scheduler predicts."""
+    from demo_qwen3 import Qwen3Decoder, Qwen3Shape, random_weights
+    shape, B, P, new_tokens = Qwen3Shape(), 8, 80, 320
+    max_seq = P + new_tokens + 1
+    _say(capsys, "generating weights (36 layers)")
+    w = random_weights(shape, seed=0)
+    prompts = [torch.randint(0, shape.vocab_size, (P,), generator=torch.Generator().manual_seed(r)) for r in range(B)]
+    runs = {}
+    for ps in (4096, 64):
+        dec = Qwen3Decoder(shape, w, max_num_batched_tokens=B, max_num_batched_requests=B, max_seq_length=max_seq, page_size=ps)
+        _say(capsys, f"page_size {ps}: one persistent launch")
+        toks, steps = dec.generate(prompts)
+        st = dec.mpk.stats()
+        assert st["aborted"] == 0 and all(int(s) == max_seq - 1 for s in steps)
+        ref, iters = _sched_oracle_end_state([P] * B, B, B, dec.max_pages, ps, max_seq)
+        assert st["iterations"] == iters
+        for name, key in (("step", "step"), ("qo_indptr", "qo_indptr_buffer"), ("kv_indptr", "paged_kv_indptr_buffer")):
+            assert dec.meta[key].cpu().tolist() == ref[name].tolist(), (ps, name)
+        runs[ps] = toks
+        dec.mpk.finalize()
+    if not torch.equal(runs[4096], runs[64]):
+        bad = (runs[4096] != runs[64]).nonzero()[0].tolist()
+        raise AssertionError(f"tokens depend on the page size, first at request {bad[0]} position {bad[1]}")
+    _say(capsys, "done\n")
