@@ -2,9 +2,11 @@
  *
  * This is the drop-in boundary for the decode path of mirage's PersistentKernel:
  * the Python front end (fleet-chiplet-megakernel_amd/mirage) binds these entry
- * points with ctypes where the reference binds its C++ graph through Cython
- * (python/mirage/_cython/core.pyx, CCore.pxd:236-253) and its generated launcher
- * through a CPython module (python/mirage/mpk/persistent_kernel.py:17-130).
+ * points twice -- with ctypes (mirage/_capi.py) and with a compiled Cython module
+ * (mirage/_cython/core.pyx over fleet_mk.pxd) -- where the reference binds its C++
+ * graph through Cython (python/mirage/_cython/core.pyx, CCore.pxd:236-253) and its
+ * generated launcher through a CPython module
+ * (python/mirage/mpk/persistent_kernel.py:17-130).
  *
  * Conventions: plain pointers and sizes only; every function returns 0 on success
  * or a negative MK_E* code, and mk_last_error() then returns a description (thread
