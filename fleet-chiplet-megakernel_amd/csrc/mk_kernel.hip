@@ -47,6 +47,9 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_MOE_M1_R2
 #define MK_TUNE_MOE_M1_R2 1   // single-token expert W2: output rows (x 8 experts) in flight per wavefront
 #endif
+#ifndef MK_TUNE_MOE_M1_PARK
+#define MK_TUNE_MOE_M1_PARK 2 // ... and parked in LDS per wavefront while the barrier is awaited
+#endif
 // units per group of the multi-token expert linears (W13 / W2)
 #ifndef MK_TUNE_MOE_R13
 #define MK_TUNE_MOE_R13 4
@@ -2667,13 +2670,33 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
   int ut[R];
 #pragma unroll
   for (int j = 0; j < R; j++) ut[j] = -1;
+  // W2 form after the W13 stage of the same token: the experts are known before the barrier, and a workgroup's whole
+  // share of the weights (a few tickets of TK rows) fits the idle LDS above the routing lists.  Each worker wavefront
+  // keeps its R tickets in flight as a rolling window: a ticket that has landed is parked in LDS and its slot refilled,
+  // NLP tickets per wavefront; they are reduced from LDS once the input rows are there.
+  constexpr int NLP = SILU ? 0 : MK_TUNE_MOE_M1_PARK;
+  constexpr int PARK_OFF = MK_MOE_OFFSET + 8192;
+  static_assert(sizeof(MoeLds) <= 8192, "routing lists overlap the parked rows");
+  static_assert(PARK_OFF + (MK_WAVES - 1) * NLP * NSUB * KL * 1024 <= MK_LDS_BYTES, "parked rows exceed the LDS window");
+  u32x4 *lrows = (u32x4 *)(smem + PARK_OFF) + (size_t)(wave > 0 ? wave - 1 : 0) * (NLP > 0 ? NLP : 1) * NSUB * KL * 64;
+  int lo_[NLP > 0 ? NLP : 1];
+#pragma unroll
+  for (int i = 0; i < (NLP > 0 ? NLP : 1); i++) lo_[i] = -1;
   if (!ctrl) {
     if (reuse) {
       set_bases();
 #pragma unroll
-      for (int j = 0; j < R; j++) {
-        ut[j] = take();
-        if (ut[j] >= 0) load_ticket(ut[j], buf[j]);
+      for (int i = 0; i < NLP + R; i++) {
+        const int sl = i % R;
+        if (i >= R) {
+#pragma unroll
+          for (int h = 0; h < NSUB; h++)
+#pragma unroll
+            for (int kc = 0; kc < KL; kc++) lrows[(((i - R) * NSUB + h) * KL + kc) * 64 + lane] = buf[sl][h][kc];
+          lo_[i - R] = ut[sl];
+        }
+        ut[sl] = take();
+        if (ut[sl] >= 0) load_ticket(ut[sl], buf[sl]);
       }
     }
   } else {
@@ -2763,6 +2786,35 @@ __device__ __forceinline__ void stage_moe_linear_m1(CStage &st, Ctx &c, char *sm
       if (ut[j] >= 0) load_ticket(ut[j], buf[j]);
     }
     ures[j] = (!SILU && ut[j] >= 0) ? bf2f(ldc_u16((const uint16_t *)st.res + ut[j])) : 0.f;
+  }
+  if constexpr (NLP > 0) {
+    // the parked tickets first: no memory traffic, the register slots keep landing meanwhile
+    float lres[NLP];
+#pragma unroll
+    for (int i = 0; i < NLP; i++) lres[i] = lo_[i] >= 0 ? bf2f(ldc_u16((const uint16_t *)st.res + lo_[i])) : 0.f;
+#pragma unroll
+    for (int i = 0; i < NLP; i++) {
+      if (lo_[i] >= 0) {
+        const int tk = lo_[i];
+        float acc[NSUB];
+#pragma unroll
+        for (int h = 0; h < NSUB; h++) {
+          acc[h] = 0.f;
+#pragma unroll
+          for (int kc = 0; kc < KL; kc++) acc[h] = dot8(lrows[((i * NSUB + h) * KL + kc) * 64 + lane], xr[SILU ? 0 : h][kc], acc[h]);
+        }
+#pragma unroll
+        for (int h = 0; h < NSUB; h++) acc[h] = wave_sum(acc[h]);
+        float comb = lres[i];
+#pragma unroll
+        for (int h = 0; h < NSUB; h++) {
+          const uint32_t v = f2bf(acc[h]);
+          if (lane == 0) so[h * n_loc + tk - t_begin] = (uint16_t)v;
+          comb = fmaf(bf2f((uint16_t)v), L->w[SILU ? 0 : h], comb);
+        }
+        if (lane == 0) so[TK * n_loc + tk - t_begin] = (uint16_t)f2bf(comb);
+      }
+    }
   }
   while (true) {
     bool any = false;
