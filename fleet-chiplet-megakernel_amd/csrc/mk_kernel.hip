@@ -47,6 +47,13 @@ typedef const __attribute__((address_space(4))) MkWeight CWeight;
 #ifndef MK_TUNE_MOE_M1_R2
 #define MK_TUNE_MOE_M1_R2 1   // single-token expert W2: output rows (x 8 experts) in flight per wavefront
 #endif
+// multi-token expert linears: cost of a unit's row load relative to one token's reduction (W13 / W2)
+#ifndef MK_TUNE_MOE_ROWCOST13
+#define MK_TUNE_MOE_ROWCOST13 4
+#endif
+#ifndef MK_TUNE_MOE_ROWCOST2
+#define MK_TUNE_MOE_ROWCOST2 3
+#endif
 #ifndef MK_TUNE_MOE_M1_PARK
 #define MK_TUNE_MOE_M1_PARK 2 // ... and parked in LDS per wavefront while the barrier is awaited
 #endif
@@ -2886,23 +2893,25 @@ __device__ __forceinline__ void stage_moe_linear_multi(CStage &st, Ctx &c, int M
   const int n_act = L->n_act;
   const int NR = SILU ? st.n / 2 : st.n;  // units per expert
   const int n_units = n_act * NR;
-  // A unit of expert a costs one row load plus one reduction per token routed to a: split the units so that every
-  // workgroup gets the same cost.  With w_a = tokens(a) + 1 the cost before expert a is NR * (pair_off[a] + a).
+  // A unit of expert a costs one row load (RC, in units of one reduction) plus one reduction per token routed to a: split
+  // the units so that every workgroup gets the same cost.  With w_a = tokens(a) + RC the cost before expert a is
+  // NR * (pair_off[a] + RC * a).
+  constexpr int RC = SILU ? MK_TUNE_MOE_ROWCOST13 : MK_TUNE_MOE_ROWCOST2;
   int *bnd = L->wtot[0];  // reused: the scans of the list building are done
   if (tid < 2) bnd[tid] = 0;
   __syncthreads();
-  const long long total = (long long)NR * (L->pair_off[n_act] + n_act);
+  const long long total = (long long)NR * (L->pair_off[n_act] + RC * n_act);
   const long long tgt0 = total * c.vid / c.G, tgt1 = total * (c.vid + 1) / c.G;
   if (tid < n_act) {
-    const long long before = (long long)NR * (L->pair_off[tid] + tid);
+    const long long before = (long long)NR * (L->pair_off[tid] + RC * tid);
     if (before <= tgt0) __hip_atomic_fetch_max(&bnd[0], tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
     if (before <= tgt1) __hip_atomic_fetch_max(&bnd[1], tid, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_WORKGROUP);
   }
   __syncthreads();
   auto unit_at = [&](long long tgt, int a) -> int {
     if (n_act == 0) return 0;
-    const long long before = (long long)NR * (L->pair_off[a] + a);
-    const int w = L->pair_off[a + 1] - L->pair_off[a] + 1;
+    const long long before = (long long)NR * (L->pair_off[a] + RC * a);
+    const int w = L->pair_off[a + 1] - L->pair_off[a] + RC;
     return a * NR + min(NR, (int)((tgt - before) / w));
   };
   const int u_begin = __builtin_amdgcn_readfirstlane(unit_at(tgt0, bnd[0]));
