@@ -90,9 +90,24 @@ def export_to_perfetto_trace(profiler_buffer: torch.Tensor, file_name: str) -> s
             continue
         tag, ts = wd & 0xFFFFFFFF, (wd >> 32) & 0xFFFFFFFF
         entries.append(decode_tag(tag, num_blocks, num_groups) + (ts,))
-    # entries of one workgroup in the order they were written (begin before end on equal times); times count from the first
-    t0 = min((e[5] for e in entries), default=0)
-    entries = sorted((e[:5] + (e[5] - t0,) for e in entries), key=lambda e: (e[1], e[2], e[5], e[0], e[4]))
+    # The timestamps are the low 32 bits of a ns clock and wrap every 4.3 s.  Within a workgroup time only moves forward
+    # (entries are in the order they were written), so each workgroup's sequence is unwrapped by its forward differences;
+    # its first entry is placed by its signed 32-bit distance to the first entry of the buffer.
+    ref, last, unwrapped = None, {}, []
+    for e in entries:
+        ts, key = e[5], (e[1], e[2])
+        if ref is None:
+            ref = ts
+        if key in last:
+            prev_raw, prev_t = last[key]
+            t = prev_t + ((ts - prev_raw) & 0xFFFFFFFF)
+        else:
+            t = ((ts - ref + (1 << 31)) & 0xFFFFFFFF) - (1 << 31)
+        last[key] = (ts, t)
+        unwrapped.append(e[:5] + (t,))
+    # entries of one workgroup in time order (begin before end on equal times); times count from the earliest
+    t0 = min((e[5] for e in unwrapped), default=0)
+    entries = sorted((e[:5] + (e[5] - t0,) for e in unwrapped), key=lambda e: (e[1], e[2], e[5], e[0], e[4]))
     try:
         from tg4perfetto import TraceGenerator  # the reference's writer
     except ImportError:

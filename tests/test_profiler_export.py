@@ -37,6 +37,31 @@ def test_profiler_tensor_round_trip(tmp_path):
     assert fill_profiler_tensor(small, profiles) == 2
 
 
+def test_export_unwraps_the_32_bit_clock(tmp_path):
+    """The entries hold the low word of a ns clock (profiler.h:42-54), which wraps every 4.3 s: a recording that crosses
+    the wrap exports with times that keep rising within each workgroup."""
+    from mirage.mpk.profiler_persistent import encode_tag, export_to_perfetto_trace
+    G = 2
+    # kernel layout: entry k of workgroup b at 1 + b + k * G; workgroup 1 starts just before the wrap, workgroup 0 after
+    raw = {0: [0xFFFFFF00, 0xFFFFFFF0, 0x00000010, 0x00000400], 1: [0xFFFFFE00, 0xFFFFFF80, 0xFFFFFFFF, 0x00000300]}
+    buf = torch.zeros(1 + 4 * G, dtype=torch.int64)
+    buf[0] = G | (1 << 32)
+    for b in range(G):
+        for k, ts in enumerate(raw[b]):
+            word = encode_tag(k // 2, b, 0, 1, 101 if k < 2 else 102, k & 1) | (ts << 32)
+            buf[1 + b + k * G] = word - (1 << 64) if word >= (1 << 63) else word
+    out = tmp_path / "w.perfetto-trace"
+    if export_to_perfetto_trace(buf.view(torch.uint64), str(out)) != "json":
+        pytest.skip("tg4perfetto writes the protobuf form")
+    ev = [e for e in json.loads(out.read_text())["traceEvents"] if e["ph"] in ("B", "E")]
+    for b in range(G):
+        ts = [e["ts"] for e in ev if e["pid"] == b]
+        assert ts == sorted(ts) and len(ts) == 4
+        assert abs((ts[-1] - ts[0]) * 1000 - ((raw[b][-1] - raw[b][0]) & 0xFFFFFFFF)) < 1e-3  # ns, across the wrap
+    # the earliest entry of the buffer (workgroup 1's first) is time zero, workgroup 0 starts 0x100 ns later
+    assert min(e["ts"] for e in ev) == 0 and abs(min(e["ts"] for e in ev if e["pid"] == 0) * 1000 - 0x100) < 1e-3
+
+
 @pytest.mark.gpu
 def test_profiler_tensor_records_every_iteration(tmp_path):
     """The kernel itself writes the tensor (profiler.h:129-180): every stage of every iteration, workgroup-interleaved."""
@@ -56,6 +81,9 @@ def test_profiler_tensor_records_every_iteration(tmp_path):
     G, iters = st["num_workgroups"], st["iterations"]
     assert iters >= 10
     assert words[0] & 0xFFFFFFFF == G and words[0] >> 32 == 1
+    def after(a, b):  # signed distance a - b of two 32-bit ns timestamps (the clock's low word wraps every 4.3 s)
+        return ((a - b + (1 << 31)) & 0xFFFFFFFF) - (1 << 31)
+
     per_wg = {}
     for i, wd in enumerate(words[1:]):
         if wd == 0:
@@ -69,9 +97,9 @@ def test_profiler_tensor_records_every_iteration(tmp_path):
         assert len(ent) == n0 and n0 % 2 == 0  # every workgroup passes the same stages
         for k in range(0, n0, 2):
             (e0, ev0, t0, ts0), (e1, ev1, t1, ts1) = ent[k], ent[k + 1]
-            assert (e0, ev0, t0, t1) == (e1, ev1, 0, 1) and ts1 >= ts0
+            assert (e0, ev0, t0, t1) == (e1, ev1, 0, 1) and after(ts1, ts0) >= 0
             if k:
-                assert ts0 >= ent[k - 1][3] and 0 < ((e0 - ent[k - 2][0]) & 0x1FFF) < 8  # stages follow one another (skipped ones leave gaps in the numbering)
+                assert after(ts0, ent[k - 1][3]) >= 0 and 0 < ((e0 - ent[k - 2][0]) & 0x1FFF) < 8  # stages follow one another (skipped ones leave gaps in the numbering)
     # one embedding and one sampling stage per iteration; the fused single-token forms are among the stages
     evs = [e[1] for e in per_wg[0][::2]]
     assert evs.count(101) == iters and evs.count(111) == iters
@@ -79,7 +107,8 @@ def test_profiler_tensor_records_every_iteration(tmp_path):
     # a stage's begin on one workgroup is never before the previous stage's end... on the slowest workgroup of that stage is
     # what the barrier gives; checked on whole microseconds of slack for clock skew between dies
     for k in range(2, min(n0, 200), 2):
-        assert min(per_wg[b][k][3] for b in per_wg) + 2000 >= max(per_wg[b][k - 2][3] for b in per_wg)
+        base = per_wg[0][k - 2][3]
+        assert min(after(per_wg[b][k][3], base) for b in per_wg) + 2000 >= max(after(per_wg[b][k - 2][3], base) for b in per_wg)
     assert (tmp_path / "run.perfetto-trace").exists() and (tmp_path / "run.pt").exists()
     # a tensor that is too small keeps the first entries and nothing is written past its end
     guard = torch.zeros(4 * G + 1 + 64, dtype=torch.uint64, device="cuda")
