@@ -4,6 +4,8 @@ linear weight once, in matrix-core tile order; the attached row-major tensors ca
 of one and two tokens run the matrix-core forms.  Checked: the same parity bars as the two-copy default (stage by stage at
 full width, end to end against the oracle), that the kernel really never reads the released tensors (they are overwritten
 with NaN and freed), and the byte accounting."""
+import gc
+
 import pytest
 import torch
 
@@ -120,6 +122,7 @@ def test_checkpoint_loaded_model_holds_its_linears_once(tmp_path):
     prompts = [make_prompt(cfg, n, 700 + i) for i, n in enumerate((5, 11, 8, 3, 17))]
     held = {}
     for single in (False, True):
+        gc.collect()  # (what earlier tests left in reference cycles must not be freed inside the measured window)
         torch.cuda.synchronize()
         base = torch.cuda.memory_allocated()
         md = _metadata(cfg, w, "cuda", R=R, T=T, total=total, max_seq=max_seq, PS=PS, from_path=str(ck))
