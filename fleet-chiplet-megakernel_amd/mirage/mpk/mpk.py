@@ -10,6 +10,7 @@ generation in "offline" mode, ONE pass over the batch the caller described in th
 What differs on the host: no MPI / multi-GPU set-up (one GPU), nothing is compiled at run time, checkpoints are local
 directories (no hub access).
 """
+import sys
 from dataclasses import dataclass
 from typing import Optional
 
@@ -98,6 +99,11 @@ class MPKMetadata:
     def print_info(self):
         print(self.info_as_string())
 
+    def write_to_file(self, file_path: str):
+        """The same summary as print_info, into a text file (mpk.py:102-104)."""
+        with open(file_path, "w") as f:
+            f.write(self.info_as_string())
+
 
 class MPK:
     def __init__(self, meta: MPKMetadata):
@@ -135,6 +141,11 @@ class MPK:
             self.num_workers, self.num_schedulers = get_configurations_from_gpu(dev.index if dev.index is not None else torch.cuda.current_device())
         else:
             self.num_workers, self.num_schedulers = meta.num_workers, max(meta.num_schedulers, 0)
+        # `profiling` without a tensor of the caller's: one of the reference's size (mpk.py:276-279); the kernel fills it
+        # from the first iteration on until it is full
+        self.profiler_tensor = meta.profiler_tensor
+        if meta.profiling and self.profiler_tensor is None:
+            self.profiler_tensor = torch.zeros(3000 * 128, dtype=torch.uint64, device=self.device)
         if meta.spec_decode_config is None and meta.spec_decode:
             meta.spec_decode_config = spec_decode_class(meta.spec_decode, ngram_size=meta.ngram_size, spec_length=meta.spec_length)
         self.spec_decode_config = meta.spec_decode_config
@@ -147,7 +158,7 @@ class MPK:
                 "num_new_tokens": self.num_new_tokens, "prompt_lengths": self.prompt_lengths, "qo_indptr_buffer": self.qo_indptr_buffer,
                 "paged_kv_indptr_buffer": self.paged_kv_indptr_buffer, "paged_kv_indices_buffer": self.paged_kv_indices_buffer,
                 "paged_kv_last_page_len_buffer": self.paged_kv_last_page_len_buffer},
-            profiler_tensor=meta.profiler_tensor, trace_name=meta.trace_name, spec_decode_config=meta.spec_decode_config,
+            profiler_tensor=self.profiler_tensor, trace_name=meta.trace_name, spec_decode_config=meta.spec_decode_config,
             use_cutlass_kernel=False, eos_token_id=meta.eos_token_id if meta.eos_token_id is not None else 151645,
             max_tokens_per_request=meta.max_tokens_per_request, single_weight_copy=meta.single_weight_copy)
         self.is_built = self.task_graph_generated = self.is_compiled = False
@@ -191,6 +202,24 @@ class MPK:
         for t in (self.step, self.tokens, self.input_tokens, self.output_tokens, self.num_new_tokens, self.prompt_lengths, self.qo_indptr_buffer,
                   self.paged_kv_indptr_buffer, self.paged_kv_indices_buffer, self.paged_kv_last_page_len_buffer):
             t.fill_(0)
+
+    def print_buffers(self, logger=None):
+        """The ten meta tensors, to `logger.info` or to stdout (mpk.py:329-341)."""
+        emit = logger.info if logger is not None else print
+        for name in ("step", "tokens", "input_tokens", "output_tokens", "num_new_tokens", "prompt_lengths", "qo_indptr_buffer",
+                     "paged_kv_indptr_buffer", "paged_kv_indices_buffer", "paged_kv_last_page_len_buffer"):
+            emit(f"{name}: {getattr(self, name)}")
+
+    def grid_dim_sanitizer(self, grid_dim):
+        """Halve the last dimension that is still above one until the task grid fits `max_sm_num` workers
+        (mpk.py:369-382).  The builders here size their grids from `num_workers` already; kept for callers that build
+        layers by hand."""
+        dims = list(grid_dim)
+        limit = max(int(self.metadata.max_sm_num or 0), 1)
+        while dims[0] * dims[1] * dims[2] > limit and any(d > 1 for d in dims):
+            i = max(j for j in range(3) if dims[j] > 1)
+            dims[i] //= 2
+        return tuple(dims)
 
     def init_per_request(self):
         self.persistent_kernel.init_request_resources()
@@ -260,3 +289,12 @@ class MPK:
 
     def finalize(self):
         self.persistent_kernel.finalize()
+
+    def __del__(self, _is_finalizing=sys.is_finalizing):
+        # the reference finalizes in its destructor (mpk.py:426-429); a kernel the caller finalized already is left alone
+        pk = getattr(self, "persistent_kernel", None)
+        if pk is not None and not _is_finalizing() and not getattr(pk, "__finalized__", True):
+            try:
+                pk.finalize()
+            except Exception:
+                pass

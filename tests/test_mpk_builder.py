@@ -84,6 +84,61 @@ def test_builder_task_sequence_lowers_on_the_host():
     mpk.finalize()
 
 
+def test_tensor_interleaving_helpers():
+    """models/utils.py:42-147 against an element-by-element construction, on the QKV case (uneven chunk sizes) and an inner dim."""
+    from mirage.mpk.models.utils import inplace_shuffle_tensors, shuffle_tensors
+    g = torch.Generator().manual_seed(3)
+    q, k, v = torch.randn(8 * 4, 6, generator=g), torch.randn(4 * 4, 6, generator=g), torch.randn(4 * 4, 6, generator=g)
+    out = shuffle_tensors([q, k, v], 4, 0)
+    rows = []
+    for h in range(4):
+        rows += [q[r] for r in range(8 * h, 8 * h + 8)] + [k[r] for r in range(4 * h, 4 * h + 4)] + [v[r] for r in range(4 * h, 4 * h + 4)]
+    assert out.shape == (64, 6) and torch.equal(out, torch.stack(rows))
+    a, b = torch.arange(12.).reshape(2, 6), 100 + torch.arange(6.).reshape(2, 3)
+    assert shuffle_tensors([a, b], 3, -1).tolist() == [[0, 1, 100, 2, 3, 101, 4, 5, 102], [6, 7, 103, 8, 9, 104, 10, 11, 105]]
+    tgt = torch.zeros(64, 6, dtype=torch.bfloat16)
+    assert inplace_shuffle_tensors([q, k, v], tgt, 4, 0) is None and torch.equal(tgt, out.to(torch.bfloat16))
+    for bad, exc in ((lambda: shuffle_tensors([], 2, 0), ValueError), (lambda: shuffle_tensors([q, k], 3, 0), ValueError),
+                     (lambda: shuffle_tensors([q, k.double()], 4, 0), TypeError), (lambda: shuffle_tensors([q, k[:, :5]], 4, 0), ValueError),
+                     (lambda: shuffle_tensors([q], 4, 2), ValueError), (lambda: shuffle_tensors([q], 0, 0), ValueError)):
+        with pytest.raises(exc):
+            bad()
+
+
+def test_wrapper_helpers_of_the_reference(tmp_path, capsys):
+    """The small conveniences of the reference's wrapper (mpk.py:102-104, 276-279, 329-341, 369-382, 426-429), host only."""
+    import logging
+    from mirage.mpk import MPK
+    from oracle.qwen3_ref import make_model_weights
+    cfg = _cfg()
+    md = _metadata(cfg, make_model_weights(cfg, seed=62), "cpu", num_workers=256)
+    md.write_to_file(str(tmp_path / "meta.txt"))
+    assert (tmp_path / "meta.txt").read_text() == md.info_as_string()
+    md.profiling = True
+    mpk = MPK(md)
+    assert mpk.profiler_tensor.dtype == torch.uint64 and mpk.profiler_tensor.numel() == 3000 * 128
+    assert mpk.persistent_kernel.profiler_tensor is mpk.profiler_tensor
+    # grids are halved from the last dimension until they fit max_sm_num (108 in the reference's metadata too)
+    assert mpk.grid_dim_sanitizer((96, 1, 1)) == (96, 1, 1)
+    assert mpk.grid_dim_sanitizer((64, 4, 1)) == (64, 1, 1)
+    assert mpk.grid_dim_sanitizer((256, 1, 1)) == (64, 1, 1) and mpk.grid_dim_sanitizer((3, 5, 16)) == (3, 5, 4)
+    assert mpk.grid_dim_sanitizer((1, 1, 1)) == (1, 1, 1)
+    mpk.print_buffers()
+    out = capsys.readouterr().out
+    assert out.count("\n") >= 10 and "paged_kv_last_page_len_buffer:" in out and out.startswith("step:")
+    seen = []
+    lg = logging.getLogger("mpk-test")
+    lg.info = lambda msg: seen.append(msg)
+    mpk.print_buffers(lg)
+    assert len(seen) == 10 and seen[1].startswith("tokens:")
+    pk = mpk.persistent_kernel
+    del mpk  # the destructor finalizes the kernel ...
+    assert pk.__finalized__
+    mpk2 = MPK(_metadata(cfg, make_model_weights(cfg, seed=62), "cpu", num_workers=256))
+    mpk2.finalize()
+    del mpk2  # ... and leaves one the caller finalized alone
+
+
 def _write_checkpoint(ck, cfg, w, tokenizer=False):
     from safetensors.torch import save_file
     ck.mkdir()
