@@ -798,6 +798,11 @@ class PersistentKernel:
         """persistent_kernel.py:2404.  Lowers the recorded tasks and uploads descriptors; nothing is compiled at run time."""
         assert not self._is_compiled
         output_dir = kwargs.get("output_dir", None)
+        # The library allocates its buffers (tile copies of the weights, intermediates, partial buffers) with hipMalloc,
+        # next to torch's caching allocator: blocks torch only caches are handed back first, or a process that has
+        # built and dropped large models before can run out of device memory with most of it unused.
+        if torch.cuda.is_available():
+            torch.cuda.empty_cache()
         self._g.compile()
         self._is_compiled = True
         if self._profiler_tensor is not None:

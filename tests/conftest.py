@@ -12,3 +12,16 @@ for p in (ROOT, PKG, os.path.dirname(os.path.abspath(__file__))):
 
 def pytest_configure(config):
     config.addinivalue_line("markers", "gpu: needs a real MI355X (run with -m gpu)")
+
+
+@pytest.fixture(autouse=True)
+def _release_device_memory_between_tests(request):
+    """GPU tests build models of up to 30 GB each; what a finished test leaves in reference cycles or in torch's block
+    cache must not add up over the session (the library under test allocates with hipMalloc, outside that cache)."""
+    yield
+    if request.node.get_closest_marker("gpu") is not None:
+        import gc
+        import torch
+        gc.collect()
+        if torch.cuda.is_available():
+            torch.cuda.empty_cache()
